@@ -1,0 +1,135 @@
+/*
+ * C ABI of libommx_hip.so: the OMMX paged decode-attention path for AMD gfx950.
+ *
+ * Three device entry points replace the reference's Python/Triton functions
+ * (paths relative to the reference checkout):
+ *
+ *   ommx_store_pack       <- ommx_gpu_serve/attention/pack.py:293-655
+ *                            ommx_pack_kv_canonical_block (quantize-on-store), and the
+ *                            slot placement of attention/kv_pool.py:711-734
+ *   ommx_decode_splitkv   <- ommx_gpu_serve/attention/paged_decode.py:1255-2284
+ *                            _canonical_splitkv_stage1 as launched at :3344-3436
+ *   ommx_decode_combine   <- ommx_gpu_serve/attention/paged_decode.py:2366-2500
+ *                            _canonical_lse_merge (bf16 tail folded in) at :3528-3549
+ *
+ * Conventions: every pointer is a device pointer unless its name starts with host_;
+ * strides are in ELEMENTS of the pointed-to type; nothing is allocated, freed or
+ * retained; nothing synchronises; `stream` is a hipStream_t passed as void*.
+ * Return value 0 = launched, negative = argument error (text in ommx_last_error()).
+ */
+#ifndef OMMX_HIP_H
+#define OMMX_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OMMX_ABI_VERSION 1
+
+/* number of floats in the store decision table: 256 pow2 thresholds + 8 FP4 slots */
+#define OMMX_STORE_TABLE_FLOATS 264
+
+/* error bits OR-ed into *err_flag by ommx_store_pack */
+#define OMMX_ERR_NONFINITE_K   1   /* pack.py:515-538 / codec.py:55-57 */
+#define OMMX_ERR_NONFINITE_V   2   /* pack.py:605-607 */
+#define OMMX_ERR_UNDERFILLED   4   /* fewer than k distinct outlier lanes, pack.py:520-538 */
+#define OMMX_ERR_EXP_RANGE     8   /* scale exponent does not fit the int8 plane */
+
+int ommx_abi_version(void);
+const char* ommx_last_error(void);
+
+/*
+ * Decision tables of the quantiser, exact-arithmetic defaults (host memory out).
+ *   host_table[kb], kb = biased fp32 exponent 0..255: smallest x in that binade with
+ *       rint(log2(x)) == kb-127+1, i.e. the first float above sqrt(2)*2^(kb-127)
+ *       (pack.py:462 `2^round(log2(scale))`);
+ *   host_table[256+j], j = 1..7: smallest |x| that encodes to FP4 level index j
+ *       (codec.py:45-65, geometric-mean boundaries, ties to the lower level).
+ * A caller that must agree bit-for-bit with a particular libm replaces entries with
+ * thresholds measured from that libm and uploads the table to the device.
+ */
+void ommx_store_default_table(float* host_table);
+
+/*
+ * Quantize-on-store: pack T = 32*n tokens of K and V into the ten planes.
+ *   K, V          rows [*, H, D]; element type bf16 (in_dtype 0) or fp32 (in_dtype 1);
+ *                 row r of head h starts at r*tok_stride + h*head_stride, D contiguous
+ *   src_rows      NULL, or int32[T]: source row of packed token t (ring gather)
+ *   dst_pages     NULL (identity), or int32[T/page_size]: physical page of logical page
+ *   dst_groups    NULL (identity), or int32[T/32]: group slot of logical group
+ *   table         float[OMMX_STORE_TABLE_FLOATS] on the device
+ *   planes        as written by pack.py:576-623:
+ *                 k_base,v_main u8[P,ps,H,D/4]; k_scale i8[G,H,D]; k_zp,k_ms,k_mc bf16[G,H,D];
+ *                 k_obmp u8[G,H,D,4]; k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32];
+ *                 v_zp bf16[P,ps,H,D/32]
+ *   err_flag      NULL or int32[1], OR-ed with OMMX_ERR_* (caller zeroes it)
+ * k_outliers in 0..8; D a multiple of 32, at most 256; T a multiple of 32 and page_size;
+ * 32 % page_size == 0.
+ */
+int ommx_store_pack(const void* K, const void* V, int in_dtype,
+                    int64_t k_tok_stride, int64_t k_head_stride,
+                    int64_t v_tok_stride, int64_t v_head_stride,
+                    const int32_t* src_rows,
+                    int T, int H, int D, int page_size, int k_outliers,
+                    const int32_t* dst_pages, const int32_t* dst_groups,
+                    const float* table,
+                    uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
+                    uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_obmp, uint8_t* k_oval,
+                    uint8_t* v_main, int8_t* v_scale, uint16_t* v_zp,
+                    int32_t* err_flag, void* stream);
+
+/*
+ * Split-KV decode over the packed planes (stage 1).
+ *   q             bf16 [B,Hq,D], strides q_stride_b, q_stride_h, D contiguous
+ *   planes        contiguous, layouts as above; k_outliers in 0..8 with the bitmap index
+ *                 plane, dedicated FP4 map and int8 exponents (the serving recipe)
+ *   req_to_token  int32 or int64 (table_i64) [B, >= ceil((L+off)/ps)], row stride rt_stride
+ *   req_to_group  same type [B, >= seg_group_base + ceil(L/32)], row stride rg_stride
+ *   b_seq_len     int32[B] packed tokens per request (device; bounds the loop)
+ *   attn_logits   f32 [B,Hq,>=num_splits,D+1] with strides al_stride_b/h/s: partial
+ *                 o (normalised) in [0,D) and lse at D; an empty split writes o=0,
+ *                 lse=-inf (paged_decode.py:2262-2284)
+ * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
+ * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in 1..8; D = 128 or 64.
+ */
+int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                        const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+                        const uint16_t* k_ms, const uint16_t* k_mc,
+                        const uint8_t* k_obmp, const uint8_t* k_oval,
+                        const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+                        const void* req_to_token, int64_t rt_stride,
+                        const void* req_to_group, int64_t rg_stride, int table_i64,
+                        const int32_t* b_seq_len,
+                        float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
+                        int64_t al_stride_s,
+                        int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
+                        int num_splits, float sm_scale, float logit_cap,
+                        int packed_start_offset, int seg_group_base, void* stream);
+
+/*
+ * Split combine with the bf16 sink/recent tail folded in (stage 2).
+ *   k_tail,v_tail bf16 [B,Tmax,Hkv,D] with strides t_stride_b/t/h (K and V alike)
+ *   b_tail_len    int32[B] valid tail rows (0 allowed)
+ *   o             f32 [B,Hq,D] strides o_stride_b/h;  lse f32 [B,Hq] stride lse_stride_b
+ * Valid splits are recomputed from b_seq_len with the stage-1 rounding
+ * (paged_decode.py:2407-2410); nothing attended gives o = 0, lse = -inf.
+ * emit_mode 0: merged final (splits + tail).  emit_mode 1: segment partial (no tail).
+ */
+int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
+                        int64_t al_stride_s,
+                        const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                        const uint16_t* k_tail, const uint16_t* v_tail,
+                        int64_t kt_stride_b, int64_t kt_stride_t, int64_t kt_stride_h,
+                        int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
+                        const int32_t* b_tail_len, const int32_t* b_seq_len,
+                        float* o, int64_t o_stride_b, int64_t o_stride_h,
+                        float* lse, int64_t lse_stride_b,
+                        int B, int Hq, int Hkv, int D, int num_splits,
+                        float sm_scale, float logit_cap, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMMX_HIP_H */

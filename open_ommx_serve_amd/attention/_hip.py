@@ -1,0 +1,93 @@
+"""ctypes binding of ``libommx_hip.so`` (the C ABI declared in ``include/ommx_hip.h``).
+
+The library is built in-tree by ``open_ommx_serve_amd.csrc.build``.  There is no fallback:
+if it is missing or an entry point fails, the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                         "csrc", "libommx_hip.so")
+_lib: Optional[C.CDLL] = None
+
+STORE_TABLE_FLOATS = 264
+ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE = 1, 2, 4, 8
+
+_P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
+
+_DECODE_ARGS = [
+    _P, _L, _L,                       # q, strides
+    _P, _P, _P, _P, _P, _P, _P,       # k planes
+    _P, _P, _P,                       # v planes
+    _P, _L, _P, _L, _I,               # tables
+    _P,                               # b_seq_len
+    _P, _L, _L, _L,                   # attn_logits, strides
+    _I, _I, _I, _I, _I, _I, _I,       # B Hq Hkv D ps kout S
+    _F, _F, _I, _I, _P,               # sm_scale cap off gbase stream
+]
+
+_SIGNATURES = {
+    "ommx_abi_version": (_I, []),
+    "ommx_last_error": (C.c_char_p, []),
+    "ommx_store_default_table": (None, [_P]),
+    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _P,
+                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ommx_decode_splitkv": (_I, _DECODE_ARGS),
+    "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),
+    "ommx_decode_combine": (_I, [_P, _L, _L, _L, _P, _L, _L, _P, _P, _L, _L, _L, _L, _L, _L,
+                                 _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _F, _F, _P]),
+}
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> C.CDLL:
+    """Load the shared library (once) and declare every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"{_LIB_PATH} is missing: build it with `python -m open_ommx_serve_amd.csrc.build` "
+            "(the OMMX operators have no fallback path)")
+    lib = C.CDLL(_LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.ommx_abi_version() != 1:
+        raise RuntimeError("libommx_hip.so ABI version mismatch; rebuild it")
+    _lib = lib
+    return lib
+
+
+def exported_symbols():
+    return tuple(_SIGNATURES)
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().ommx_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (rc={rc}): {msg}")
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(device: torch.device) -> None:
+    if device.type != "cuda":
+        raise RuntimeError(
+            f"OMMX HIP operators need tensors on a ROCm GPU; got device {device}. "
+            "There is no CPU fallback.")

@@ -1,0 +1,226 @@
+"""OMMX paged decode attention: host launcher of the HIP split-KV and combine kernels.
+
+``ommx_paged_decode_attention_canonical`` keeps the positional and keyword signature of the
+reference launcher (``ommx_gpu_serve/attention/paged_decode.py:2768-2798``), its argument
+checks and exception types (``:2916-3064``, ``:3323-3325``), the workspace shape
+``[B, Hq, splits+1, D+1]`` (``:247-253``) and the split rounding (``:1429-1432``).  It
+writes ``o`` and ``lse`` in place on the current stream, allocates nothing when
+``attn_logits`` is passed, and never synchronises when ``max_seq_len`` is passed.
+
+Implemented on the device: the serving recipe (INT2 base, bitmap-indexed FP4 outliers with
+the dedicated map, int8 exponent scales, 32-token / 32-channel vectors).  The reference's
+environment knobs are not read; ``num_stages`` / ``num_warps`` / ``qzp_buf`` are accepted
+and ignored (they tune Triton, not this kernel).
+"""
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+
+from . import _hip
+
+_CU_COUNT = {}
+
+
+def _cu_count(device: torch.device) -> int:
+    key = str(device)
+    if key not in _CU_COUNT:
+        _CU_COUNT[key] = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return _CU_COUNT[key]
+
+
+def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256) -> int:
+    """Split count that gives every compute unit about two workgroups of at least four
+    32-token groups each; never more than 128 (the reference's ceiling,
+    ``paged_decode.py:340-353``)."""
+    groups = max(1, (int(max_seq_len) + 31) // 32)
+    want = max(1, (2 * int(n_cu)) // max(1, int(batch) * int(kv_heads)))
+    return int(max(1, min(128, want, max(1, groups // 4))))
+
+
+def make_attn_logits(batch: int, q_heads: int, num_kv_splits: int, head_dim: int, device) -> torch.Tensor:
+    """fp32 workspace ``[B, Hq, splits + 1, D + 1]`` (reference ``paged_decode.py:247-253, 3220-3222``)."""
+    return torch.empty(batch, q_heads, num_kv_splits + 1, head_dim + 1,
+                       dtype=torch.float32, device=device)
+
+
+def ommx_paged_decode_attention_canonical(
+    q,
+    k_base, k_scale, k_zp, k_oidx, k_oval,
+    v_main, v_scale, v_zp,
+    k_tail, v_tail, b_tail_len,
+    o, lse,
+    req_to_token, req_to_group, b_seq_len,
+    *,
+    sm_scale: float = 1.0,
+    page_size: int = 16,
+    logit_cap: float = 0.0,
+    k_outliers_per_vector: int = 3,
+    k_format: str = "i2f4",
+    combinadic_read: bool = False,
+    k_crank: Any = None,
+    bitmap_read: bool = False,
+    k_obmp: Any = None,
+    k_fp4_mapscale: Any = None,
+    k_fp4_mapcenter: Any = None,
+    kv_outlier_map: bool = False,
+    kv_int8_scale: bool = False,
+    num_kv_splits: Optional[int] = None,
+    num_stages: Optional[int] = None,
+    num_warps: Optional[int] = None,
+    max_seq_len: Optional[int] = None,
+    max_tail_len: Optional[int] = None,
+    attn_logits: Any = None,
+    qzp_buf: Any = None,
+    packed_start_offset: int = 0,
+    seg_group_base: int = 0,
+    _force_reference_kernel: bool = False,
+) -> None:
+    """Canonical-KV paged decode attention.  Writes ``o [B,Hq,D]`` / ``lse [B,Hq]`` in place.
+
+    Plane layouts, tables and the tail are as documented for the reference launcher
+    (``paged_decode.py:2856-2887``).  ``seg_group_base > 0`` emits the un-merged state of a
+    group-range segment without the tail (``:2892-2902``).
+    """
+    pages, ngroups = int(k_base.shape[0]), int(k_scale.shape[0])
+    ps = int(page_size)
+    if pages == 0 or ngroups == 0:
+        group_tokens = 32
+    else:
+        group_tokens = (pages * ps) // ngroups
+        if group_tokens not in (16, 32, 64, 128):
+            raise ValueError(
+                f"derived GROUP_TOKENS={group_tokens} (pages={pages} page_size={ps} "
+                f"n_group_slots={ngroups}) must be in {{16,32,64,128}}")
+    vsc = int(v_scale.shape[-1])
+    group_channels = 32 if vsc == 0 else (int(v_main.shape[-1]) * 4) // vsc
+    if group_channels not in (16, 32, 64, 128):
+        raise ValueError(f"derived GROUP_CHANNELS={group_channels} must be in {{16,32,64,128}}")
+    kfmt = str(k_format).lower()
+    if kfmt not in ("i2f4", "itf4"):
+        raise ValueError(f"k_format must be i2f4|itf4; got {k_format!r}")
+    if bitmap_read and combinadic_read:
+        raise ValueError("combinadic_read and bitmap_read are mutually exclusive outlier-index sources")
+    B, Hq = int(q.shape[0]), int(q.shape[1])
+    D = int(k_base.shape[-1]) * 4
+    Dv = int(v_main.shape[-1]) * 4
+    Hkv = int(k_base.shape[-2])
+    if Dv % group_channels != 0:
+        raise ValueError(f"canonical KV requires head_dim % {group_channels} == 0; got Lv={Dv}.")
+    if Hkv < 1 or Hq < Hkv or Hq % Hkv != 0:
+        raise NotImplementedError(
+            "ommx_paged_decode_attention_canonical requires q_head_num to be an integer "
+            f"multiple of n_kv_heads; got q_head_num={Hq} n_kv_heads={Hkv}.")
+    for name, t in (("k_base", k_base), ("v_main", v_main), ("v_scale", v_scale), ("v_zp", v_zp)):
+        if t.stride(0) != ps * t.stride(1) or t.stride(-1) != 1:
+            raise ValueError(f"{name} must be a contiguous [pages, page_size, h, w] plane "
+                             "(kv_loc addressing needs stride(0) == page_size*stride(1)).")
+    off = int(packed_start_offset or 0)
+    if off < 0 or off >= ps:
+        raise ValueError(f"packed_start_offset={off} must be in [0, page_size={ps})")
+    gbase = int(seg_group_base or 0)
+    if gbase < 0:
+        raise ValueError(f"seg_group_base={gbase} must be >= 0")
+    k = int(k_outliers_per_vector)
+    if k > 0 and k_oval is None:
+        raise ValueError("k_outliers_per_vector > 0 requires the k_oval sidecar plane.")
+    if combinadic_read and k > 0 and k_crank is None:
+        raise ValueError("combinadic_read=True requires the k_crank combinadic-rank plane.")
+    if bitmap_read and k > 0 and k_obmp is None:
+        raise ValueError("bitmap_read=True requires the k_obmp flat-bitmask plane "
+                         "(pack with ommx_pack_kv_canonical_block(..., outlier_repr='bitmap')).")
+    if bitmap_read and k > 8:
+        raise ValueError("bitmap_read packs the k_oval value stream into ONE int32 word, "
+                         f"i.e. k <= 8; got k={k}. Use relidx7.")
+    if (not combinadic_read) and (not bitmap_read) and k > 0 and k_oidx is None:
+        raise ValueError("k_outliers_per_vector > 0 requires the k_oidx relidx7 sidecar plane "
+                         "(or bitmap_read=True with a k_obmp plane).")
+    use_map = bool(kv_outlier_map) and k > 0
+    if use_map and (k_fp4_mapscale is None or k_fp4_mapcenter is None):
+        raise ValueError("kv_outlier_map=True requires k_fp4_mapscale + k_fp4_mapcenter planes.")
+
+    unsupported = []
+    if group_tokens != 32 or group_channels != 32:
+        unsupported.append("group sizes other than 32")
+    if k > 0 and not bitmap_read:
+        unsupported.append("relidx7 / combinadic outlier index planes")
+    if k > 0 and not use_map:
+        unsupported.append("base-shared outliers (kv_outlier_map=False)")
+    if k_scale.dtype != torch.int8 or v_scale.dtype != torch.int8:
+        unsupported.append("bf16 scale planes (int8 exponents only)")
+    if D != Dv or D not in (64, 128) or (Hq // Hkv) not in (1, 2, 4, 8):
+        unsupported.append(f"head_dim {D}/{Dv} or GQA ratio {Hq // Hkv}")
+    if 32 % ps != 0:
+        unsupported.append("page_size not dividing 32")
+    if q.dtype != torch.bfloat16 or q.stride(-1) != 1:
+        unsupported.append("q that is not bf16 with unit inner stride")
+    if unsupported:
+        raise NotImplementedError(
+            "the HIP decode kernel implements the serving recipe only; not: " + ", ".join(unsupported))
+    for name, t in (("k_scale", k_scale), ("k_zp", k_zp), ("k_oval", k_oval), ("k_obmp", k_obmp),
+                    ("k_fp4_mapscale", k_fp4_mapscale), ("k_fp4_mapcenter", k_fp4_mapcenter)):
+        if t is not None and not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+    if req_to_token.dtype != req_to_group.dtype or req_to_token.dtype not in (torch.int32, torch.int64):
+        raise ValueError("req_to_token / req_to_group must both be int32 or both int64")
+    if req_to_token.stride(-1) != 1 or req_to_group.stride(-1) != 1:
+        raise ValueError("page / group tables must be contiguous along their last axis")
+    if b_seq_len.dtype != torch.int32 or b_tail_len.dtype != torch.int32:
+        raise ValueError("b_seq_len / b_tail_len must be int32")
+    if o.dtype != torch.float32 or lse.dtype != torch.float32 or o.stride(-1) != 1 or lse.stride(-1) != 1:
+        raise ValueError("o / lse must be fp32 with unit inner stride")
+
+    _hip.require_gpu(q.device)
+    if max_seq_len is not None:
+        max_seq = max(1, int(max_seq_len))
+    else:
+        max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
+    if num_kv_splits is None:
+        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device))
+    S = max(1, int(num_kv_splits))
+    if attn_logits is None:
+        attn_logits = make_attn_logits(B, Hq, S, D, q.device)
+    else:
+        if attn_logits.dtype != torch.float32 or attn_logits.dim() != 4 \
+                or tuple(attn_logits.shape[:2]) != (B, Hq) or int(attn_logits.shape[2]) < S \
+                or int(attn_logits.shape[3]) < D + 1 or attn_logits.stride(-1) != 1:
+            raise ValueError(f"attn_logits must be fp32 [B={B}, Hq={Hq}, >= {S}, >= {D + 1}] "
+                             f"with unit inner stride; got {tuple(attn_logits.shape)}")
+    has_tail = gbase == 0 and k_tail is not None and int(k_tail.shape[1]) > 0 \
+        and (max_tail_len is None or int(max_tail_len) > 0)
+    if has_tail:
+        if k_tail.dtype != torch.bfloat16 or v_tail.dtype != torch.bfloat16 \
+                or k_tail.stride(-1) != 1 or v_tail.stride(-1) != 1:
+            raise ValueError("k_tail / v_tail must be bf16 [B, T, Hkv, D] with unit inner stride")
+
+    lib = _hip.load()
+    stream = _hip.current_stream_ptr(q.device)
+    splitkv = lib.ommx_decode_splitkv_ref if _force_reference_kernel else lib.ommx_decode_splitkv
+    with torch.cuda.device(q.device):
+        rc = splitkv(
+            q.data_ptr(), q.stride(0), q.stride(1),
+            k_base.data_ptr(), k_scale.data_ptr(), k_zp.data_ptr(),
+            _hip.ptr(k_fp4_mapscale) if k > 0 else None, _hip.ptr(k_fp4_mapcenter) if k > 0 else None,
+            _hip.ptr(k_obmp) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
+            v_main.data_ptr(), v_scale.data_ptr(), v_zp.data_ptr(),
+            req_to_token.data_ptr(), req_to_token.stride(0),
+            req_to_group.data_ptr(), req_to_group.stride(0),
+            1 if req_to_token.dtype == torch.int64 else 0,
+            b_seq_len.data_ptr(),
+            attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
+            B, Hq, Hkv, D, ps, k, S, float(sm_scale), float(logit_cap), off, gbase, stream)
+        _hip.check(rc, "ommx_decode_splitkv")
+        rc = lib.ommx_decode_combine(
+            attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
+            q.data_ptr(), q.stride(0), q.stride(1),
+            k_tail.data_ptr() if has_tail else None, v_tail.data_ptr() if has_tail else None,
+            *( (k_tail.stride(0), k_tail.stride(1), k_tail.stride(2),
+                v_tail.stride(0), v_tail.stride(1), v_tail.stride(2)) if has_tail else (0,) * 6),
+            b_tail_len.data_ptr() if has_tail else None, b_seq_len.data_ptr(),
+            o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(0),
+            B, Hq, Hkv, D, S, float(sm_scale), float(logit_cap), stream)
+        _hip.check(rc, "ommx_decode_combine")
+
+
+__all__ = ["ommx_paged_decode_attention_canonical", "auto_num_kv_splits", "make_attn_logits"]

@@ -1,0 +1,137 @@
+// extern "C" entry points of libommx_hip.so for the decode side, argument checks and
+// kernel selection.  The store entry point lives beside its kernel in ommx_store.hip.
+#include <string>
+
+#include "ommx_decode_args.h"
+
+namespace ommx {
+
+static thread_local std::string g_error;
+
+void set_error(const char* msg) { g_error = msg; }
+
+int launch_decode_fast(const DecodeArgs& a, int D, int R, hipStream_t st);
+
+}  // namespace ommx
+
+extern "C" int ommx_abi_version(void) { return OMMX_ABI_VERSION; }
+
+extern "C" const char* ommx_last_error(void) { return ommx::g_error.c_str(); }
+
+extern "C" int ommx_decode_splitkv(
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+    const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_obmp, const uint8_t* k_oval,
+    const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
+    int table_i64, const int32_t* b_seq_len,
+    float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int num_splits,
+    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
+    void* stream) {
+    using namespace ommx;
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) {
+        set_error("ommx_decode_splitkv: q heads must be a positive multiple of kv heads");
+        return -1;
+    }
+    const int R = Hq / Hkv;
+    if (!(R == 1 || R == 2 || R == 4 || R == 8) || !(D == 64 || D == 128)) {
+        set_error("ommx_decode_splitkv: supported shapes are head_dim 64|128 and 1|2|4|8 q heads per kv head");
+        return -1;
+    }
+    if (page_size <= 0 || 32 % page_size) {
+        set_error("ommx_decode_splitkv: page_size must divide the 32-token group");
+        return -1;
+    }
+    if (packed_start_offset < 0 || packed_start_offset >= page_size || seg_group_base < 0) {
+        set_error("ommx_decode_splitkv: packed_start_offset must be in [0,page_size), seg_group_base >= 0");
+        return -1;
+    }
+    if (k_outliers < 0 || k_outliers > 8 || num_splits < 1) {
+        set_error("ommx_decode_splitkv: k_outliers in [0,8], num_splits >= 1");
+        return -1;
+    }
+    if (!q || !b_seq_len || !attn_logits || !req_to_token || !req_to_group) {
+        set_error("ommx_decode_splitkv: null pointer");
+        return -1;
+    }
+    if (k_outliers > 0 && (!k_ms || !k_mc || !k_obmp || !k_oval)) {
+        set_error("ommx_decode_splitkv: outlier planes missing");
+        return -1;
+    }
+    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_obmp, k_oval,
+                 v_main, v_scale, v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
+                 table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
+                 B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
+                 packed_start_offset, seg_group_base};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = launch_decode_fast(a, D, R, st);
+    if (rc == 1) rc = launch_decode_ref(a, D, R, st);
+    if (rc != 0) { set_error("ommx_decode_splitkv: no kernel for this shape"); return -1; }
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_splitkv: launch failed"); return -2; }
+    return 0;
+}
+
+// Same operator through the plain fp32 kernel only (cross-check entry used by tests).
+extern "C" int ommx_decode_splitkv_ref(
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+    const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_obmp, const uint8_t* k_oval,
+    const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
+    int table_i64, const int32_t* b_seq_len,
+    float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int num_splits,
+    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
+    void* stream) {
+    using namespace ommx;
+    if (B <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 || 32 % page_size || num_splits < 1 ||
+        k_outliers < 0 || k_outliers > 8) {
+        set_error("ommx_decode_splitkv_ref: bad arguments");
+        return -1;
+    }
+    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_obmp, k_oval,
+                 v_main, v_scale, v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
+                 table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
+                 B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
+                 packed_start_offset, seg_group_base};
+    if (launch_decode_ref(a, D, Hq / Hkv, static_cast<hipStream_t>(stream)) != 0) {
+        set_error("ommx_decode_splitkv_ref: unsupported shape");
+        return -1;
+    }
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_splitkv_ref: launch failed"); return -2; }
+    return 0;
+}
+
+extern "C" int ommx_decode_combine(
+    const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+    const uint16_t* k_tail, const uint16_t* v_tail,
+    int64_t kt_stride_b, int64_t kt_stride_t, int64_t kt_stride_h,
+    int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
+    const int32_t* b_tail_len, const int32_t* b_seq_len,
+    float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
+    int B, int Hq, int Hkv, int D, int num_splits, float sm_scale, float logit_cap,
+    void* stream) {
+    using namespace ommx;
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || num_splits < 1 || !(D == 64 || D == 128)) {
+        set_error("ommx_decode_combine: bad shape");
+        return -1;
+    }
+    if (!attn_logits || !o || !lse || !b_seq_len) { set_error("ommx_decode_combine: null pointer"); return -1; }
+    if (b_tail_len && (!k_tail || !v_tail || !q)) {
+        set_error("ommx_decode_combine: tail lengths given without tail rows");
+        return -1;
+    }
+    CombineArgs a{attn_logits, al_stride_b, al_stride_h, al_stride_s, q, q_stride_b, q_stride_h,
+                  k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h,
+                  vt_stride_b, vt_stride_t, vt_stride_h, b_tail_len, b_seq_len,
+                  o, o_stride_b, o_stride_h, lse, lse_stride_b, B, Hq, Hkv, num_splits,
+                  sm_scale, logit_cap};
+    if (launch_combine(a, D, static_cast<hipStream_t>(stream)) != 0) {
+        set_error("ommx_decode_combine: unsupported head_dim");
+        return -1;
+    }
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_combine: launch failed"); return -2; }
+    return 0;
+}

@@ -1,0 +1,46 @@
+// Argument block and small helpers shared by the decode kernels.
+#pragma once
+#include "ommx_common.h"
+
+namespace ommx {
+
+struct DecodeArgs {
+    const uint16_t* q; int64_t q_sb, q_sh;
+    const uint8_t* k_base; const int8_t* k_scale; const uint16_t* k_zp;
+    const uint16_t* k_ms; const uint16_t* k_mc; const uint8_t* k_obmp; const uint8_t* k_oval;
+    const uint8_t* v_main; const int8_t* v_scale; const uint16_t* v_zp;
+    const void* rt; int64_t rt_s; const void* rg; int64_t rg_s; int i64;
+    const int32_t* seq;
+    float* al; int64_t al_b, al_h, al_s;
+    int B, Hq, Hkv, ps, kout, S;
+    float sm_scale, cap;
+    int off, gbase;
+};
+
+__device__ __forceinline__ int64_t table_at(const void* t, int64_t i, int i64) {
+    return i64 ? static_cast<const int64_t*>(t)[i] : static_cast<const int32_t*>(t)[i];
+}
+
+__device__ __forceinline__ float apply_cap(float x, float cap) {
+    // cap * tanh(x / cap) written as the reference does: cap * (2*sigmoid(2x/cap) - 1)
+    if (cap > 0.0f) x = cap * (2.0f / (1.0f + __expf(-2.0f * x / cap)) - 1.0f);
+    return x;
+}
+
+
+struct CombineArgs {
+    const float* al; int64_t al_b, al_h, al_s;
+    const uint16_t* q; int64_t q_sb, q_sh;
+    const uint16_t* kt; const uint16_t* vt;
+    int64_t kt_b, kt_t, kt_h, vt_b, vt_t, vt_h;
+    const int32_t* tail; const int32_t* seq;
+    float* o; int64_t o_b, o_h;
+    float* lse; int64_t lse_b;
+    int B, Hq, Hkv, S;
+    float sm_scale, cap;
+};
+
+int launch_decode_ref(const DecodeArgs& a, int D, int R, hipStream_t st);
+int launch_combine(const CombineArgs& a, int D, hipStream_t st);
+
+}  // namespace ommx

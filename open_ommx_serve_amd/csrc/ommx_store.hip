@@ -1,0 +1,296 @@
+// Quantize-on-store kernel: bf16/fp32 K,V rows -> the ten OMMX planes, bit-exact with
+// the reference packer (ommx_gpu_serve/attention/pack.py:419-623; codec.py:45-65,
+// 330-372).  Compiled with -ffp-contract=off: every fp32 operation below is a single
+// IEEE rounding in the order the reference performs it.
+//
+// One workgroup packs one (32-token group, kv head).  It has D threads and does two jobs:
+//   K: thread d owns the vector "channel d over the 32 tokens": outlier selection,
+//      min/max of the rest, power-of-two scale, INT2 codes, FP4 map and nibbles.
+//   V: thread x owns the vector "token x/(D/32), channels 32*(x%(D/32))..+31".
+// The K codes of 4 neighbouring channels share a byte of k_base, so they are transposed
+// through LDS and written as 8-byte pieces of the token-major rows.
+#include "ommx_common.h"
+
+namespace ommx {
+
+struct StoreArgs {
+    const void* K;
+    const void* V;
+    int64_t k_ts, k_hs, v_ts, v_hs;
+    const int32_t* src_rows;
+    const int32_t* dst_pages;
+    const int32_t* dst_groups;
+    const float* table;
+    uint8_t* k_base;
+    int8_t* k_scale;
+    uint16_t* k_zp;
+    uint16_t* k_ms;
+    uint16_t* k_mc;
+    uint8_t* k_obmp;
+    uint8_t* k_oval;
+    uint8_t* v_main;
+    int8_t* v_scale;
+    uint16_t* v_zp;
+    int32_t* err;
+    int H, D, ps, kout;
+};
+
+template <bool F32>
+__device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
+    if (F32) return static_cast<const float*>(base)[idx];
+    return bf16_to_f32(static_cast<const uint16_t*>(base)[idx]);
+}
+
+// rint(log2(x)) for x >= 1e-12 through the threshold table: the exponent of x's binade,
+// plus one when x has reached that binade's rounding point.
+__device__ __forceinline__ int pow2_round_exp(float x, const float* __restrict__ table) {
+    const uint32_t kb = (__float_as_uint(x) >> 23) & 0xFFu;
+    return static_cast<int>(kb) - 127 + (x >= table[kb] ? 1 : 0);
+}
+
+__device__ __forceinline__ float exp2_int(int e) {   // exact 2^e, e in [-126,127]
+    return __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+}
+
+__device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict__ fthr) {
+    const float a = fabsf(m);
+    uint32_t idx = 0;
+#pragma unroll
+    for (int j = 1; j <= 7; ++j) idx += (a >= fthr[j]) ? 1u : 0u;
+    return ((m < 0.0f) ? 8u : 0u) | idx;
+}
+
+template <bool F32>
+__global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
+    extern __shared__ uint8_t smem[];
+    const int D = a.D;
+    uint8_t* s_codes = smem;                       // [32][D] one code per byte
+    uint8_t* s_oval = smem + 32 * D;               // [D][4] nibble bytes (3 used at k=6)
+    const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int NGV = D >> 5;
+    const int kout = a.kout, kt = (kout + 1) >> 1, kb = kout - kt;
+    const int nval = (kout + 1) >> 1;              // nibble bytes per frame
+    const int64_t gs = a.dst_groups ? a.dst_groups[g] : g;
+    const float* __restrict__ tab = a.table;
+    int err = 0;
+
+    // ------------------------------------------------------------------ K vector
+    {
+        const int d = tid;
+        float w[32];
+        bool fin = true;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int64_t row = a.src_rows ? a.src_rows[g * 32 + i] : (int64_t)g * 32 + i;
+            w[i] = load_elem<F32>(a.K, row * a.k_ts + (int64_t)h * a.k_hs + d);
+            fin = fin && is_finite_f32(w[i]);
+        }
+        if (!fin) err |= OMMX_ERR_NONFINITE_K;
+
+        // signed select (pack.py:436-445): kt largest, ties to the lower index ...
+        uint32_t top = 0;
+        for (int r = 0; r < kt; ++r) {
+            float best = 0.0f; int bi = -1;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const bool free_lane = !((top >> i) & 1u);
+                if (free_lane && (bi < 0 || w[i] > best)) { best = w[i]; bi = i; }
+            }
+            if (bi >= 0) top |= 1u << bi;
+        }
+        // ... then kb smallest of the vector with chosen lanes replaced by +1e9.
+        uint32_t bot = 0;
+        for (int r = 0; r < kb; ++r) {
+            float best = 0.0f; int bi = -1;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const float v = ((top >> i) & 1u) ? 1e9f : w[i];
+                const bool free_lane = !((bot >> i) & 1u);
+                if (free_lane && (bi < 0 || v < best)) { best = v; bi = i; }
+            }
+            if (bi >= 0) bot |= 1u << bi;
+        }
+        const uint32_t om = top | bot;
+        if (__popc(om) != kout) err |= OMMX_ERR_UNDERFILLED;
+
+        // affine base over the non-outlier lanes (pack.py:455-465)
+        float mn = 1e9f, mx = -1e9f, omn = 1e9f, omx = -1e9f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const bool o = (om >> i) & 1u;
+            mn = fminf(mn, o ? 1e9f : w[i]);
+            mx = fmaxf(mx, o ? -1e9f : w[i]);
+            omn = fminf(omn, o ? w[i] : 1e9f);
+            omx = fmaxf(omx, o ? w[i] : -1e9f);
+        }
+        if (mn > 1e8f) mn = 0.0f;
+        if (mx < -1e8f) mx = 0.0f;
+        if (omn > 1e8f) omn = 0.0f;
+        if (omx < -1e8f) omx = 0.0f;
+        const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
+        const int e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
+        if (e < -126 || e > 127) err |= OMMX_ERR_EXP_RANGE;
+        const float scale = exp2_int(e);
+        const uint16_t zp_b = f32_to_bf16_rne(mn);
+        const float zp = bf16_to_f32(zp_b);
+
+        // dedicated FP4 map over the outlier lanes (pack.py:486-498)
+        uint16_t mc_b = 0, ms_b = 0;
+        float mc = 0.0f, ms = 0.0f;
+        if (kout > 0) {
+            mc_b = f32_to_bf16_rne(__fdiv_rn(omx + omn, 2.0f));
+            ms_b = f32_to_bf16_rne(__fdiv_rn(12.0f, fmaxf(omx - omn, 1e-8f)));
+            mc = bf16_to_f32(mc_b);
+            ms = bf16_to_f32(ms_b);
+        }
+
+        uint32_t nib = 0;
+        int slot = 0;
+        bool mfin = true;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            float c = rintf(__fdiv_rn(w[i] - zp, scale));
+            c = fminf(fmaxf(c, 0.0f), 3.0f);
+            s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
+            if (kout > 0) {
+                const float mapped = (w[i] - mc) * ms;
+                mfin = mfin && is_finite_f32(mapped);
+                if ((om >> i) & 1u) {
+                    nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
+                    ++slot;
+                }
+            }
+        }
+        if (!mfin) err |= OMMX_ERR_NONFINITE_K;
+
+        const int64_t gidx = (gs * a.H + h) * D + d;
+        a.k_scale[gidx] = static_cast<int8_t>(e);
+        a.k_zp[gidx] = zp_b;
+        if (kout > 0) {
+            a.k_ms[gidx] = ms_b;
+            a.k_mc[gidx] = mc_b;
+            reinterpret_cast<uint32_t*>(a.k_obmp)[gidx] = om;      // byte p>>3, bit p&7
+            reinterpret_cast<uint32_t*>(s_oval)[d] = nib;
+        }
+    }
+    __syncthreads();
+
+    // nibble plane: D frames of nval bytes, contiguous in memory
+    if (kout > 0) {
+        const int64_t obase = (gs * a.H + h) * (int64_t)D * nval;
+        for (int b = tid; b < D * nval; b += D)
+            a.k_oval[obase + b] = s_oval[(b / nval) * 4 + (b % nval)];
+    }
+
+    // ------------------------------------------------- k_base rows and the V vector
+    {
+        const int t = tid / NGV, j = tid % NGV;           // token in group, 32-channel slice
+        const int tok = g * 32 + t;
+        const int lp = tok / a.ps;
+        const int64_t page = a.dst_pages ? a.dst_pages[lp] : lp;
+        const int64_t prow = page * a.ps + (tok % a.ps);  // physical token row
+
+        uint64_t kb8 = 0;
+        const uint8_t* cr = s_codes + t * D + 32 * j;
+#pragma unroll
+        for (int c = 0; c < 32; ++c) kb8 |= static_cast<uint64_t>(cr[c] & 3u) << (2 * c);
+        reinterpret_cast<uint64_t*>(a.k_base)[(prow * a.H + h) * NGV + j] = kb8;
+
+        const int64_t row = a.src_rows ? a.src_rows[tok] : tok;
+        const int64_t vbase = row * a.v_ts + (int64_t)h * a.v_hs + 32 * j;
+        float v[32];
+        bool fin = true;
+        float mn = 0.0f, mx = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 32; ++c) {
+            v[c] = load_elem<F32>(a.V, vbase + c);
+            fin = fin && is_finite_f32(v[c]);
+            mn = c == 0 ? v[c] : fminf(mn, v[c]);
+            mx = c == 0 ? v[c] : fmaxf(mx, v[c]);
+        }
+        if (!fin) err |= OMMX_ERR_NONFINITE_V;
+        const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
+        const int e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
+        if (e < -126 || e > 127) err |= OMMX_ERR_EXP_RANGE;
+        const float scale = exp2_int(e);
+        const uint16_t zp_b = f32_to_bf16_rne(mn);
+        const float zp = bf16_to_f32(zp_b);
+        uint64_t vb8 = 0;
+#pragma unroll
+        for (int c = 0; c < 32; ++c) {
+            float q = rintf(__fdiv_rn(v[c] - zp, scale));
+            q = fminf(fmaxf(q, 0.0f), 3.0f);
+            vb8 |= static_cast<uint64_t>(static_cast<int>(q)) << (2 * c);
+        }
+        const int64_t vidx = (prow * a.H + h) * NGV + j;
+        reinterpret_cast<uint64_t*>(a.v_main)[vidx] = vb8;
+        a.v_scale[vidx] = static_cast<int8_t>(e);
+        a.v_zp[vidx] = zp_b;
+    }
+    if (err && a.err) atomicOr(a.err, err);
+}
+
+}  // namespace ommx
+
+extern "C" void ommx_store_default_table(float* t) {
+    // first float strictly above sqrt(2)*2^k: exact rint(log2(x)) switches there
+    for (int kb = 0; kb < 256; ++kb) {
+        const double b = 1.4142135623730951 * __builtin_ldexp(1.0, kb - 127);
+        float c = static_cast<float>(b);
+        if (static_cast<double>(c) < b) c = __builtin_nextafterf(c, __builtin_inff());
+        t[kb] = (kb == 0 || kb == 255) ? __builtin_inff() : c;
+    }
+    // FP4 level boundaries: geometric means of neighbouring magnitudes (the zero level
+    // counts as 1e-8), a tie staying with the lower level
+    const double lv[8] = {1e-8, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
+    t[256] = 0.0f;
+    for (int j = 1; j < 8; ++j) {
+        const double b = __builtin_sqrt(lv[j - 1] * lv[j]);
+        float c = static_cast<float>(b);
+        if (static_cast<double>(c) <= b) c = __builtin_nextafterf(c, __builtin_inff());
+        t[256 + j] = c;
+    }
+}
+
+extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
+                               int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
+                               const int32_t* src_rows, int T, int H, int D, int page_size,
+                               int k_outliers, const int32_t* dst_pages,
+                               const int32_t* dst_groups, const float* table,
+                               uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
+                               uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_obmp,
+                               uint8_t* k_oval, uint8_t* v_main, int8_t* v_scale,
+                               uint16_t* v_zp, int32_t* err_flag, void* stream) {
+    using namespace ommx;
+    if (T < 0 || T % 32 || page_size <= 0 || 32 % page_size || T % page_size) {
+        set_error("ommx_store_pack: T must be a multiple of 32 and page_size must divide 32");
+        return -1;
+    }
+    if (D < 32 || D > 256 || D % 32 || H <= 0) {
+        set_error("ommx_store_pack: head_dim must be a multiple of 32 in [32,256]");
+        return -1;
+    }
+    if (k_outliers < 0 || k_outliers > 8) {
+        set_error("ommx_store_pack: outliers_per_vector must be in [0,8] for the bitmap plane");
+        return -1;
+    }
+    if (in_dtype != 0 && in_dtype != 1) { set_error("ommx_store_pack: in_dtype"); return -1; }
+    if (!K || !V || !table || !k_base || !k_scale || !k_zp || !v_main || !v_scale || !v_zp ||
+        (k_outliers > 0 && (!k_ms || !k_mc || !k_obmp || !k_oval))) {
+        set_error("ommx_store_pack: null plane or input pointer");
+        return -1;
+    }
+    if (T == 0) return 0;
+    StoreArgs a{K, V, k_ts, k_hs, v_ts, v_hs, src_rows, dst_pages, dst_groups, table,
+                k_base, k_scale, k_zp, k_ms, k_mc, k_obmp, k_oval, v_main, v_scale, v_zp,
+                err_flag, H, D, page_size, k_outliers};
+    const dim3 grid(T / 32, H), block(D);
+    const size_t shm = 32 * (size_t)D + 4 * (size_t)D;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (in_dtype == 1)
+        hipLaunchKernelGGL(store_pack_kernel<true>, grid, block, shm, st, a);
+    else
+        hipLaunchKernelGGL(store_pack_kernel<false>, grid, block, shm, st, a);
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_store_pack: launch failed"); return -2; }
+    return 0;
+}

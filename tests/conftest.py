@@ -1,0 +1,65 @@
+"""Shared fixtures.  Tests marked ``gpu`` need one ROCm GPU; the rest run on the CPU."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+PLANE_NAMES = ("k_base", "k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale",
+               "k_fp4_mapcenter", "v_main", "v_scale", "v_zp")
+GOLDEN_CASES = ("tiny_ties", "small_gauss", "layer_outliers", "wide_range", "fp32_inputs")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a ROCm GPU (run with -m gpu on the GPU box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no GPU in this process")
+    for it in items:
+        if "gpu" in it.keywords:
+            it.add_marker(skip)
+
+
+def tensor_from_bits(a: np.ndarray) -> torch.Tensor:
+    """Inverse of the fixture writer: uint16 -> bf16, uint32 -> fp32, else as stored."""
+    t = torch.from_numpy(a.copy())
+    if a.dtype == np.uint16:
+        return t.view(torch.int16).view(torch.bfloat16)
+    if a.dtype == np.uint32:
+        return t.view(torch.int32).view(torch.float32)
+    return t
+
+
+def bits_of(t: torch.Tensor) -> np.ndarray:
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).numpy().view(np.uint16)
+    if t.dtype == torch.float32:
+        return t.view(torch.int32).numpy().view(np.uint32)
+    return t.numpy()
+
+
+def load_golden(name: str):
+    z = np.load(os.path.join(GOLDEN_DIR, f"pack_{name}.npz"))
+    return {k: z[k] for k in z.files}
+
+
+def assert_planes_equal(got, want_bits, what=""):
+    """Bit-exact comparison of a plane dict against raw golden arrays (or another dict)."""
+    for name in PLANE_NAMES:
+        w = want_bits[name]
+        if torch.is_tensor(w):
+            w = bits_of(w)
+        g = bits_of(got[name])
+        assert g.shape == w.shape, f"{what} {name}: shape {g.shape} != {w.shape}"
+        bad = int((g != w).sum())
+        assert bad == 0, f"{what} {name}: {bad} of {g.size} elements differ"

@@ -1,0 +1,242 @@
+"""HIP split-KV decode + combine against the dequantise-then-attend oracle.
+
+Tolerance (fp32 accumulation on the device, fp64 in the oracle): max-abs 2e-3 and
+mean-abs 2e-4 on ``o``; ``lse`` within 2e-3.  All calls go through the C ABI."""
+import math
+
+import pytest
+import torch
+
+import oracle.ommx_oracle as O
+from open_ommx_serve_amd.attention.kv_window import WindowSpec
+from open_ommx_serve_amd.attention.paged_decode import (make_attn_logits,
+                                                        ommx_paged_decode_attention_canonical)
+from open_ommx_serve_amd.synth import build_decode_case
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-3, 2e-4
+
+
+def _cpu_planes(case):
+    return {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in case.planes.items()} | {
+        "outliers_per_vector": case.outliers_per_vector}
+
+
+def _oracle(case, **kw):
+    return O.decode_reference(
+        case.q.cpu(), _cpu_planes(case), case.k_tail.cpu(), case.v_tail.cpu(),
+        case.b_tail_len.tolist(), case.req_to_token.cpu(), case.req_to_group.cpu(),
+        case.b_seq_len.tolist(), sm_scale=case.sm_scale, page_size=case.page_size, **kw)
+
+
+def _run(case, num_kv_splits=None, ref_kernel=False, **over):
+    B, Hq, D = case.q.shape
+    o = torch.full((B, Hq, D), float("nan"), dtype=torch.float32, device=case.q.device)
+    lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=case.q.device)
+    kw = case.decode_kwargs()
+    kw.update(over)
+    ommx_paged_decode_attention_canonical(*case.decode_args(o, lse), num_kv_splits=num_kv_splits,
+                                          _force_reference_kernel=ref_kernel, **kw)
+    torch.cuda.synchronize()
+    return o.cpu(), lse.cpu()
+
+
+def _check(got, want, what=""):
+    (o, lse), (wo, wl) = got, want
+    assert torch.isfinite(o).all(), f"{what}: non-finite output"
+    err = (o.double() - wo).abs()
+    assert err.max().item() <= MAX_ABS, f"{what}: max-abs {err.max().item():.3e}"
+    assert err.mean().item() <= MEAN_ABS, f"{what}: mean-abs {err.mean().item():.3e}"
+    fin = torch.isfinite(wl)
+    assert torch.equal(torch.isfinite(lse), fin), f"{what}: lse finiteness"
+    assert (lse.double()[fin] - wl[fin]).abs().max().item() <= 2e-3 if fin.any() else True, f"{what}: lse"
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+@pytest.mark.parametrize("seq_len", [128, 136, 200, 232])
+def test_small_gqa2_d64_like_the_reference_parity_test(seq_len, ref_kernel):
+    """H_KV=2, H_Q=4, D=64, page 16, sink 8, recent 32, k=6: 2/3/5/6 packed groups."""
+    case = build_decode_case([seq_len], q_heads=4, kv_heads=2, head_dim=64, seed=11)
+    _check(_run(case, ref_kernel=ref_kernel), _oracle(case), f"seq{seq_len}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+@pytest.mark.parametrize("splits", [1, 2, 4])
+def test_forced_splits_4k_d64(splits, ref_kernel):
+    case = build_decode_case([4096 + 40], q_heads=4, kv_heads=2, head_dim=64, seed=23,
+                             table_dtype=torch.int64)
+    _check(_run(case, num_kv_splits=splits, ref_kernel=ref_kernel), _oracle(case), f"S{splits}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_layer_ctx1024(ref_kernel):
+    """32 q / 8 kv heads, d=128, ctx 1024: 960 packed tokens + 64 tail rows."""
+    case = build_decode_case([1024], seed=42)
+    assert case.b_seq_len.tolist() == [960] and case.b_tail_len.tolist() == [64]
+    assert case.algorithmic_bytes() == 960 * 8 * 132 + 64 * 8 * 128 * 4
+    want = _oracle(case)
+    for S in (None, 1, 3, 8):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"S{S}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_layer_ctx4096_identity_tables(ref_kernel):
+    case = build_decode_case([4096], seed=42)
+    assert case.b_seq_len.tolist() == [4032]
+    want = _oracle(case)
+    for S in (None, 4, 16):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"S{S}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_permuted_tables_ctx8192(ref_kernel):
+    case = build_decode_case([8192], seed=7, permute_tables=True, sparse_frac=0.005)
+    want = _oracle(case)
+    for S in (1, 8, 32):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"S{S}")
+
+
+def test_long_context_64k_permuted_all_split_counts():
+    """ctx 65536, permuted page and group tables, sparse x8 outliers; 1, 8, 32, 64 splits."""
+    case = build_decode_case([65536], seed=42, permute_tables=True, sparse_frac=0.005)
+    assert case.b_seq_len.tolist() == [65472]
+    assert case.algorithmic_bytes() == 65472 * 8 * 132 + 64 * 8 * 128 * 4
+    want = _oracle(case)
+    for S in (1, 8, 32, 64, None):
+        _check(_run(case, num_kv_splits=S), want, f"S{S}")
+    _check(_run(case, num_kv_splits=64, ref_kernel=True), want, "ref S64")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_ragged_batch_shared_pool(ref_kernel):
+    """Twelve requests of different lengths sharing one shuffled pool, incl. one with no
+    packed tokens at all and one with an empty tail slot beyond its length."""
+    lens = [1024, 40, 4000, 71, 72, 2047, 16384, 9, 1500, 333, 8192, 5000]
+    case = build_decode_case(lens, seed=5, permute_tables=True, sparse_frac=0.005)
+    want = _oracle(case)
+    for S in (None, 1, 7, 16):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"S{S}")
+
+
+def test_ragged_batch_32_requests():
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(1024, 16385, (32,), generator=g).tolist()
+    case = build_decode_case(lens, seed=6, permute_tables=True, sparse_frac=0.005)
+    _check(_run(case), _oracle(case), "B32")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_gqa8_64_q_heads(ref_kernel):
+    case = build_decode_case([2048, 3000], q_heads=64, kv_heads=8, seed=8, sparse_frac=0.005)
+    want = _oracle(case)
+    for S in (None, 5):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"S{S}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_other_head_ratios(ref_kernel):
+    for hq, hkv in ((8, 8), (8, 4), (2, 1)):
+        case = build_decode_case([520], q_heads=hq, kv_heads=hkv, seed=9)
+        _check(_run(case, ref_kernel=ref_kernel), _oracle(case), f"{hq}/{hkv}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
+def test_no_outliers_recipe(ref_kernel):
+    case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)
+    _check(_run(case, ref_kernel=ref_kernel), _oracle(case), "k0")
+
+
+def test_tail_only_and_nothing_attended():
+    case = build_decode_case([33, 1], q_heads=8, kv_heads=2, seed=12)
+    assert case.b_seq_len.tolist() == [0, 0]
+    _check(_run(case, num_kv_splits=4), _oracle(case), "tail-only")
+    # zero tail rows as well: o = 0, lse = -inf
+    case.b_tail_len.zero_()
+    o, lse = _run(case, num_kv_splits=2)
+    assert float(o.abs().sum()) == 0.0 and bool(torch.isinf(lse).all()) and bool((lse < 0).all())
+
+
+def test_partial_last_group_is_masked():
+    """b_seq_len need not be a whole number of groups: tokens past it are ignored."""
+    case = build_decode_case([2048], q_heads=8, kv_heads=2, seed=13)
+    for L in (1, 31, 33, 1000, 1999):
+        case.b_seq_len.fill_(L)
+        case.extra["packed_lens"] = [L]
+        want = _oracle(case)
+        for S in (1, 3):
+            _check(_run(case, num_kv_splits=S), want, f"L{L} S{S}")
+
+
+def test_logit_cap_and_caller_workspace():
+    case = build_decode_case([3000], q_heads=8, kv_heads=2, seed=14)
+    S = 6
+    ws = make_attn_logits(1, 8, S, 128, "cuda")
+    ws.fill_(float("nan"))
+    got = _run(case, num_kv_splits=S, attn_logits=ws)
+    _check(got, _oracle(case), "workspace")
+    # partial states: splits x (D+1), lse column finite, tail slot untouched by stage 1
+    assert torch.isfinite(ws[:, :, :S, :]).all()
+    # capped logits: compare with an oracle that caps
+    cap = 5.0
+    Kd, Vd = O.gather_request(_cpu_planes(case), case.req_to_token[0].cpu(), case.req_to_group[0].cpu(),
+                              case.b_seq_len.tolist()[0], page_size=16)
+    tl = case.b_tail_len.tolist()[0]
+    Kf = torch.cat([Kd, case.k_tail[0, :tl].cpu().float()]).double()
+    Vf = torch.cat([Vd, case.v_tail[0, :tl].cpu().float()]).double()
+    want = torch.zeros(8, 128, dtype=torch.float64)
+    for h in range(8):
+        s = (Kf[:, h // 4] @ case.q[0, h].cpu().double()) * case.sm_scale
+        s = cap * torch.tanh(s / cap)
+        want[h] = torch.softmax(s, 0) @ Vf[:, h // 4]
+    o, _ = _run(case, num_kv_splits=S, logit_cap=cap)
+    assert (o[0].double() - want).abs().max().item() <= MAX_ABS
+
+
+def test_segment_partial_emit_composes_to_the_full_result():
+    """Two group-range segments plus the tail, merged with the textbook state merge."""
+    case = build_decode_case([4096], q_heads=8, kv_heads=2, seed=15)
+    want = _oracle(case)
+    L = case.b_seq_len.tolist()[0]
+    g_split = (L // 32) // 3
+    parts = []
+    for gb, n in ((0, g_split * 32), (g_split, L - g_split * 32)):
+        case.b_seq_len.fill_(n)
+        o, lse = _run(case, num_kv_splits=4, seg_group_base=gb,
+                      max_tail_len=0 if gb > 0 else None)
+        parts.append((o, lse))
+    case.b_seq_len.fill_(L)
+    # first call (gb=0) included the tail; second is a pure segment
+    o, lse = O.merge_states(torch.stack([p[0][0].double() for p in parts]),
+                            torch.stack([p[1][0].double() for p in parts]))
+    assert (o - want[0][0]).abs().max().item() <= MAX_ABS
+    assert (lse - want[1][0]).abs().max().item() <= 2e-3
+
+
+def test_host_argument_checks_raise_before_launch():
+    case = build_decode_case([200], q_heads=4, kv_heads=2, head_dim=64, seed=16)
+    B, Hq, D = case.q.shape
+    o = torch.empty(B, Hq, D, dtype=torch.float32, device="cuda")
+    lse = torch.empty(B, Hq, dtype=torch.float32, device="cuda")
+    args = list(case.decode_args(o, lse))
+    kw = case.decode_kwargs()
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "packed_start_offset": 16})
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "k_obmp": None})
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "combinadic_read": True})
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "k_fp4_mapscale": None})
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "k_format": "i4"})
+    bad = list(args); bad[0] = case.q[:, :3]
+    with pytest.raises(NotImplementedError):
+        ommx_paged_decode_attention_canonical(*bad, **kw)
+    bad = list(args); bad[1] = case.planes["k_base"].transpose(0, 1)
+    with pytest.raises(ValueError):
+        ommx_paged_decode_attention_canonical(*bad, **kw)
+    with pytest.raises(ValueError):          # k > 0 with no index plane at all
+        ommx_paged_decode_attention_canonical(*args, **{**kw, "bitmap_read": False})
+    ommx_paged_decode_attention_canonical(*args, **kw)
+    torch.cuda.synchronize()

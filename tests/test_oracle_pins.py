@@ -1,0 +1,301 @@
+"""Pins of the CPU oracle: golden planes from the reference packer, closed forms, invariants
+and brute force.  Each check is chosen so that a plausible slip in the oracle (wrong tie
+order, wrong rounding, transposed index, dropped term) fails it.  Runs on the CPU."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle.ommx_oracle as O
+from conftest import (GOLDEN_CASES, assert_planes_equal, bits_of, load_golden,
+                      tensor_from_bits)
+
+
+# ---- the composed packer against the reference's own output ---------------------------
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_pack_matches_reference_golden_planes(name):
+    z = load_golden(name)
+    K, V = tensor_from_bits(z["K_bits"]), tensor_from_bits(z["V_bits"])
+    planes = O.pack_kv(K, V, page_size=16, outliers_per_vector=6)
+    assert_planes_equal(planes, z, what=name)
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_dequant_matches_reference_golden(name):
+    z = load_golden(name)
+    planes = {k: tensor_from_bits(z[k]) for k in z if not k.endswith("_bits")}
+    planes["outliers_per_vector"] = 6
+    Kd, Vd = O.dequant_kv(planes)
+    assert np.array_equal(bits_of(Kd), z["K_dq_bits"])
+    assert np.array_equal(bits_of(Vd), z["V_dq_bits"])
+
+
+def test_gather_through_identity_tables_equals_linear_dequant():
+    z = load_golden("layer_outliers")
+    planes = {k: tensor_from_bits(z[k]) for k in z if not k.endswith("_bits")}
+    planes["outliers_per_vector"] = 6
+    Kd, Vd = O.dequant_kv(planes)
+    T = Kd.shape[0]
+    Kg, Vg = O.gather_request(planes, torch.arange(T // 16), torch.arange(T // 32), T, page_size=16)
+    assert torch.equal(Kg, Kd) and torch.equal(Vg, Vd)
+    # a shorter request sees a prefix
+    Kg2, _ = O.gather_request(planes, torch.arange(T // 16), torch.arange(T // 32), 64, page_size=16)
+    assert torch.equal(Kg2, Kd[:64])
+
+
+def test_gather_through_permuted_tables():
+    """Move pages and group slots around physically; the logical rows must not change."""
+    z = load_golden("layer_outliers")
+    planes = {k: tensor_from_bits(z[k]) for k in z if not k.endswith("_bits")}
+    planes["outliers_per_vector"] = 6
+    Kd, Vd = O.dequant_kv(planes)
+    T, P, G = Kd.shape[0], Kd.shape[0] // 16, Kd.shape[0] // 32
+    g = torch.Generator().manual_seed(3)
+    pp, gp = torch.randperm(P, generator=g), torch.randperm(G, generator=g)
+    moved = dict(planes)
+    for n in ("k_base", "v_main", "v_scale", "v_zp"):
+        t = torch.empty_like(planes[n]); t[pp] = planes[n]; moved[n] = t
+    for n in ("k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter"):
+        t = torch.empty_like(planes[n]); t[gp] = planes[n]; moved[n] = t
+    Kg, Vg = O.gather_request(moved, pp, gp, T, page_size=16)
+    assert torch.equal(Kg, Kd) and torch.equal(Vg, Vd)
+
+
+# ---- FP4 codec --------------------------------------------------------------------------
+
+def test_fp4_levels_are_fixed_points_and_codes_cover_the_table():
+    lv = torch.tensor(O.FP4_LEVELS)
+    x = torch.cat([lv, -lv])
+    assert torch.equal(O.fp4_decode(O.fp4_encode(x)), x)        # -0.0 == 0.0 under torch.equal
+    codes = torch.arange(16, dtype=torch.uint8)
+    want = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6])
+    assert torch.equal(O.fp4_decode(codes), want)
+    # sign bit follows x < 0 even when the level is 0; +-0 give code 0
+    assert O.fp4_encode(torch.tensor([-1e-9, 0.0, -0.0])).tolist() == [8, 0, 0]
+
+
+def test_fp4_encode_is_nearest_in_log_with_ties_down():
+    """Brute force in float64 away from the boundaries; exact geometric means go down."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.exp(torch.rand(20000, generator=g) * 14 - 11)         # 1.7e-5 .. 20
+    lv = np.array([1e-8, .5, 1, 1.5, 2, 3, 4, 6])
+    d = np.abs(np.log(x.double().numpy())[:, None] - np.log(lv)[None, :])
+    srt = np.sort(d, axis=1)
+    clear = (srt[:, 1] - srt[:, 0]) > 1e-4                           # not within fp32 noise of a tie
+    want = d.argmin(1)
+    got = (O.fp4_encode(x).to(torch.int64) & 7).numpy()
+    assert clear.sum() > 19000 and np.array_equal(got[clear], want[clear])
+    assert O.fp4_encode(torch.tensor([100.0, 6.0, 4.9, 4.89, 2.0])).tolist() == [7, 7, 7, 6, 4]
+
+
+def test_fp4_encode_monotone_over_all_floats_near_boundaries():
+    for lo, hi in zip(O.FP4_LEVELS[1:-1], O.FP4_LEVELS[2:]):
+        c = torch.tensor([math.sqrt(lo * hi)], dtype=torch.float32)
+        win = (c.view(torch.int32) + torch.arange(-200, 201, dtype=torch.int32)).view(torch.float32)
+        idx = (O.fp4_encode(win).to(torch.int64) & 7)
+        assert bool((idx[1:] >= idx[:-1]).all()) and idx[0] != idx[-1]
+
+
+# ---- bit layouts ------------------------------------------------------------------------
+
+def test_int2_layout_closed_form_and_round_trip():
+    codes = torch.tensor([[1, 2, 3, 0, 3, 3, 0, 1]])
+    plane = O.pack_int2(codes)
+    assert plane.tolist() == [[1 | 2 << 2 | 3 << 4 | 0 << 6, 3 | 3 << 2 | 0 << 4 | 1 << 6]]
+    g = torch.Generator().manual_seed(1)
+    c = torch.randint(0, 4, (7, 3, 64), generator=g)
+    assert torch.equal(O.unpack_int2(O.pack_int2(c)), c)
+
+
+def test_bitmap_layout_popcount_and_rank_rule():
+    pos = torch.tensor([[0, 7, 8, 15, 30, 31]])
+    bm = O.bitmap_pack(pos)
+    assert bm.tolist() == [[0x81, 0x81, 0x00, 0xC0]]
+    word = int.from_bytes(bytes(bm[0].tolist()), "little")
+    assert bin(word).count("1") == 6 and word >> 32 == 0
+    # nibble ordinal of a set bit == popcount of the lower set bits
+    for s, p in enumerate(pos[0].tolist()):
+        assert bin(word & ((1 << p) - 1)).count("1") == s
+    assert torch.equal(O.bitmap_unpack(bm, 6), pos)
+    with pytest.raises(ValueError):
+        O.bitmap_pack(torch.tensor([[1, 1, 2, 3, 4, 5]]))
+    with pytest.raises(ValueError):
+        O.bitmap_pack(torch.tensor([[1, 2, 3, 4, 5, 32]]))
+    with pytest.raises(ValueError):
+        O.bitmap_unpack(torch.tensor([[0xFF, 0, 0, 0]], dtype=torch.uint8), 6)
+
+
+def test_nibble_stream_even_slot_low():
+    v = torch.tensor([[1, 2, 3, 4, 5, 6]])
+    assert O.nibbles_pack(v).tolist() == [[0x21, 0x43, 0x65]]
+    assert torch.equal(O.nibbles_unpack(O.nibbles_pack(v), 6), v)
+    assert O.nibbles_pack(torch.tensor([[9, 8, 7]])).tolist() == [[0x89, 0x07]]
+
+
+def test_bytes_per_token_head_is_8_25_bits_per_pair():
+    assert O.plane_bytes_per_token_head(128, 6) == 132.0
+    assert O.plane_bytes_per_token_head(128, 6) * 8 / (2 * 128) == 4.125      # per element
+    assert 2 * 4.125 == 8.25
+
+
+# ---- power-of-two scale -----------------------------------------------------------------
+
+def test_pow2_rule_away_from_ties_and_exact_powers():
+    g = torch.Generator().manual_seed(2)
+    x = torch.exp(torch.rand(50000, generator=g) * 40 - 20)
+    e = O.pow2_exponent(x)
+    frac = np.log2(x.double().numpy()) - np.floor(np.log2(x.double().numpy()))
+    clear = np.abs(frac - 0.5) > 1e-4
+    assert np.array_equal(e.numpy()[clear], np.rint(np.log2(x.double().numpy()))[clear])
+    n = torch.arange(-39, 61, dtype=torch.float32)      # the rule clamps below 1e-12 ~ 2^-39.9
+    p = torch.pow(2.0, n)
+    assert torch.equal(p, torch.ldexp(torch.ones_like(n), n.to(torch.int32)))   # exact powers
+    assert torch.equal(O.pow2_exponent(p), n)                                    # lossless exponent
+    assert torch.equal(torch.exp2(n), p)
+
+
+def test_pow2_exact_log2_ties_round_half_to_even():
+    """Vectors whose (max-min)/3 has fp32 log2 exactly n+0.5 must land on the even exponent;
+    the same construction as the reference's tie test."""
+    hits = []
+    for n in range(-12, 6):
+        t = torch.tensor([3.0 * 2.0 ** (n + 0.5)], dtype=torch.float32)
+        cand = (t.view(torch.int32) + torch.arange(-8192, 8193, dtype=torch.int32)).view(torch.float32)
+        raw = cand.clamp_min(1e-8) / 3.0
+        hit = torch.log2(raw.clamp_min(1e-12)) == (n + 0.5)
+        if bool(hit.any()):
+            hits.append((n, float(cand[hit][0])))
+    if not hits:
+        pytest.skip("this libm produces no exact n+0.5 ties")
+    T = 32
+    K = torch.rand(T, 1, 32, generator=torch.Generator().manual_seed(7)) + 0.5
+    V = K.clone()
+    ramp = torch.arange(32, dtype=torch.float32) / 31.0
+    hits = hits[:32]
+    for j, (_, m) in enumerate(hits):
+        K[:, 0, j] = m * ramp
+        V[j, 0, :] = m * ramp
+    p = O.pack_kv(K, V, outliers_per_vector=0)
+    want = [n if n % 2 == 0 else n + 1 for n, _ in hits]
+    assert p["k_scale"][0, 0, :len(hits)].tolist() == want
+    assert p["v_scale"].reshape(T)[:len(hits)].tolist() == want
+
+
+# ---- outlier selection ------------------------------------------------------------------
+
+def _brute_select(w, k):
+    """Rank counting: lane i is in the top set iff fewer than kt lanes beat it, where j
+    beats i when w[j] > w[i] or (w[j] == w[i] and j < i); likewise for the bottom set on the
+    vector with the top lanes replaced by 1e9."""
+    kt, kb = (k + 1) // 2, k // 2
+    n = len(w)
+    top = [i for i in range(n)
+           if sum(1 for j in range(n) if w[j] > w[i] or (w[j] == w[i] and j < i)) < kt]
+    rest = [1e9 if i in top else w[i] for i in range(n)]
+    bot = [i for i in range(n)
+           if sum(1 for j in range(n) if rest[j] < rest[i] or (rest[j] == rest[i] and j < i)) < kb]
+    return sorted(set(top) | set(bot))
+
+
+@pytest.mark.parametrize("k", [2, 5, 6, 8])
+def test_signed_selection_matches_brute_force_with_heavy_ties(k):
+    g = torch.Generator().manual_seed(11 + k)
+    lv = torch.tensor([-3.0, -1.0, -1.0, 0.0, 0.0, 0.0, 0.5, 2.0, 2.0])
+    w = lv[torch.randint(0, 9, (200, 32), generator=g)]
+    w[0] = 1.25                                              # a constant vector
+    w[1, :16] = -2.0; w[1, 16:] = 2.0                        # two plateaus
+    mask = O.select_outliers_signed(w, k)
+    for r in range(w.shape[0]):
+        assert mask[r].nonzero().flatten().tolist() == _brute_select(w[r].tolist(), k), r
+    assert bool((mask.sum(-1) == k).all())
+
+
+def test_base_range_excludes_outliers_and_map_closed_form():
+    """One hand-built vector: the scale comes from the 26 inner lanes only, the FP4 map is
+    centred on the 6 outliers, and every stored value follows the closed forms."""
+    w = torch.linspace(-1.0, 1.0, 26).tolist() + [50.0, 40.0, 30.0, -50.0, -40.0, -20.0]
+    K = torch.tensor(w, dtype=torch.float32).reshape(32, 1, 1).repeat(1, 1, 32)
+    V = torch.zeros(32, 1, 32)
+    p = O.pack_kv(K, V, outliers_per_vector=6)
+    assert p["k_scale"][0, 0, 0].item() == round(math.log2(2.0 / 3.0))          # range 2 -> 2^-1
+    assert p["k_zp"][0, 0, 0].item() == -1.0
+    assert O.bitmap_unpack(p["k_obmp"], 6)[0, 0, 0].tolist() == [26, 27, 28, 29, 30, 31]
+    assert p["k_fp4_mapcenter"][0, 0, 0].item() == 0.0                           # (50 + -50)/2
+    ms = torch.tensor(12.0 / 100.0).to(torch.bfloat16)
+    assert p["k_fp4_mapscale"][0, 0, 0] == ms
+    lvl = O.fp4_decode(O.nibbles_unpack(p["k_oval"], 6))[0, 0, 0]
+    assert lvl.tolist() == [6.0, 4.0, 4.0, -6.0, -4.0, -2.0]                      # 50*.12=6, 4.8->4, 3.6->4, -2.4->-2
+    Kd, Vd = O.dequant_kv(p)
+    assert torch.equal(Kd[26:, 0, 0], lvl / ms.float() + 0.0)
+    inner = Kd[:26, 0, 0]
+    assert torch.equal(inner, torch.round((torch.tensor(w[:26]) + 1.0) / 0.5).clamp(0, 3) * 0.5 - 1.0)
+    # V all zeros: range clamps to 1e-8, exponent rint(log2(1e-8/3)) = -28, codes 0
+    assert int(p["v_scale"].flatten()[0]) == round(math.log2(1e-8 / 3.0)) and int(p["v_main"].sum()) == 0
+    assert torch.equal(Vd, torch.zeros_like(Vd))
+
+
+def test_pack_refuses_nonfinite_like_the_reference():
+    K = torch.randn(32, 1, 32); V = torch.randn(32, 1, 32)
+    Kbad = K.clone(); Kbad[3, 0, 5] = float("inf")
+    with pytest.raises((ValueError, IndexError)):
+        O.pack_kv(Kbad, V)
+    Vbad = V.clone(); Vbad[0, 0, 0] = float("nan")
+    with pytest.raises(ValueError):
+        O.pack_kv(K, Vbad)
+
+
+# ---- attention and the split merge --------------------------------------------------------
+
+def test_attend_equals_torch_softmax_and_fp64():
+    g = torch.Generator().manual_seed(4)
+    K = torch.randn(300, 2, 64, generator=g); V = torch.randn(300, 2, 64, generator=g)
+    q = torch.randn(4, 64, generator=g)
+    o32, l32 = O.attend(q, K, V, 0.125, dtype=torch.float32)
+    o64, l64 = O.attend(q, K, V, 0.125, dtype=torch.float64)
+    for h in range(4):
+        s = (K[:, h // 2].double() @ q[h].double()) * 0.125
+        want = torch.softmax(s, 0) @ V[:, h // 2].double()
+        assert torch.allclose(o64[h], want, atol=1e-12)
+        assert abs(l64[h].item() - torch.logsumexp(s, 0).item()) < 1e-12
+    assert (o32.double() - o64).abs().max() < 1e-5 and (l32.double() - l64).abs().max() < 1e-5
+    # one token: output is that token's V; uniform K: output is the mean of V
+    o1, l1 = O.attend(q, K[:1], V[:1], 0.5, dtype=torch.float64)
+    assert torch.allclose(o1[3], V[0, 1].double())
+    ou, _ = O.attend(q, torch.zeros(10, 2, 64), V[:10], 1.0, dtype=torch.float64)
+    assert torch.allclose(ou[0], V[:10, 0].double().mean(0))
+    oe, le = O.attend(q, K[:0], V[:0], 1.0)
+    assert float(oe.abs().sum()) == 0.0 and bool(torch.isinf(le).all())
+
+
+@pytest.mark.parametrize("S", [1, 2, 3, 8, 64])
+def test_split_merge_is_independent_of_the_split_count(S):
+    g = torch.Generator().manual_seed(6)
+    L = 1000
+    K = torch.randn(L, 1, 32, generator=g); V = torch.randn(L, 1, 32, generator=g)
+    q = torch.randn(2, 32, generator=g)
+    want_o, want_l = O.attend(q, K, V, 0.2, dtype=torch.float64)
+    parts = [O.attend(q, K[a:b], V[a:b], 0.2, dtype=torch.float64) for a, b in O.split_bounds(L, S)]
+    o, l = O.merge_states(torch.stack([p[0] for p in parts]), torch.stack([p[1] for p in parts]))
+    assert torch.allclose(o, want_o, atol=1e-12) and torch.allclose(l, want_l, atol=1e-12)
+
+
+def test_split_bounds_rounding_and_empty_splits():
+    assert O.split_bounds(960, 4) == [(0, 256), (256, 512), (512, 768), (768, 960)]
+    b = O.split_bounds(96, 8)                       # per = 32: five splits are empty
+    assert b[:3] == [(0, 32), (32, 64), (64, 96)] and all(a >= e for a, e in b[3:])
+    o, l = O.merge_states(torch.zeros(3, 2, 4), torch.full((3, 2), -math.inf))
+    assert float(o.abs().sum()) == 0.0 and bool(torch.isinf(l).all())
+
+
+def test_window_closed_forms_and_invariant():
+    assert O.packed_boundary(1024) == 968 and O.packed_boundary(4096) == 4040
+    assert O.packed_boundary(65536) == 65480 and O.packed_boundary(40) == 8 and O.packed_boundary(5) == 5
+    for n in range(0, 400):
+        b = O.packed_boundary(n)
+        if n >= 40:
+            assert 32 <= n - b < 64 and (b - 8) % 32 == 0
+        ti = O.tail_indices(n)
+        assert len(ti) == len(set(ti)) and len(ti) <= 72
+        assert sorted(ti + list(range(min(8, n), max(min(8, n), b)))) == list(range(n))

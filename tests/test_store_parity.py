@@ -1,0 +1,215 @@
+"""HIP quantize-on-store against the reference packer's golden planes and the CPU oracle.
+Bit-exact on every plane.  All calls go through the C ABI (ctypes)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle.ommx_oracle as O
+from conftest import (GOLDEN_CASES, PLANE_NAMES, assert_planes_equal, bits_of, load_golden,
+                      tensor_from_bits)
+from open_ommx_serve_amd.attention import pack as hip_pack
+from open_ommx_serve_amd.attention.pack import (alloc_planes, ommx_pack_kv_canonical_block,
+                                                store_pack_into)
+from open_ommx_serve_amd.synth import synth_kv
+
+pytestmark = pytest.mark.gpu
+
+RECIPE = dict(outliers_per_vector=6, outlier_select="signed", outlier_repr="bitmap",
+              k_format="i2f4", use_pow2=True, page_size=16)
+
+
+def _hip(K, V, **kw):
+    r = dict(RECIPE); r.update(kw)
+    return ommx_pack_kv_canonical_block(K.cuda(), V.cuda(), **r)
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_store_matches_reference_golden_planes(name):
+    z = load_golden(name)
+    K, V = tensor_from_bits(z["K_bits"]), tensor_from_bits(z["V_bits"])
+    planes = _hip(K, V)
+    assert planes["k_base"].device.type == "cpu"            # default output device, like the reference
+    assert_planes_equal(planes, z, what=name)
+    for key in ("head_dim", "n_kv_heads", "num_tokens", "n_groups", "page_size",
+                "outliers_per_vector", "outlier_repr", "outlier_select", "group_tokens",
+                "group_channels", "k_format", "v_format", "k_base_bits", "oval_bits",
+                "use_pow2", "kv_outlier_map", "kv_int8_scale", "k_field_bytes",
+                "req_to_token", "req_to_group", "k_oidx", "k_crank"):
+        assert key in planes
+    assert planes["k_field_bytes"] == 4 and planes["k_oidx"] is None
+
+
+@pytest.mark.parametrize("seed,T,H,D", [(1, 32, 1, 32), (2, 96, 3, 64), (3, 256, 8, 128),
+                                        (4, 64, 2, 256), (5, 960, 8, 128)])
+def test_store_matches_oracle_random_bf16(seed, T, H, D):
+    K, V = synth_kv(T, H, D, seed, outlier_channels=min(4, D // 8), sparse_frac=0.01)
+    assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what=f"seed{seed}")
+
+
+@pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
+def test_store_other_outlier_counts(k):
+    K, V = synth_kv(128, 2, 64, 10 + k)
+    want = O.pack_kv(K, V, outliers_per_vector=k)
+    got = _hip(K, V, outliers_per_vector=k)
+    names = PLANE_NAMES if k > 0 else ("k_base", "k_scale", "k_zp", "v_main", "v_scale", "v_zp")
+    for n in names:
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+    if k == 0:
+        assert got["k_obmp"] is None and got["k_oval"] is None and got["kv_outlier_map"] is False
+
+
+def test_store_heavy_ties_and_degenerate_vectors():
+    g = torch.Generator().manual_seed(77)
+    lv = torch.tensor([-4.0, -1.0, -1.0, 0.0, 0.0, 0.0, 0.25, 2.0, 2.0, 8.0])
+    K = lv[torch.randint(0, 10, (128, 2, 64), generator=g)].to(torch.bfloat16)
+    V = lv[torch.randint(0, 10, (128, 2, 64), generator=g)].to(torch.bfloat16)
+    K[:32, 0, 0] = 3.0            # constant K vector: every range clamps to 1e-8
+    V[0, 0, :32] = -7.0           # constant V vector
+    K[32:64, 1, 5] = 0.0
+    assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what="ties")
+
+
+def test_store_fp32_inputs_round_zero_point_and_map():
+    g = torch.Generator().manual_seed(9)
+    K = torch.randn(128, 2, 64, generator=g) * 3.0
+    V = torch.randn(128, 2, 64, generator=g) * torch.exp2(torch.randint(-10, 8, (128, 2, 1), generator=g).float())
+    assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what="fp32")
+
+
+def test_store_scale_rounding_points_across_binades():
+    """Vectors whose range/3 sits within a few ulps of sqrt(2)*2^n, where the reference's fp32
+    log2 decides the exponent: the kernel has to take the same side for every n."""
+    rows = []
+    for n in range(-20, 12):
+        c = torch.tensor([3.0 * 2.0 ** (n + 0.5)], dtype=torch.float32)
+        rows.append((c.view(torch.int32) + torch.arange(-16, 16, dtype=torch.int32)).view(torch.float32))
+    m = torch.stack(rows)                                    # [32 binades, 32 neighbours]
+    ramp = torch.arange(32, dtype=torch.float32) / 31.0
+    # V: token t = (binade), channel group j = neighbour  -> vector = m[t, j] * ramp
+    V = (m.unsqueeze(-1) * ramp).reshape(32, 1, 32 * 32)[:, :, :256].contiguous()
+    V = torch.cat([V, (m[:, 8:16].unsqueeze(-1) * ramp).reshape(32, 1, 256)], 1)
+    K = V.clone()
+    got = _hip(K, V, outliers_per_vector=0)
+    want = O.pack_kv(K, V, outliers_per_vector=0)
+    for nme in ("k_base", "k_scale", "k_zp", "v_main", "v_scale", "v_zp"):
+        assert np.array_equal(bits_of(got[nme]), bits_of(want[nme])), nme
+
+
+def test_store_fp4_rounding_points():
+    """Outliers whose mapped value sits within a few ulps of an FP4 level boundary."""
+    bounds = [7.0710678e-05, 0.70710678, 1.2247449, 1.7320508, 2.4494897, 3.4641016, 4.8989795]
+    K = torch.zeros(32, 1, 256)
+    g = torch.Generator().manual_seed(3)
+    K[:] = torch.randn(32, 1, 256, generator=g) * 0.01
+    col = 0
+    for b in bounds:
+        c = torch.tensor([b], dtype=torch.float32)
+        for step in range(-18, 18):
+            x = (c.view(torch.int32) + step).view(torch.float32).item()
+            # outliers +6-ish top and -6 bottom fix the map to centre 0, scale 1
+            K[0, 0, col], K[1, 0, col], K[2, 0, col] = 6.0, 5.0, x if x > 0.05 else 5.5
+            K[3, 0, col], K[4, 0, col], K[5, 0, col] = -6.0, -5.0, -x if x > 0.05 else -5.5
+            col += 1
+            if col == 256:
+                break
+        if col == 256:
+            break
+    V = torch.randn(32, 1, 256, generator=g)
+    assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what="fp4-bounds")
+
+
+def test_store_into_pool_with_tables_and_ring_gather():
+    """Pages and group slots chosen by tables, source rows gathered from a shuffled ring."""
+    T, H, D, ps = 128, 2, 64, 16
+    K, V = synth_kv(T, H, D, 21)
+    want = O.pack_kv(K, V)
+    g = torch.Generator().manual_seed(4)
+    perm = torch.randperm(T, generator=g)
+    ringK = torch.empty(T + 5, H, D, dtype=torch.bfloat16); ringV = torch.empty_like(ringK)
+    ringK[perm] = K; ringV[perm] = V                               # token t lives in ring row perm[t]
+    pool_pages, pool_groups = 20, 9
+    planes = alloc_planes(pool_pages, pool_groups, H, D, page_size=ps, device="cuda")
+    for t in planes.values():
+        if torch.is_tensor(t):
+            t.fill_(0x5A if t.dtype == torch.uint8 else 1)
+    pages = torch.randperm(pool_pages, generator=g)[:T // ps].to(torch.int32)
+    groups = torch.randperm(pool_groups, generator=g)[:T // 32].to(torch.int32)
+    err = torch.zeros(1, dtype=torch.int32, device="cuda")
+    store_pack_into(ringK.cuda(), ringV.cuda(), planes, page_size=ps,
+                    src_rows=perm.to(torch.int32).cuda(), dst_pages=pages.cuda(),
+                    dst_groups=groups.cuda(), err_flag=err)
+    assert int(err.item()) == 0
+    for n in ("k_base", "v_main", "v_scale", "v_zp"):
+        assert np.array_equal(bits_of(planes[n][pages.long().cuda()]), bits_of(want[n])), n
+        untouched = torch.ones(pool_pages, dtype=torch.bool); untouched[pages.long()] = False
+        ref = torch.full_like(planes[n][untouched.cuda()].cpu(), 0x5A if planes[n].dtype == torch.uint8 else 1)
+        assert torch.equal(planes[n][untouched.cuda()].cpu(), ref), f"{n}: a foreign page was written"
+    for n in ("k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter"):
+        assert np.array_equal(bits_of(planes[n][groups.long().cuda()]), bits_of(want[n])), n
+
+
+def test_store_page_sizes():
+    K, V = synth_kv(64, 2, 64, 31)
+    for ps in (8, 16, 32):
+        assert_planes_equal(_hip(K, V, page_size=ps), O.pack_kv(K, V, page_size=ps), what=f"ps{ps}")
+
+
+def test_store_refuses_nonfinite_and_bad_arguments():
+    K, V = synth_kv(64, 1, 64, 41)
+    Kb = K.clone(); Kb[3, 0, 5] = float("inf")
+    with pytest.raises((ValueError, IndexError)):
+        _hip(Kb, V)
+    Kn = K.clone(); Kn[:, 0, 7] = float("nan")
+    with pytest.raises((ValueError, IndexError)):
+        _hip(Kn, V)
+    Vb = V.clone(); Vb[0, 0, 0] = float("nan")
+    with pytest.raises(ValueError):
+        _hip(K, Vb)
+    with pytest.raises(ValueError):
+        _hip(K[:48], V[:48])                       # not a multiple of 32
+    with pytest.raises(ValueError):
+        _hip(K, V[:32])
+    with pytest.raises(ValueError):
+        _hip(K, V, outlier_repr="nope")
+    with pytest.raises(ValueError):
+        _hip(K, V, outliers_per_vector=33)
+    with pytest.raises(NotImplementedError):
+        _hip(K, V, outlier_repr="relidx7")
+    _hip(K, V)                                     # and a good call still works afterwards
+
+
+def test_store_prefill_sized_block_is_bit_exact():
+    """4032 tokens of the 8-head, 128-channel layer (the store of the ctx-4096 case)."""
+    K, V = synth_kv(4032, 8, 128, 42, sparse_frac=0.005)
+    assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what="ctx4096")
+
+
+def test_store_bulk_32k_block_invariants_and_sampled_parity():
+    """32704 tokens (bulk prefill store): every frame holds exactly 6 outliers, codes of
+    constant groups obey the closed form, and 64 sampled groups are bit-exact."""
+    T, H, D = 32704, 8, 128
+    K, V = synth_kv(T, H, D, 43, sparse_frac=0.005)
+    planes = _hip(K, V, device="cuda")
+    bm = planes["k_obmp"].view(torch.int32).reshape(-1)
+    pop = torch.zeros_like(bm)
+    for i in range(32):
+        pop += (bm >> i) & 1
+    assert bool((pop == 6).all())
+    g = np.random.default_rng(0).choice(T // 32, size=64, replace=False)
+    for gi in g.tolist():
+        sl = slice(gi * 32, gi * 32 + 32)
+        want = O.pack_kv(K[sl], V[sl])
+        for n in ("k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter"):
+            assert np.array_equal(bits_of(planes[n][gi]), bits_of(want[n][0])), (n, gi)
+        for n in ("k_base", "v_main", "v_scale", "v_zp"):
+            assert np.array_equal(bits_of(planes[n][2 * gi:2 * gi + 2]), bits_of(want[n])), (n, gi)
+
+
+def test_decision_table_measured_on_this_host_is_monotone_and_near_the_exact_one():
+    t = hip_pack.measure_store_table()
+    d = torch.zeros(264)
+    from open_ommx_serve_amd.attention import _hip as H
+    H.load().ommx_store_default_table(d.data_ptr())
+    ulps = (t[88:254].view(torch.int32) - d[88:254].view(torch.int32)).abs()
+    assert int(ulps.max()) <= 64
+    assert bool((t[257:264][1:] > t[257:264][:-1]).all())
