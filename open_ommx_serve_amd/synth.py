@@ -120,7 +120,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     packed = [win.packed_len(int(n)) for n in seq_lens]
     n_pages = [p // ps for p in packed]
     n_groups = [p // 32 for p in packed]
-    tot_pages, tot_groups = max(1, sum(n_pages)), max(1, sum(n_groups))
+    # at least one whole group (32 // ps pages), so the planes keep the 32-token geometry
+    tot_pages, tot_groups = max(32 // ps, sum(n_pages)), max(1, sum(n_groups))
     g = _rng(seed, 424242)
     page_ids = g.permutation(tot_pages) if permute_tables else np.arange(tot_pages)
     # group slots follow their pages only through the tables, so shuffle them separately
