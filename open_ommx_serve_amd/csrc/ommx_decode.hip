@@ -1,9 +1,471 @@
-// Tuned split-KV decode kernel (placeholder selection: nothing covered yet).
+// Tuned split-KV decode kernel for gfx950: head_dim 128, 4 q heads per kv head, 6 (or 0)
+// outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
+//
+// Work decomposition.  A wavefront owns one kv head of one split and walks it 64 tokens
+// (two 32-token K groups) at a time; waves never synchronise with each other.  A
+// workgroup is 4 waves = 4 neighbouring kv heads, so together they consume whole 128-byte
+// lines of the token-major k_base / v_main rows.
+//
+// Arithmetic.  All dot products run on the matrix pipe (v_mfma_f32_16x16x32, fp32
+// accumulate) with operands that are EXACT in their 16-bit type:
+//   K base   B = (1 + code/4) * 2^e   bf16, built with one shift and one and-or per channel
+//            pair: the 2-bit code lands in the two top mantissa bits of a bf16 whose
+//            exponent field already holds the group's power-of-two scale;
+//            A = 4*q (bf16).  sum A*B = sum q*code*s + 4*sum q*s, the second term and
+//            sum q*zp come out of one small "bias" MFMA per 64 tokens.
+//   outliers a per-group tile [32 tokens][128 channels] of (outlier - base)/4 in f16,
+//            scattered by a channel-major pass (one lane = two channels), consumed as the
+//            B operand of an f16 MFMA against A = 4*q (f16).
+//   P.V      B = (1 + code/4) f16 for 8 tokens of one channel (V rows are transposed
+//            through LDS at dword granularity), A = p * 2^e_v (f16, exact scaling);
+//            sum_t p*vs and sum_t p*vz come from one extra MFMA per 32 tokens.
+// MFMA row groups are used as selectors: rows 4x..4x+3 carry the 4 q heads for token
+// block x (QK) or for V channel group x (P.V); a lane keeps the row group that matches
+// its column.
 #include "ommx_decode_args.h"
 
 namespace ommx {
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int D = 128;
+// per-wave LDS map (bytes)
+constexpr int OFF_MAGIC = 0;       // [2 groups][64 pairs] bf16x2: 2^e of channels (p, p+8)
+constexpr int OFF_ZPP = 512;       // same order, bf16 zero points
+constexpr int OFF_KT = 1024;       // [64 tokens][32 B] K code rows
+constexpr int OFF_VT = 3072;       // [8 dword columns][64 tokens] V code dwords
+constexpr int OFF_PT = 5120;       // [4 heads][64 tokens] f16 softmax weights
+constexpr int OFF_VS = 5632;       // [4 channel groups][64 tokens] f16 2^e_v
+constexpr int OFF_VZ = 6144;       // [4 channel groups][64 tokens] f16 v zero points
+constexpr int OFF_DT = 6656;       // [32 tokens][DT_ROW B] f16 outlier deltas of one group
+constexpr int DT_ROW = 272;
+constexpr int WAVE_LDS = OFF_DT + 32 * DT_ROW;      // 15360
+
+__device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma_f16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ void lds_fence() {
+    // LDS traffic of one wave is executed in order; this only stops the compiler from
+    // moving accesses across a point where lanes exchange data through LDS.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+__device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
+    const f16x2 r = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// K pair p of a code dword: channels p (low half) and p+8 (high half) as bf16 (1+c/4)*2^e.
+template <int P>
+__device__ __forceinline__ uint32_t k_pair(uint32_t w, uint32_t magic) {
+    const uint32_t sh = (2 * P >= 5) ? (w >> (2 * P - 5 < 0 ? 0 : 2 * P - 5))
+                                     : (w << (5 - 2 * P < 0 ? 0 : 5 - 2 * P));
+    return (sh & 0x00600060u) | magic;
+}
+// V channel y of a merged dword (token a in the low 16 bits, token b in the high 16 bits).
+template <int Y>
+__device__ __forceinline__ uint32_t v_pair(uint32_t m) {
+    const uint32_t sh = (2 * Y >= 8) ? (m >> (2 * Y - 8 < 0 ? 0 : 2 * Y - 8))
+                                     : (m << (8 - 2 * Y < 0 ? 0 : 8 - 2 * Y));
+    return (sh & 0x03000300u) | 0x3C003C00u;
+}
+
+template <bool OUTLIERS>
+__global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint8_t* const sm = smem_all + wave * WAVE_LDS;
+    const int j = lane & 15, kq = lane >> 4;
+    const int Hkv = a.Hkv;
+    const int waves = blockDim.x >> 6;
+    const int kvh = blockIdx.y * waves + wave;
+    const int b = blockIdx.z, sp = blockIdx.x;
+    const int L = a.seq[b];
+    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
+    const int n_begin = per * sp;
+    const int n_end = min(n_begin + per, L);
+    const int64_t tok_base = (int64_t)a.gbase * 32 + a.off;
+    const float c_log2e = 1.4426950408889634f;
+    const float qk_scale = a.sm_scale * c_log2e;
+
+    // ---- A operands: 4*q of head j%4 for this lane's 32-channel quarter ---------------
+    // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
+    // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
+    u32x4 aq_pair[4], aq_nat[4];
+    {
+        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(kvh * 4 + (j & 3)) * a.q_sh + 32 * kq;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
+                const float lo = 4.0f * bf16_to_f32(qh[cl]), hi = 4.0f * bf16_to_f32(qh[cl + 8]);
+                aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
+                const float n0 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr]);
+                const float n1 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr + 1]);
+                aq_nat[ks][rr] = pack_f16x2(n0, n1);
+            }
+        }
+    }
+
+    if (OUTLIERS) {   // the outlier tile starts out all zero; readers clear what they consume
+        u32x4* dt = reinterpret_cast<u32x4*>(sm + OFF_DT);
+        for (int i = lane; i < 32 * DT_ROW / 16; i += 64) dt[i] = u32x4{0, 0, 0, 0};
+    }
+
+    f32x4 acc[8];
+    f32x4 accz = {0, 0, 0, 0};
+#pragma unroll
+    for (int y = 0; y < 8; ++y) acc[y] = f32x4{0, 0, 0, 0};
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { m_run[r] = -INFINITY; l_run[r] = 0.0f; }
+
+    const int64_t row_bytes = (int64_t)Hkv * 32;          // k_base / v_main bytes per token row
+
+    for (int n0 = n_begin; n0 < n_end; n0 += 64) {
+        // ---------------------------------------------------------------- addressing
+        const int last = n_end - 1;
+        int64_t rows[4];
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            const int64_t p = (int64_t)min(n0 + 16 * tb + j, last) + tok_base;
+            rows[tb] = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
+        }
+        const int my_tok = n0 + lane;
+        const bool tok_ok = my_tok < n_end;
+        int64_t my_row;
+        {
+            const int64_t p = (int64_t)min(my_tok, last) + tok_base;
+            my_row = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
+        }
+        int64_t gidx[2];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const int gi = min(n0 / 32 + g, last / 32);
+            gidx[g] = (table_at(a.rg, b * a.rg_s + a.gbase + gi, a.i64) * Hkv + kvh) * D;
+        }
+
+        // ---------------------------------------------------------------- loads
+        u32x2 kw[4], vw[4];
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            kw[tb] = *reinterpret_cast<const u32x2*>(a.k_base + rows[tb] * row_bytes + kvh * 32 + 8 * kq);
+            vw[tb] = *reinterpret_cast<const u32x2*>(a.v_main + rows[tb] * row_bytes + kvh * 32 + 8 * kq);
+        }
+        const uint32_t vsc = *reinterpret_cast<const uint32_t*>(a.v_scale + (my_row * Hkv + kvh) * 4);
+        const u32x2 vzp = *reinterpret_cast<const u32x2*>(a.v_zp + (my_row * Hkv + kvh) * 4);
+
+        // channel pair (2*lane, 2*lane+1) parameters of both groups
+        uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
+        u32x2 g_bm[2], g_ov[2];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            g_sc[g] = *reinterpret_cast<const uint16_t*>(a.k_scale + gidx[g] + 2 * lane);
+            g_zp[g] = *reinterpret_cast<const uint32_t*>(a.k_zp + gidx[g] + 2 * lane);
+            if (OUTLIERS) {
+                g_ms[g] = *reinterpret_cast<const uint32_t*>(a.k_ms + gidx[g] + 2 * lane);
+                g_mc[g] = *reinterpret_cast<const uint32_t*>(a.k_mc + gidx[g] + 2 * lane);
+                g_bm[g] = *reinterpret_cast<const u32x2*>(a.k_obmp + (gidx[g] + 2 * lane) * 4);
+                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(a.k_oval + gidx[g] * 3) + (3 * lane) / 2;
+                g_ov[g] = u32x2{ovp[0], ovp[1]};
+            }
+        }
+
+        // ---------------------------------------------------------------- stage to LDS
+        // K code rows (for the outlier pass), transposed V dwords
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            *reinterpret_cast<u32x2*>(sm + OFF_KT + (16 * tb + j) * 32 + 8 * kq) = kw[tb];
+            uint32_t* vt = reinterpret_cast<uint32_t*>(sm + OFF_VT);
+            vt[(2 * kq) * 64 + 16 * tb + j] = vw[tb][0];
+            vt[(2 * kq + 1) * 64 + 16 * tb + j] = vw[tb][1];
+        }
+        // V scales / zero points of this lane's token as f16, [group][token]
+        {
+            uint16_t* vs16 = reinterpret_cast<uint16_t*>(sm + OFF_VS);
+            uint16_t* vz16 = reinterpret_cast<uint16_t*>(sm + OFF_VZ);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int e = static_cast<int8_t>((vsc >> (8 * g4)) & 0xFFu);
+                float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                const uint32_t zb = (g4 & 1) ? (vzp[g4 >> 1] & 0xFFFF0000u) : (vzp[g4 >> 1] << 16);
+                float z = __uint_as_float(zb);
+                if (!tok_ok) { s = 0.0f; z = 0.0f; }
+                vs16[g4 * 64 + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(s));
+                vz16[g4 * 64 + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
+            }
+        }
+        // per-channel 2^e and zp in pair order
+        {
+            uint16_t* mg = reinterpret_cast<uint16_t*>(sm + OFF_MAGIC);
+            uint16_t* zp = reinterpret_cast<uint16_t*>(sm + OFF_ZPP);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int c = 2 * lane + u;
+                    const int y = c & 15;
+                    const int hw = (((c >> 4) * 8) + (y & 7)) * 2 + (y >> 3);
+                    const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
+                    mg[g * 128 + hw] = static_cast<uint16_t>((e + 127) << 7);
+                    zp[g * 128 + hw] = static_cast<uint16_t>(u ? (g_zp[g] >> 16) : (g_zp[g] & 0xFFFFu));
+                }
+            }
+        }
+        lds_fence();
+
+        // ---------------------------------------------------------------- QK base
+        f32x4 dq[4];
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) {
+            const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + (tb >> 1) * 256 + kq * 64);
+            const u32x4 m0 = mg[0], m1 = mg[1], m2 = mg[2], m3 = mg[3];
+            const uint32_t w0 = kw[tb][0], w1 = kw[tb][1];
+            f32x4 d = {0, 0, 0, 0};
+            d = mfma_bf16(aq_pair[0], u32x4{k_pair<0>(w0, m0[0]), k_pair<1>(w0, m0[1]), k_pair<2>(w0, m0[2]), k_pair<3>(w0, m0[3])}, d);
+            d = mfma_bf16(aq_pair[1], u32x4{k_pair<4>(w0, m1[0]), k_pair<5>(w0, m1[1]), k_pair<6>(w0, m1[2]), k_pair<7>(w0, m1[3])}, d);
+            d = mfma_bf16(aq_pair[2], u32x4{k_pair<0>(w1, m2[0]), k_pair<1>(w1, m2[1]), k_pair<2>(w1, m2[2]), k_pair<3>(w1, m2[3])}, d);
+            d = mfma_bf16(aq_pair[3], u32x4{k_pair<4>(w1, m3[0]), k_pair<5>(w1, m3[1]), k_pair<6>(w1, m3[2]), k_pair<7>(w1, m3[3])}, d);
+            dq[tb] = d;
+        }
+        // bias columns: 0 zp(g0) 1 zp(g1) 2 2^e(g0) 3 2^e(g1); other columns repeat them
+        f32x4 dbias = {0, 0, 0, 0};
+        {
+            const int src = ((j & 2) ? OFF_MAGIC : OFF_ZPP) + (j & 1) * 256 + kq * 64;
+            const u32x4* bp = reinterpret_cast<const u32x4*>(sm + src);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) dbias = mfma_bf16(aq_pair[ks], bp[ks], dbias);
+        }
+
+        // ---------------------------------------------------------------- outliers
+        // delta = (outlier - base)/4 goes through the tile twice: its f16 rounding first,
+        // then the f16 rounding of what the first pass left over, so that the pair carries
+        // ~22 significant bits (a single f16 is not enough for outliers of magnitude 100+).
+        if (OUTLIERS) {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                uint32_t lo_pk[2][3];     // residuals, two f16 per register
+                uint32_t pos_pk[2];       // six 5-bit token positions per channel
+                // channel pass: lane owns channels 2*lane, 2*lane+1 of group g
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int c = 2 * lane + u;
+                    const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
+                    const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                    const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
+                    const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
+                    const float mc = __uint_as_float(u ? (g_mc[g] & 0xFFFF0000u) : (g_mc[g] << 16));
+                    const float inv_ms = __builtin_amdgcn_rcpf(ms);
+                    uint32_t bm = g_bm[g][u];
+                    // 6 nibbles of this channel: bytes 3c..3c+2 of the block
+                    const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
+                    const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
+                    const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                    const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
+                    const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
+                    const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
+                    const uint8_t* kt = sm + OFF_KT + g * 1024 + (c >> 2);
+                    uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
+                    float lo[6];
+                    uint32_t pp = 0;
+#pragma unroll
+                    for (int sidx = 0; sidx < 6; ++sidx) {
+                        lo[sidx] = 0.0f;
+                        if (bm != 0) {
+                            const int pos = __ffs(bm) - 1;
+                            bm &= bm - 1;
+                            pp |= static_cast<uint32_t>(pos) << (5 * sidx);
+                            const float val = fmaf(lv[sidx], inv_ms, mc);
+                            const uint32_t code = (static_cast<uint32_t>(kt[pos * 32]) >> (2 * (c & 3))) & 3u;
+                            const float base = fmaf(static_cast<float>(code), s, zp);
+                            const float dl = (val - base) * 0.25f;
+                            const _Float16 hi = static_cast<_Float16>(dl);
+                            lo[sidx] = dl - static_cast<float>(hi);
+                            dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
+                        }
+                    }
+                    pos_pk[u] = pp;
+                    lo_pk[u][0] = pack_f16x2(lo[0], lo[1]);
+                    lo_pk[u][1] = pack_f16x2(lo[2], lo[3]);
+                    lo_pk[u][2] = pack_f16x2(lo[4], lo[5]);
+                }
+#pragma unroll
+                for (int pass = 0; pass < 2; ++pass) {
+                    if (pass == 1) {
+                        // the tile is all zero again: scatter the residuals to the same places
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + 2 * lane + u;
+#pragma unroll
+                            for (int sidx = 0; sidx < 6; ++sidx) {
+                                const int pos = (pos_pk[u] >> (5 * sidx)) & 31;
+                                const uint32_t w = lo_pk[u][sidx >> 1];
+                                const uint16_t hw = static_cast<uint16_t>((sidx & 1) ? (w >> 16) : (w & 0xFFFFu));
+                                if (hw != 0) dt[pos * (DT_ROW / 2)] = hw;
+                            }
+                        }
+                    }
+                    lds_fence();
+                    // token blocks 2g, 2g+1 read their rows of the tile and clear them
+#pragma unroll
+                    for (int t2 = 0; t2 < 2; ++t2) {
+                        u32x4* row = reinterpret_cast<u32x4*>(sm + OFF_DT + (16 * t2 + j) * DT_ROW + 64 * kq);
+                        f32x4 d = dq[2 * g + t2];
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) {
+                            const u32x4 bt = row[ks];
+                            row[ks] = u32x4{0, 0, 0, 0};
+                            d = mfma_f16(aq_nat[ks], bt, d);
+                        }
+                        dq[2 * g + t2] = d;
+                    }
+                    lds_fence();
+                }
+            }
+        }
+
+        // ---------------------------------------------------------------- softmax
+        // bias of (group, head r): 0.25*ZP' - S1' ; columns 0..3 live in lanes 0..3 (kq 0)
+        float logit[4];
+        {
+            const f32x4 dsel = kq == 0 ? dq[0] : (kq == 1 ? dq[1] : (kq == 2 ? dq[2] : dq[3]));
+            const int gsel = lane >> 5;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float zpv = __shfl(dbias[r], gsel);          // column gsel, rows 0..3
+                const float s1v = __shfl(dbias[r], 2 + gsel);
+                const float raw = dsel[r] + (0.25f * zpv - s1v);
+                float x = raw * a.sm_scale;
+                x = apply_cap(x, a.cap) * c_log2e;
+                logit[r] = tok_ok ? x : -INFINITY;
+            }
+        }
+        float alpha[4], p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float mx = wave_max(logit[r]);
+            const float m_new = fmaxf(m_run[r], mx);
+            alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : exp2f(m_run[r] - m_new);
+            p[r] = tok_ok ? exp2f(logit[r] - m_new) : 0.0f;
+            m_run[r] = m_new;
+        }
+        {
+            uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const _Float16 ph = static_cast<_Float16>(p[r]);
+                // accumulate the weight that P.V really uses (the f16-rounded one)
+                l_run[r] = l_run[r] * alpha[r] + static_cast<float>(ph);
+                pt[r * 64 + lane] = __builtin_bit_cast(uint16_t, ph);
+            }
+        }
+#pragma unroll
+        for (int y = 0; y < 8; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[y][r] *= alpha[r];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) accz[r] *= alpha[r];
+        lds_fence();
+
+        // ---------------------------------------------------------------- P.V
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int t0 = 32 * kb + 8 * kq;
+            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & 3) * 64 + t0) * 2);
+            const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * 64 + t0) * 2);
+            const u32x4 apv = {pk_mul_f16(pw[0], sw[0]), pk_mul_f16(pw[1], sw[1]),
+                               pk_mul_f16(pw[2], sw[2]), pk_mul_f16(pw[3], sw[3])};
+            // columns 0..3: vz of channel group j, columns 4..7: vs; others repeat
+            const u32x4 bz = *reinterpret_cast<const u32x4*>(
+                sm + ((j & 4) ? OFF_VS : OFF_VZ) + ((j & 3) * 64 + t0) * 2);
+            accz = mfma_f16(pw, bz, accz);
+            // V codes: dword column j%8, half j/8, tokens t0..t0+7
+            const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (j & 7) * 64 + t0;
+            const u32x4 va = *reinterpret_cast<const u32x4*>(vt);
+            const u32x4 vb = *reinterpret_cast<const u32x4*>(vt + 4);
+            const uint32_t sel = (j & 8) ? 0x07060302u : 0x05040100u;
+            const uint32_t mg0 = __builtin_amdgcn_perm(va[1], va[0], sel);
+            const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], sel);
+            const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], sel);
+            const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], sel);
+#define OMMX_PV(Y) acc[Y] = mfma_f16(apv, u32x4{v_pair<Y>(mg0), v_pair<Y>(mg1), v_pair<Y>(mg2), v_pair<Y>(mg3)}, acc[Y]);
+            OMMX_PV(0) OMMX_PV(1) OMMX_PV(2) OMMX_PV(3) OMMX_PV(4) OMMX_PV(5) OMMX_PV(6) OMMX_PV(7)
+#undef OMMX_PV
+        }
+        lds_fence();
+    }
+
+    // ---- epilogue: o = (4*(acc - PVS) + PVZ) / l, lse = m + ln l -------------------------
+    float l_tot[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) l_tot[r] = wave_sum(l_run[r]);
+    const int jg = (j & 7) >> 1;
+    float pvz[4], pvs[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        pvz[r] = __shfl(accz[r], jg);          // column jg, rows 0..3 (kq 0)
+        pvs[r] = __shfl(accz[r], 4 + jg);
+    }
+    if (kq == jg) {
+        const int ch0 = 16 * (j & 7) + 8 * (j >> 3);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float* dst = a.al + b * a.al_b + (int64_t)(kvh * 4 + r) * a.al_h + (int64_t)sp * a.al_s;
+            const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+#pragma unroll
+            for (int y = 0; y < 8; ++y)
+                dst[ch0 + y] = (4.0f * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
+        }
+    }
+    if (lane < 4) {
+        float* dst = a.al + b * a.al_b + (int64_t)(kvh * 4 + lane) * a.al_h + (int64_t)sp * a.al_s;
+        const float lt = lane == 0 ? l_tot[0] : (lane == 1 ? l_tot[1] : (lane == 2 ? l_tot[2] : l_tot[3]));
+        const float mt = lane == 0 ? m_run[0] : (lane == 1 ? m_run[1] : (lane == 2 ? m_run[2] : m_run[3]));
+        dst[D] = lt > 0.0f ? (mt + log2f(lt)) * 0.6931471805599453f : -INFINITY;
+    }
+}
+
+}  // namespace
+
 // Returns 0 when launched, 1 when the shape is not covered by the tuned kernel.
-int launch_decode_fast(const DecodeArgs&, int, int, hipStream_t) { return 1; }
+int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
+    if (Dh != 128 || R != 4 || !(a.kout == 6 || a.kout == 0)) return 1;
+    const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
+    const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
+    const size_t shm = (size_t)waves * WAVE_LDS;
+    if (a.kout == 6)
+        hipLaunchKernelGGL(decode_splitkv_mfma_kernel<true>, grid, block, shm, st, a);
+    else
+        hipLaunchKernelGGL(decode_splitkv_mfma_kernel<false>, grid, block, shm, st, a);
+    return 0;
+}
 
 }  // namespace ommx
