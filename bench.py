@@ -6,8 +6,9 @@ operator (split-KV kernel + combine kernel) on one MI355X, Llama-3.1-8B attentio
                     [--no-cpu-baseline]
 
 One step = one decode call over one batch: the split-KV launch followed by the combine
-launch, operands resident in HBM, workspace preallocated, replayed from a HIP graph (eager
-launches if capture fails).  Prints ONE JSON line.  ``value`` is the p50 over the K timed
+launch, operands resident in HBM, workspace preallocated.  Steps are replayed from HIP
+graphs of 32 consecutive steps (the 32 layers of one model forward; eager launches if
+capture fails), so K is rounded up to a multiple of 32.  Prints ONE JSON line.  ``value`` is the p50 over the K timed
 steps at the headline context; ``roofline`` is the split-KV kernel alone (algorithmic bytes
 of the packed planes it must read over its average duration, against 8 TB/s);
 ``cpu_baseline`` is the CPU checker (dequantise-then-attend, torch on the host cores) on
@@ -28,6 +29,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+STAGE1_REP = 20
+LAYERS = 32                  # decode steps (layers) per graph replay
 H200_P50_US_64K = 563.0      # reference Triton kernel, H200 NVL, B=1 ctx 65536 (other hardware)
 
 
@@ -49,13 +52,14 @@ def _graph_or_eager(fn):
         return fn, "eager"
 
 
-def _time_steps(fn, steps, warmup):
-    """(wall ms per step over exactly `steps` steps, per-step GPU microseconds)."""
+def _time_steps(fn, calls, warmup, per_call=1):
+    """Time `calls` invocations of fn, each worth `per_call` steps.  Returns (wall ms per
+    step over the whole timed region, GPU microseconds per step of each invocation)."""
     import torch
     for _ in range(warmup):
         fn()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(steps)]
+          for _ in range(calls)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for a, b in ev:
@@ -63,8 +67,8 @@ def _time_steps(fn, steps, warmup):
         fn()
         b.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return wall_ms, [a.elapsed_time(b) * 1e3 for a, b in ev]
+    wall_ms = (time.perf_counter() - t0) * 1e3 / (calls * per_call)
+    return wall_ms, [a.elapsed_time(b) * 1e3 / per_call for a, b in ev]
 
 
 def _make_runner(case, splits=None):
@@ -128,8 +132,8 @@ def _cpu_reference(case, runs):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--ctx", type=int, default=65536)
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--no-ladder", action="store_true")
@@ -154,10 +158,21 @@ def main() -> int:
     def measure(ctx, steps, warmup):
         case = build_decode_case([ctx], seed=42, permute_tables=True, sparse_frac=0.005)
         step, stage1, o, lse, S = _make_runner(case, args.splits or None)
-        run, mode = _graph_or_eager(step)
-        wall_ms, us = _time_steps(run, steps, warmup)
-        run1, _ = _graph_or_eager(stage1)
-        _, us1 = _time_steps(run1, steps, warmup)
+        # one model forward runs this operator once per layer inside a single graph, so the
+        # steps are timed in graphs of LAYERS consecutive steps (steps is rounded up to that)
+        def layers():
+            for _ in range(LAYERS):
+                step()
+        run, mode = _graph_or_eager(layers)
+        calls = -(-steps // LAYERS)
+        wall_ms, us = _time_steps(run, calls, max(1, -(-warmup // LAYERS)), per_call=LAYERS)
+        # the kernel alone: REP launches back to back inside one graph, so that the event
+        # pair brackets kernel time and not the launch latency of a one-kernel graph
+        def stage1_rep():
+            for _ in range(STAGE1_REP):
+                stage1()
+        run1, _ = _graph_or_eager(stage1_rep)
+        _, us1 = _time_steps(run1, max(5, steps // STAGE1_REP), 2, per_call=STAGE1_REP)
         return dict(case=case, o=o, lse=lse, S=S, mode=mode, wall_ms=wall_ms, us=us, us1=us1)
 
     ladder = {}
@@ -165,7 +180,7 @@ def main() -> int:
         for ctx in (1024, 4096, 16384, 32768):
             if ctx == args.ctx:
                 continue
-            m = measure(ctx, max(20, args.steps // 4), max(3, args.warmup // 4))
+            m = measure(ctx, max(LAYERS, args.steps // 2), max(3, args.warmup // 4))
             ab = m["case"].algorithmic_bytes()
             p50 = statistics.median(m["us"])
             ladder[str(ctx)] = {"p50_us": round(p50, 2), "splits": m["S"], "bytes": ab,
@@ -202,7 +217,7 @@ def main() -> int:
     out = {
         "metric": "p50 decode-attn us/step/layer, 8B shape bs1",
         "value": round(p50, 3), "unit": "us/step/layer", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup,
+        "steps": -(-args.steps // LAYERS) * LAYERS, "warmup": -(-args.warmup // LAYERS) * LAYERS,
         "ms_per_step": round(m["wall_ms"], 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": round(p50 / H200_P50_US_64K, 5) if args.ctx == 65536 else None,
         "dtype": "u8 planes, bf16 q, f32 accumulate", "data": "synthetic",

@@ -31,12 +31,13 @@ def _cu_count(device: torch.device) -> int:
 
 
 def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256) -> int:
-    """Split count that gives every compute unit about two workgroups of at least four
-    32-token groups each; never more than 128 (the reference's ceiling,
-    ``paged_decode.py:340-353``)."""
-    groups = max(1, (int(max_seq_len) + 31) // 32)
-    want = max(1, (2 * int(n_cu)) // max(1, int(batch) * int(kv_heads)))
-    return int(max(1, min(128, want, max(1, groups // 4))))
+    """Split count that gives every compute unit two workgroups (a workgroup covers four kv
+    heads of one split) of at least four 64-token steps each; at most 256, the number of
+    partial states the combine kernel keeps on chip."""
+    steps = max(1, (int(max_seq_len) + 63) // 64)
+    wgs_per_split = max(1, int(batch) * max(1, int(kv_heads) // 4))
+    want = max(1, (2 * int(n_cu)) // wgs_per_split)
+    return int(max(1, min(256, want, max(1, steps // 4))))
 
 
 def make_attn_logits(batch: int, q_heads: int, num_kv_splits: int, head_dim: int, device) -> torch.Tensor:

@@ -47,8 +47,15 @@ extern "C" int ommx_decode_splitkv(
         set_error("ommx_decode_splitkv: packed_start_offset must be in [0,page_size), seg_group_base >= 0");
         return -1;
     }
-    if (k_outliers < 0 || k_outliers > 8 || num_splits < 1) {
-        set_error("ommx_decode_splitkv: k_outliers in [0,8], num_splits >= 1");
+    if (k_outliers < 0 || k_outliers > 8 || num_splits < 1 || num_splits > 256) {
+        set_error("ommx_decode_splitkv: k_outliers in [0,8], num_splits in [1,256]");
+        return -1;
+    }
+    if ((reinterpret_cast<uintptr_t>(k_base) | reinterpret_cast<uintptr_t>(v_main) |
+         reinterpret_cast<uintptr_t>(v_zp) | reinterpret_cast<uintptr_t>(k_obmp) |
+         reinterpret_cast<uintptr_t>(k_oval) | reinterpret_cast<uintptr_t>(k_zp) |
+         reinterpret_cast<uintptr_t>(k_ms) | reinterpret_cast<uintptr_t>(k_mc)) & 7) {
+        set_error("ommx_decode_splitkv: planes must be 8-byte aligned");
         return -1;
     }
     if (!q || !b_seq_len || !attn_logits || !req_to_token || !req_to_group) {
@@ -121,6 +128,15 @@ extern "C" int ommx_decode_combine(
     if (!attn_logits || !o || !lse || !b_seq_len) { set_error("ommx_decode_combine: null pointer"); return -1; }
     if (b_tail_len && (!k_tail || !v_tail || !q)) {
         set_error("ommx_decode_combine: tail lengths given without tail rows");
+        return -1;
+    }
+    if (b_tail_len && ((reinterpret_cast<uintptr_t>(k_tail) & 15) || kt_stride_b % 8 ||
+                       kt_stride_t % 8 || kt_stride_h % 8)) {
+        set_error("ommx_decode_combine: k_tail rows must be 16-byte aligned (strides multiples of 8)");
+        return -1;
+    }
+    if (num_splits > 256) {
+        set_error("ommx_decode_combine: at most 256 KV splits");
         return -1;
     }
     CombineArgs a{attn_logits, al_stride_b, al_stride_h, al_stride_s, q, q_stride_b, q_stride_h,

@@ -1,130 +1,163 @@
-// Split combine with the bf16 sink/recent tail folded in: one workgroup of 2*D threads per
+// Split combine with the bf16 sink/recent tail folded in: one workgroup of 8*D threads per
 // (request, q head).  Follows ommx_gpu_serve/attention/paged_decode.py:2366-2500: valid
 // splits are recomputed from the packed length with the stage-1 rounding; the tail is one
 // more softmax part computed here from k_tail/v_tail; o = sum w_i o_i / sum w_i,
 // lse = max + ln sum w_i; nothing attended gives o = 0, lse = -inf.
 //
-// The two halves of the workgroup work side by side: threads [0,D) reduce the split
-// partials for channel d, threads [D,2D) compute the tail (one row's q.k per thread with
-// 16-byte loads, then one channel's p.v per thread) and hand it over through LDS.
+// The kernel is latency bound (B*Hq small workgroups, a few KB each), so every global load
+// is issued before the first wait: thread (d, sg) owns channel d of the splits
+// sg, sg+8, ... and of the tail rows sg, sg+8, ...; for the tail logits the same threads
+// regroup as (row, 16 parts of the row).
 #include "ommx_decode_args.h"
 
 namespace ommx {
 
 template <int D>
-__global__ void __launch_bounds__(2 * D) combine_kernel(CombineArgs a) {
-    constexpr int MAXS = 256;            // split slots kept in LDS (host checks S <= MAXS)
+__global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
+    constexpr int NT = 8 * D;
+    constexpr int MAXS = 256;            // split slots (the launcher refuses more)
+    constexpr int ROWS = NT / 16;        // tail rows handled per chunk (64 at D=128)
+    constexpr int PER = ROWS / 8;        // tail rows per thread in the P.V step
+    constexpr int NSP = MAXS / 8;        // split partials per thread, upper bound
     __shared__ float s_q[D];
     __shared__ float s_lse[MAXS];
-    __shared__ float s_logit[D];         // tail logits / weights of the current chunk
-    __shared__ float s_tail[D + 2];      // tail part: o[D], l, m
+    __shared__ __attribute__((aligned(16))) float s_logit[ROWS];
+    __shared__ float s_acc[8][D];        // per-sg sums of the split part
+    __shared__ float s_tacc[8][D];       // per-sg sums of the tail part
+    __shared__ float s_w[8], s_tl[8], s_wmax[MAXS / 64];
     const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int d = tid % D, sg = tid / D;
     const int kvh = h / (a.Hq / a.Hkv);
     const int L = a.seq[b];
     const int tail = a.tail ? a.tail[b] : 0;
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
     const float* base = a.al + b * a.al_b + (int64_t)h * a.al_h;
-    const bool lower = tid < D;
 
-    if (lower) {
-        if (tail > 0) s_q[tid] = bf16_to_f32(a.q[b * a.q_sb + (int64_t)h * a.q_sh + tid]);
-        for (int s = tid; s < a.S; s += D) {
-            const bool valid = min(per * s + per, L) > per * s;
-            s_lse[s] = valid ? base[(int64_t)s * a.al_s + D] : -INFINITY;
-        }
+    // ---- all loads of the split part --------------------------------------------------
+    // (clamped addresses and a uniform trip count keep the loads free of per-lane branches,
+    // so they are all in flight together)
+    float pv[NSP];
+    const int n_i = (a.S + 7) >> 3;
+#pragma unroll
+    for (int i = 0; i < NSP; ++i) {
+        pv[i] = 0.0f;
+        if (i < n_i) pv[i] = base[(int64_t)min(sg + 8 * i, a.S - 1) * a.al_s + d];
     }
-    __syncthreads();
+    float my_lse = -INFINITY;
+    if (tid < MAXS) {
+        const bool valid = tid < a.S && min(per * tid + per, L) > per * tid;
+        if (valid) my_lse = base[(int64_t)tid * a.al_s + D];
+    }
+    const uint32_t q_raw = a.q[b * a.q_sb + (int64_t)h * a.q_sh + d];
 
+    if (tid < D) s_q[tid] = __uint_as_float(q_raw << 16);
+    if (tid < MAXS) {
+        s_lse[tid] = my_lse;
+        float wm = my_lse;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) wm = fmaxf(wm, __shfl_xor(wm, o));
+        if ((tid & 63) == 0) s_wmax[tid >> 6] = wm;
+    }
+
+    // ---- tail: chunks of ROWS rows (one chunk in practice: sink + recent <= 72 rows) ----
     float t_m = -INFINITY, t_l = 0.0f, t_acc = 0.0f;
-    float acc = 0.0f, wsum = 0.0f, g_max = -INFINITY;
-    if (lower) {
-        // ---- packed splits, channel d = tid -------------------------------------------
-        for (int s = 0; s < a.S; ++s) g_max = fmaxf(g_max, s_lse[s]);
-        const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
-#pragma unroll 8
-        for (int s = 0; s < a.S; ++s) {
+    for (int r0 = 0; r0 < tail; r0 += ROWS) {
+        const int nr = min(ROWS, tail - r0);
+        // loads first: 16 bytes of one K row, PER elements of V
+        const int row = tid >> 4, part = tid & 15;
+        const uint4 ku = *reinterpret_cast<const uint4*>(
+            a.kt + b * a.kt_b + (int64_t)(r0 + min(row, nr - 1)) * a.kt_t + (int64_t)kvh * a.kt_h +
+            (part * 8) % D);
+        uint32_t vv[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            vv[i] = a.vt[b * a.vt_b + (int64_t)(r0 + min(sg + 8 * i, nr - 1)) * a.vt_t +
+                         (int64_t)kvh * a.vt_h + d];
+        __syncthreads();                              // s_q ready (and previous chunk consumed)
+        float dot = 0.0f;
+        if (part * 8 < D) {
+            const uint32_t w[4] = {ku.x, ku.y, ku.z, ku.w};
+            const float* qq = s_q + part * 8;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                dot = fmaf(qq[2 * i], __uint_as_float(w[i] << 16), dot);
+                dot = fmaf(qq[2 * i + 1], __uint_as_float(w[i] & 0xFFFF0000u), dot);
+            }
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) dot += __shfl_xor(dot, o);
+        if (part == 0) s_logit[row] = row < nr ? apply_cap(dot * a.sm_scale, a.cap) : -INFINITY;
+        __syncthreads();
+        float mx = -INFINITY;                         // s_logit holds -inf past nr
+#pragma unroll
+        for (int i = 0; i < ROWS / 4; ++i) {
+            const float4 v4 = reinterpret_cast<const float4*>(s_logit)[i];
+            mx = fmaxf(mx, fmaxf(fmaxf(v4.x, v4.y), fmaxf(v4.z, v4.w)));
+        }
+        const float m_new = fmaxf(t_m, mx);
+        const float alpha = (t_m == -INFINITY) ? 0.0f : __expf(t_m - m_new);
+        t_l *= alpha;
+        t_acc *= alpha;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int r = sg + 8 * i;
+            if (r < nr) {
+                const float p = __expf(s_logit[r] - m_new);
+                t_l += p;
+                t_acc = fmaf(p, __uint_as_float(vv[i] << 16), t_acc);
+            }
+        }
+        t_m = m_new;
+    }
+    __syncthreads();                                  // s_lse ready
+
+    // ---- split part: weights from the lse column -----------------------------------------
+    float g_max = s_wmax[0];
+#pragma unroll
+    for (int w = 1; w < MAXS / 64; ++w) g_max = fmaxf(g_max, s_wmax[w]);
+    const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
+    float acc = 0.0f, wsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NSP; ++i) {
+        const int s = sg + 8 * i;
+        if (s < a.S) {
             const float ls = s_lse[s];
             if (ls != -INFINITY) {
                 const float w = __expf(ls - g_safe);
                 wsum += w;
-                acc = fmaf(w, base[(int64_t)s * a.al_s + tid], acc);
+                acc = fmaf(w, pv[i], acc);
             }
         }
     }
-    // ---- tail, chunks of D rows (uniform trip count for the whole workgroup) -----------
-    for (int r0 = 0; r0 < tail; r0 += D) {
-        const int nr = min(D, tail - r0);
-        if (!lower) {
-            const int r = tid - D;
-            float s = -INFINITY;
-            if (r < nr) {
-                const uint4* kr = reinterpret_cast<const uint4*>(
-                    a.kt + b * a.kt_b + (int64_t)(r0 + r) * a.kt_t + (int64_t)kvh * a.kt_h);
-                float dot = 0.0f;
-#pragma unroll
-                for (int i = 0; i < D / 8; ++i) {
-                    const uint4 u = kr[i];
-                    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        dot = fmaf(s_q[8 * i + 2 * j], __uint_as_float(w[j] << 16), dot);
-                        dot = fmaf(s_q[8 * i + 2 * j + 1], __uint_as_float(w[j] & 0xFFFF0000u), dot);
-                    }
-                }
-                s = apply_cap(dot * a.sm_scale, a.cap);
-            }
-            s_logit[r] = s;
-        }
-        __syncthreads();
-        if (!lower) {
-            const int d = tid - D;
-            float mx = -INFINITY;
-            for (int i = 0; i < nr; ++i) mx = fmaxf(mx, s_logit[i]);
-            const float m_new = fmaxf(t_m, mx);
-            const float alpha = (t_m == -INFINITY) ? 0.0f : __expf(t_m - m_new);
-            t_l *= alpha;
-            t_acc *= alpha;
-            const uint16_t* vr = a.vt + b * a.vt_b + (int64_t)r0 * a.vt_t + (int64_t)kvh * a.vt_h + d;
-#pragma unroll 8
-            for (int i = 0; i < nr; ++i) {
-                const float p = __expf(s_logit[i] - m_new);
-                t_l += p;
-                t_acc = fmaf(p, bf16_to_f32(vr[(int64_t)i * a.vt_t]), t_acc);
-            }
-            t_m = m_new;
-        }
-        __syncthreads();
-    }
-    if (!lower) {
-        const int d = tid - D;
-        s_tail[d] = t_l > 0.0f ? t_acc / t_l : 0.0f;
-        if (d == 0) { s_tail[D] = t_l; s_tail[D + 1] = t_m; }
-    }
+    s_acc[sg][d] = acc;
+    s_tacc[sg][d] = t_acc;
+    if (d == 0) { s_w[sg] = wsum; s_tl[sg] = t_l; }
     __syncthreads();
-    if (lower) {
-        const float tl = s_tail[D], tm = s_tail[D + 1];
-        const float tail_lse = tl > 0.0f ? tm + __logf(tl) : -INFINITY;
+    if (sg == 0) {
+        float A = 0.0f, W = 0.0f, TA = 0.0f, TL = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { A += s_acc[k][d]; W += s_w[k]; TA += s_tacc[k][d]; TL += s_tl[k]; }
+        const float tail_lse = TL > 0.0f ? t_m + __logf(TL) : -INFINITY;
         const float n_max = fmaxf(g_max, tail_lse);
         const float n_safe = (n_max == -INFINITY) ? 0.0f : n_max;
-        // re-base the split sums on the joint maximum, then add the tail part
         const float rs = (g_max == -INFINITY) ? 0.0f : __expf(g_max - n_safe);
-        wsum *= rs;
-        acc *= rs;
-        if (tl > 0.0f) {
+        W *= rs;
+        A *= rs;
+        if (TL > 0.0f) {
             const float w = __expf(tail_lse - n_safe);
-            wsum += w;
-            acc = fmaf(w, s_tail[tid], acc);
+            W += w;
+            A = fmaf(w, TA / TL, A);
         }
-        a.o[b * a.o_b + (int64_t)h * a.o_h + tid] = wsum > 0.0f ? acc / wsum : 0.0f;
-        if (tid == 0) a.lse[b * a.lse_b + h] = wsum > 0.0f ? n_max + __logf(wsum) : -INFINITY;
+        a.o[b * a.o_b + (int64_t)h * a.o_h + d] = W > 0.0f ? A / W : 0.0f;
+        if (d == 0) a.lse[b * a.lse_b + h] = W > 0.0f ? n_max + __logf(W) : -INFINITY;
     }
 }
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
     const dim3 grid(a.B, a.Hq);
-    if (D == 128) hipLaunchKernelGGL(combine_kernel<128>, grid, dim3(256), 0, st, a);
-    else if (D == 64) hipLaunchKernelGGL(combine_kernel<64>, grid, dim3(128), 0, st, a);
+    if (D == 128) hipLaunchKernelGGL(combine_kernel<128>, grid, dim3(1024), 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL(combine_kernel<64>, grid, dim3(512), 0, st, a);
     else return -1;
     return 0;
 }

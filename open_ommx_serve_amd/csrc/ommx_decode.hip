@@ -71,10 +71,26 @@ __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
     const f16x2 r = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
     return __builtin_bit_cast(uint32_t, r);
 }
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float readlane_f32(float v, int l) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+// maximum over the 64 lanes, result uniform: two quad steps, two mirror steps, four rows
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
+    v = fmaxf(v, dpp_f32<0xB1>(v));      // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_f32<0x4E>(v));      // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_f32<0x141>(v));     // row_half_mirror
+    v = fmaxf(v, dpp_f32<0x140>(v));     // row_mirror
+    return fmaxf(fmaxf(readlane_f32(v, 0), readlane_f32(v, 16)),
+                 fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
+}
+// low 32 bits of entry i of an int32 (sh=2) or int64 (sh=3) table
+__device__ __forceinline__ int table_lo(const void* t, int64_t i, int sh) {
+    return *reinterpret_cast<const int*>(static_cast<const char*>(t) + (i << sh));
 }
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -91,14 +107,14 @@ __device__ __forceinline__ uint32_t k_pair(uint32_t w, uint32_t magic) {
 }
 // V channel y of a merged dword (token a in the low 16 bits, token b in the high 16 bits).
 template <int Y>
-__device__ __forceinline__ uint32_t v_pair(uint32_t m) {
+__device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
     const uint32_t sh = (2 * Y >= 8) ? (m >> (2 * Y - 8 < 0 ? 0 : 2 * Y - 8))
                                      : (m << (8 - 2 * Y < 0 ? 0 : 8 - 2 * Y));
-    return (sh & 0x03000300u) | 0x3C003C00u;
+    return (sh & 0x03000300u) | one_f16x2;      // one v_and_or_b32 when the constant is a VGPR
 }
 
 template <bool OUTLIERS>
-__global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint8_t* const sm = smem_all + wave * WAVE_LDS;
@@ -111,9 +127,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
-    const int64_t tok_base = (int64_t)a.gbase * 32 + a.off;
     const float c_log2e = 1.4426950408889634f;
-    const float qk_scale = a.sm_scale * c_log2e;
 
     // ---- A operands: 4*q of head j%4 for this lane's 32-channel quarter ---------------
     // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
@@ -140,6 +154,9 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
         for (int i = lane; i < 32 * DT_ROW / 16; i += 64) dt[i] = u32x4{0, 0, 0, 0};
     }
 
+    uint32_t one2;                        // f16 (1.0, 1.0), pinned to a VGPR
+    asm volatile("v_mov_b32 %0, 0x3c003c00" : "=v"(one2));
+
     f32x4 acc[8];
     f32x4 accz = {0, 0, 0, 0};
 #pragma unroll
@@ -148,56 +165,79 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
 #pragma unroll
     for (int r = 0; r < 4; ++r) { m_run[r] = -INFINITY; l_run[r] = 0.0f; }
 
-    const int64_t row_bytes = (int64_t)Hkv * 32;          // k_base / v_main bytes per token row
+    // ---- addressing: 32-bit indices, 64-bit only in the final multiply-add ----------------
+    const uint32_t row_bytes = (uint32_t)Hkv * 32u;       // k_base / v_main bytes per token row
+    const int last = n_end - 1;
+    const int ps_sh = __ffs(a.ps) - 1, ps_mask = a.ps - 1;     // page_size is a power of two
+    const int tsh = a.i64 ? 3 : 2;                             // low dword of an int64 entry
+    const int tok_off = a.gbase * 32 + a.off;
+    const char* const rt_b = static_cast<const char*>(a.rt) + ((b * a.rt_s) << tsh);
+    const char* const rg_b = static_cast<const char*>(a.rg) + ((b * a.rg_s + a.gbase) << tsh);
+    const uint8_t* const kb_lane = a.k_base + kvh * 32 + 8 * kq;
+    const uint8_t* const vb_lane = a.v_main + kvh * 32 + 8 * kq;
+    const int8_t* const vs_head = a.v_scale + kvh * 4;
+    const uint16_t* const vz_head = a.v_zp + kvh * 4;
 
-    for (int n0 = n_begin; n0 < n_end; n0 += 64) {
-        // ---------------------------------------------------------------- addressing
-        const int last = n_end - 1;
-        int64_t rows[4];
+    // The loop is software-pipelined by hand: table entries are fetched two iterations
+    // ahead, plane data one iteration ahead, each into the registers its previous use
+    // has just released.
+    int rows[4], gsl[2];                  // physical token rows / group slots of the NEXT data loads
+    auto fetch_tables = [&](int n) {
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
-            const int64_t p = (int64_t)min(n0 + 16 * tb + j, last) + tok_base;
-            rows[tb] = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
+            const int p = min(n + 16 * tb + j, last) + tok_off;
+            const int pg = *reinterpret_cast<const int*>(rt_b + ((uint32_t)(p >> ps_sh) << tsh));
+            rows[tb] = (pg << ps_sh) + (p & ps_mask);
         }
-        const int my_tok = n0 + lane;
-        const bool tok_ok = my_tok < n_end;
-        int64_t my_row;
-        {
-            const int64_t p = (int64_t)min(my_tok, last) + tok_base;
-            my_row = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
-        }
-        int64_t gidx[2];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            const int gi = min(n0 / 32 + g, last / 32);
-            gidx[g] = (table_at(a.rg, b * a.rg_s + a.gbase + gi, a.i64) * Hkv + kvh) * D;
+            const int gi = min(n / 32 + g, last / 32);
+            gsl[g] = *reinterpret_cast<const int*>(rg_b + ((uint32_t)gi << tsh));
         }
-
-        // ---------------------------------------------------------------- loads
-        u32x2 kw[4], vw[4];
+    };
+    u32x2 kw[4], vw[4], vzp;
+    uint32_t vsc;
+    auto fetch_kv = [&]() {
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
-            kw[tb] = *reinterpret_cast<const u32x2*>(a.k_base + rows[tb] * row_bytes + kvh * 32 + 8 * kq);
-            vw[tb] = *reinterpret_cast<const u32x2*>(a.v_main + rows[tb] * row_bytes + kvh * 32 + 8 * kq);
+            const uint64_t ro = (uint64_t)(uint32_t)rows[tb] * row_bytes;
+            kw[tb] = *reinterpret_cast<const u32x2*>(kb_lane + ro);
+            vw[tb] = *reinterpret_cast<const u32x2*>(vb_lane + ro);
         }
-        const uint32_t vsc = *reinterpret_cast<const uint32_t*>(a.v_scale + (my_row * Hkv + kvh) * 4);
-        const u32x2 vzp = *reinterpret_cast<const u32x2*>(a.v_zp + (my_row * Hkv + kvh) * 4);
-
-        // channel pair (2*lane, 2*lane+1) parameters of both groups
-        uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
-        u32x2 g_bm[2], g_ov[2];
+        // this lane's own token (n + lane) is column j of token block kq
+        const uint32_t my_row = kq == 0 ? rows[0] : (kq == 1 ? rows[1] : (kq == 2 ? rows[2] : rows[3]));
+        vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
+        vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
+    };
+    // channel pair (2*lane, 2*lane+1) parameters of both groups
+    uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
+    u32x2 g_bm[2], g_ov[2];
+    auto fetch_params = [&]() {
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            g_sc[g] = *reinterpret_cast<const uint16_t*>(a.k_scale + gidx[g] + 2 * lane);
-            g_zp[g] = *reinterpret_cast<const uint32_t*>(a.k_zp + gidx[g] + 2 * lane);
+            const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);   // same for every lane
+            const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + (uint32_t)kvh) * D;
+            g_sc[g] = *reinterpret_cast<const uint16_t*>(a.k_scale + gidx + 2 * lane);
+            g_zp[g] = *reinterpret_cast<const uint32_t*>(a.k_zp + gidx + 2 * lane);
             if (OUTLIERS) {
-                g_ms[g] = *reinterpret_cast<const uint32_t*>(a.k_ms + gidx[g] + 2 * lane);
-                g_mc[g] = *reinterpret_cast<const uint32_t*>(a.k_mc + gidx[g] + 2 * lane);
-                g_bm[g] = *reinterpret_cast<const u32x2*>(a.k_obmp + (gidx[g] + 2 * lane) * 4);
-                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(a.k_oval + gidx[g] * 3) + (3 * lane) / 2;
+                g_ms[g] = *reinterpret_cast<const uint32_t*>(a.k_ms + gidx + 2 * lane);
+                g_mc[g] = *reinterpret_cast<const uint32_t*>(a.k_mc + gidx + 2 * lane);
+                g_bm[g] = *reinterpret_cast<const u32x2*>(a.k_obmp + gidx * 4 + 8 * lane);
+                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(a.k_oval + gidx * 3) + (3 * lane) / 2;
                 g_ov[g] = u32x2{ovp[0], ovp[1]};
             }
         }
+    };
+    if (n_begin < n_end) {
+        fetch_tables(n_begin);
+        fetch_kv();
+        fetch_params();
+        fetch_tables(n_begin + 64);
+    }
+
+    for (int n0 = n_begin; n0 < n_end; n0 += 64) {
+        const bool tok_ok = n0 + lane < n_end;
+        const bool more = n0 + 64 < n_end;
 
         // ---------------------------------------------------------------- stage to LDS
         // K code rows (for the outlier pass), transposed V dwords
@@ -264,6 +304,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) dbias = mfma_bf16(aq_pair[ks], bp[ks], dbias);
         }
+        if (more) fetch_kv();             // K/V registers are free again: start the next rows
 
         // ---------------------------------------------------------------- outliers
         // delta = (outlier - base)/4 goes through the tile twice: its f16 rounding first,
@@ -298,9 +339,8 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
                     uint32_t pp = 0;
 #pragma unroll
                     for (int sidx = 0; sidx < 6; ++sidx) {
-                        lo[sidx] = 0.0f;
-                        if (bm != 0) {
-                            const int pos = __ffs(bm) - 1;
+                        {
+                            const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32 (32 for an empty mask)
                             bm &= bm - 1;
                             pp |= static_cast<uint32_t>(pos) << (5 * sidx);
                             const float val = fmaf(lv[sidx], inv_ms, mc);
@@ -352,6 +392,11 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
             }
         }
 
+        if (more) {                        // group parameters and the tables after them
+            fetch_params();
+            fetch_tables(n0 + 128);
+        }
+
         // ---------------------------------------------------------------- softmax
         // bias of (group, head r): 0.25*ZP' - S1' ; columns 0..3 live in lanes 0..3 (kq 0)
         float logit[4];
@@ -373,8 +418,8 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
         for (int r = 0; r < 4; ++r) {
             const float mx = wave_max(logit[r]);
             const float m_new = fmaxf(m_run[r], mx);
-            alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : exp2f(m_run[r] - m_new);
-            p[r] = tok_ok ? exp2f(logit[r] - m_new) : 0.0f;
+            alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
+            p[r] = tok_ok ? __builtin_amdgcn_exp2f(logit[r] - m_new) : 0.0f;
             m_run[r] = m_new;
         }
         {
@@ -416,7 +461,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_mfma_kernel(DecodeArgs a) 
             const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], sel);
             const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], sel);
             const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], sel);
-#define OMMX_PV(Y) acc[Y] = mfma_f16(apv, u32x4{v_pair<Y>(mg0), v_pair<Y>(mg1), v_pair<Y>(mg2), v_pair<Y>(mg3)}, acc[Y]);
+#define OMMX_PV(Y) acc[Y] = mfma_f16(apv, u32x4{v_pair<Y>(mg0, one2), v_pair<Y>(mg1, one2), v_pair<Y>(mg2, one2), v_pair<Y>(mg3, one2)}, acc[Y]);
             OMMX_PV(0) OMMX_PV(1) OMMX_PV(2) OMMX_PV(3) OMMX_PV(4) OMMX_PV(5) OMMX_PV(6) OMMX_PV(7)
 #undef OMMX_PV
         }
