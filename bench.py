@@ -29,6 +29,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the split-KV kernel at the default workload (ctx 65536, 255
+# splits), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
+# (profiles/decode_ctx64k_hbm_traffic.txt); counters cannot be read from inside this script.
+TRAFFIC_BYTES_CTX64K = 80.33e6
 STAGE1_REP = 20
 LAYERS = 32                  # decode steps (layers) per graph replay
 H200_P50_US_64K = 563.0      # reference Triton kernel, H200 NVL, B=1 ctx 65536 (other hardware)
@@ -138,6 +142,9 @@ def main() -> int:
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--no-ladder", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy kernel (3 times), the known-size "
+                         "reference that scales the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the decode operator has no collective and every box "
@@ -174,6 +181,14 @@ def main() -> int:
         run1, _ = _graph_or_eager(stage1_rep)
         _, us1 = _time_steps(run1, max(5, steps // STAGE1_REP), 2, per_call=STAGE1_REP)
         return dict(case=case, o=o, lse=lse, S=S, mode=mode, wall_ms=wall_ms, us=us, us1=us1)
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     ladder = {}
     if not args.no_ladder:
@@ -232,7 +247,8 @@ def main() -> int:
                    "(reference Triton kernel on H200 NVL, page 32; other hardware)"},
         "roofline": {"bound": "hbm", "kernel": "decode_splitkv", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "bytes_per_launch": packed_bytes,
+                     "traffic": TRAFFIC_BYTES_CTX64K if (args.ctx == 65536 and not args.splits) else None,
+                     "bytes_per_launch": packed_bytes,
                      "avg_kernel_us": round(k1, 3)},
         "cpu_baseline": cpu,
         "parity_after_timing": parity,

@@ -92,7 +92,9 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 o (normalised) in [0,D) and lse at D; an empty split writes o=0,
  *                 lse=-inf (paged_decode.py:2262-2284)
  * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
- * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in 1..8; D = 128 or 64.
+ * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64;
+ * num_splits <= 256; planes 8-byte aligned.  head_dim 128 with r = 4 and 6 (or 0) outliers
+ * runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
@@ -109,13 +111,35 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
                         int packed_start_offset, int seg_group_base, void* stream);
 
 /*
+ * The same operator through the plain fp32 kernel only; identical arguments.  It has no
+ * counterpart in the reference: it exists so that tests can cross-check the two device
+ * kernels against each other and against the CPU oracle.
+ */
+int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+                            const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+                            const uint16_t* k_ms, const uint16_t* k_mc,
+                            const uint8_t* k_obmp, const uint8_t* k_oval,
+                            const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+                            const void* req_to_token, int64_t rt_stride,
+                            const void* req_to_group, int64_t rg_stride, int table_i64,
+                            const int32_t* b_seq_len,
+                            float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
+                            int64_t al_stride_s,
+                            int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
+                            int num_splits, float sm_scale, float logit_cap,
+                            int packed_start_offset, int seg_group_base, void* stream);
+
+/*
  * Split combine with the bf16 sink/recent tail folded in (stage 2).
  *   k_tail,v_tail bf16 [B,Tmax,Hkv,D] with strides t_stride_b/t/h (K and V alike)
  *   b_tail_len    int32[B] valid tail rows (0 allowed)
  *   o             f32 [B,Hq,D] strides o_stride_b/h;  lse f32 [B,Hq] stride lse_stride_b
  * Valid splits are recomputed from b_seq_len with the stage-1 rounding
  * (paged_decode.py:2407-2410); nothing attended gives o = 0, lse = -inf.
- * emit_mode 0: merged final (splits + tail).  emit_mode 1: segment partial (no tail).
+ * b_tail_len == NULL (then k_tail, v_tail, q may be NULL too) combines the splits alone:
+ * the un-merged state of a group-range segment (paged_decode.py:2892-2902).
+ * k_tail rows must be 16-byte aligned (base pointer and strides multiples of 8 elements);
+ * num_splits <= 256.
  */
 int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,

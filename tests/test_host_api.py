@@ -1,0 +1,182 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every entry point
+the header declares, the decision tables behave, argument validation raises the
+reference's exception types before anything is launched, and the operators refuse to run
+without a GPU instead of falling back."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import oracle.ommx_oracle as O
+from open_ommx_serve_amd.attention import _hip, kv_window
+from open_ommx_serve_amd.attention import pack as hip_pack
+from open_ommx_serve_amd.attention.paged_decode import (auto_num_kv_splits,
+                                                        ommx_paged_decode_attention_canonical)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "ommx_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ommx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _hip.load()
+    names = _declared_functions()
+    assert {"ommx_store_pack", "ommx_decode_splitkv", "ommx_decode_combine",
+            "ommx_store_default_table", "ommx_abi_version", "ommx_last_error"} <= set(names)
+    raw = ctypes.CDLL(_hip.lib_path())
+    for n in names:
+        assert getattr(raw, n) is not None, n
+    assert set(_hip.exported_symbols()) == set(names)
+    assert lib.ommx_abi_version() == 1
+
+
+def test_default_decision_table_is_the_exact_arithmetic_one():
+    lib = _hip.load()
+    t = torch.zeros(_hip.STORE_TABLE_FLOATS)
+    lib.ommx_store_default_table(t.data_ptr())
+    for kb in (100, 126, 127, 128, 140):
+        x = t[kb].double().item()
+        assert x > 2.0 ** (kb - 127 + 0.5) > torch.nextafter(t[kb], torch.tensor(0.0)).double().item()
+    want = [(1e-8 * 0.5) ** 0.5, 0.5 ** 0.5, 1.5 ** 0.5, 3 ** 0.5, 6 ** 0.5, 12 ** 0.5, 24 ** 0.5]
+    for j, w in enumerate(want, start=1):
+        assert abs(t[256 + j].item() - w) / w < 1e-6 and t[256 + j].double().item() > w
+
+
+def test_measured_decision_table_reproduces_the_torch_rounding():
+    """Thresholds measured from torch-CPU must give, for every float near every rounding
+    point, the exponent / FP4 level the oracle's own expressions give."""
+    t = hip_pack.measure_store_table()
+    for kb in range(95, 150):
+        c = t[kb:kb + 1]
+        win = (c.view(torch.int32) + torch.arange(-40, 41, dtype=torch.int32)).view(torch.float32)
+        got = (kb - 127) + (win >= c).to(torch.float32)
+        assert torch.equal(got, O.pow2_exponent(win)), kb
+    for j in range(2, 8):
+        c = t[256 + j:256 + j + 1]
+        win = (c.view(torch.int32) + torch.arange(-40, 41, dtype=torch.int32)).view(torch.float32)
+        idx = sum((win >= t[256 + k]).to(torch.int64) for k in range(1, 8))
+        assert torch.equal(idx, O.fp4_encode(win).to(torch.int64) & 7), j
+
+
+def test_window_arithmetic_matches_the_oracle_closed_forms():
+    w = kv_window.WindowSpec()
+    for n in list(range(0, 300)) + [1024, 4096, 32768, 65536]:
+        assert w.boundary(n) == O.packed_boundary(n)
+        assert w.tail_indices(n) == O.tail_indices(n)
+        assert w.packed_len(n) == max(0, O.packed_boundary(n) - 8)
+        assert w.num_groups(n) * 32 == w.packed_len(n)
+    assert (w.packed_len(1024), w.packed_len(4096), w.packed_len(65536)) == (960, 4032, 65472)
+    assert w.newly_completed_groups(71, 72) == 1 and w.newly_completed_groups(72, 103) == 0
+    assert w.max_tail_len() == 72 and w.packed_start_offset() == 8 and w.sink_page_shift() == 0
+    w64 = kv_window.WindowSpec(group_tokens=64)
+    assert w64.boundary(200) == 8 + 128
+    with pytest.raises(ValueError):
+        kv_window.packed_boundary(10, 8, 32, 0)
+
+
+def test_split_heuristic_bounds():
+    assert auto_num_kv_splits(960, 1, 8, 256) >= 1
+    assert auto_num_kv_splits(65472, 1, 8, 256) == 255
+    assert auto_num_kv_splits(65472, 32, 8, 256) == 8
+    assert 1 <= auto_num_kv_splits(1, 1, 1, 256) <= 256
+
+
+def test_pack_argument_errors_match_the_reference():
+    K = torch.zeros(64, 2, 64, dtype=torch.bfloat16)
+    good = dict(outliers_per_vector=6, outlier_select="signed", outlier_repr="bitmap",
+                k_format="i2f4", use_pow2=True, page_size=16)
+    P = hip_pack.ommx_pack_kv_canonical_block
+    with pytest.raises(ValueError):
+        P(K, K[:32], **good)
+    with pytest.raises(ValueError):
+        P(K[:48], K[:48], **good)
+    with pytest.raises(ValueError):
+        P(K, K, **{**good, "outlier_repr": "bogus"})
+    with pytest.raises(ValueError):
+        P(K, K, **{**good, "k_format": "i4"})
+    with pytest.raises(ValueError):
+        P(K, K, **{**good, "group_tokens": 48})
+    with pytest.raises(ValueError):
+        P(K, K, **{**good, "outliers_per_vector": 33})
+    with pytest.raises(ValueError):
+        P(K, K, **{**good, "v_format": "fp8"})
+    with pytest.raises(NotImplementedError):
+        P(K, K, **{**good, "outlier_repr": "relidx7"})
+    with pytest.raises(NotImplementedError):
+        P(K, K, **{**good, "use_pow2": False})
+    with pytest.raises(NotImplementedError):
+        P(K, K, **{**good, "group_tokens": 64})
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            P(K, K, **good)
+
+
+def test_store_error_bits_become_reference_exceptions():
+    hip_pack.raise_for_store_errors(0)
+    with pytest.raises(ValueError):
+        hip_pack.raise_for_store_errors(_hip.ERR_NONFINITE_V)
+    with pytest.raises(IndexError):
+        hip_pack.raise_for_store_errors(_hip.ERR_UNDERFILLED | _hip.ERR_NONFINITE_K)
+    with pytest.raises(ValueError):
+        hip_pack.raise_for_store_errors(_hip.ERR_NONFINITE_K)
+
+
+def _cpu_decode_args(Hq=4, Hkv=2, D=64, T=64):
+    planes = O.pack_kv(torch.randn(T, Hkv, D).to(torch.bfloat16), torch.randn(T, Hkv, D).to(torch.bfloat16))
+    q = torch.zeros(1, Hq, D, dtype=torch.bfloat16)
+    tail = torch.zeros(1, 8, Hkv, D, dtype=torch.bfloat16)
+    o = torch.zeros(1, Hq, D)
+    lse = torch.zeros(1, Hq)
+    args = [q, planes["k_base"], planes["k_scale"], planes["k_zp"], None, planes["k_oval"],
+            planes["v_main"], planes["v_scale"], planes["v_zp"], tail, tail,
+            torch.tensor([8], dtype=torch.int32), o, lse, planes["req_to_token"],
+            planes["req_to_group"], torch.tensor([T], dtype=torch.int32)]
+    kw = dict(sm_scale=0.125, page_size=16, k_outliers_per_vector=6, bitmap_read=True,
+              k_obmp=planes["k_obmp"], k_fp4_mapscale=planes["k_fp4_mapscale"],
+              k_fp4_mapcenter=planes["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
+              max_seq_len=T, max_tail_len=8)
+    return args, kw
+
+
+def test_decode_argument_errors_precede_any_launch():
+    args, kw = _cpu_decode_args()
+    D = ommx_paged_decode_attention_canonical
+    with pytest.raises(ValueError, match="packed_start_offset"):
+        D(*args, **{**kw, "packed_start_offset": 16})
+    with pytest.raises(ValueError, match="seg_group_base"):
+        D(*args, **{**kw, "seg_group_base": -1})
+    with pytest.raises(ValueError, match="k_obmp"):
+        D(*args, **{**kw, "k_obmp": None})
+    with pytest.raises(ValueError, match="mutually exclusive"):
+        D(*args, **{**kw, "combinadic_read": True})
+    with pytest.raises(ValueError, match="k_fp4_mapscale"):
+        D(*args, **{**kw, "k_fp4_mapscale": None})
+    with pytest.raises(ValueError, match="k_format"):
+        D(*args, **{**kw, "k_format": "i8"})
+    with pytest.raises(ValueError, match="k_oval"):
+        bad = list(args); bad[5] = None
+        D(*bad, **kw)
+    with pytest.raises(NotImplementedError, match="integer multiple"):
+        bad = list(args); bad[0] = args[0][:, :3]
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="contiguous"):
+        bad = list(args); bad[6] = args[6][:, ::2]
+        D(*bad, **{**kw, "page_size": 8})
+    with pytest.raises(NotImplementedError, match="serving recipe"):
+        D(*args, **{**kw, "kv_outlier_map": False, "k_fp4_mapscale": None})
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            D(*args, **kw)
+
+
+def test_missing_library_is_a_loud_error(monkeypatch):
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "_LIB_PATH", "/nonexistent/libommx_hip.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _hip.load()
