@@ -13,15 +13,21 @@
 //            exponent field already holds the group's power-of-two scale;
 //            A = 4*q (bf16).  sum A*B = sum q*code*s + 4*sum q*s, the second term and
 //            sum q*zp come out of one small "bias" MFMA per 64 tokens.
-//   outliers a per-group tile [32 tokens][128 channels] of (outlier - base)/4 in f16,
-//            scattered by a channel-major pass (one lane = two channels), consumed as the
-//            B operand of an f16 MFMA against A = 4*q (f16).
+//   outliers a channel-major pass (one lane = two channels) clears the base code of every
+//            outlier position in the staged K rows (LDS and), so that the base term of
+//            such an element is exactly covered by the bias terms, and scatters (outlier - zp)/4 as f16
+//            into a per-group tile [32 tokens][128 channels] that is consumed as the B
+//            operand of an f16 MFMA against A = 4*q (f16).  Deltas too large for one f16
+//            (|delta/4| >= 4, rare) add their rounding residual times q straight onto the
+//            logits through LDS float atomics.
 //   P.V      B = (1 + code/4) f16 for 8 tokens of one channel (V rows are transposed
 //            through LDS at dword granularity), A = p * 2^e_v (f16, exact scaling);
 //            sum_t p*vs and sum_t p*vz come from one extra MFMA per 32 tokens.
 // MFMA row groups are used as selectors: rows 4x..4x+3 carry the 4 q heads for token
 // block x (QK) or for V channel group x (P.V); a lane keeps the row group that matches
 // its column.
+#include <type_traits>
+
 #include "ommx_decode_args.h"
 
 namespace ommx {
@@ -47,7 +53,9 @@ constexpr int OFF_VS = 5632;       // [4 channel groups][64 tokens] f16 2^e_v
 constexpr int OFF_VZ = 6144;       // [4 channel groups][64 tokens] f16 v zero points
 constexpr int OFF_DT = 6656;       // [32 tokens][DT_ROW B] f16 outlier deltas of one group
 constexpr int DT_ROW = 272;
-constexpr int WAVE_LDS = OFF_DT + 32 * DT_ROW;      // 15360
+constexpr float BIG_DELTA = 8.0f;   // |outlier delta|/4 from which one f16 is not enough
+constexpr int OFF_LC = OFF_DT + 32 * DT_ROW;        // [64 tokens][4 heads] f32 logit corrections
+constexpr int WAVE_LDS = OFF_LC + 1024;             // 16384
 
 __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
@@ -71,22 +79,48 @@ __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
     const f16x2 r = __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b);
     return __builtin_bit_cast(uint32_t, r);
 }
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-        0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
 __device__ __forceinline__ float readlane_f32(float v, int l) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
 }
-// maximum over the 64 lanes, result uniform: two quad steps, two mirror steps, four rows
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_f32<0xB1>(v));      // quad_perm [1,0,3,2]
-    v = fmaxf(v, dpp_f32<0x4E>(v));      // quad_perm [2,3,0,1]
-    v = fmaxf(v, dpp_f32<0x141>(v));     // row_half_mirror
-    v = fmaxf(v, dpp_f32<0x140>(v));     // row_mirror
-    return fmaxf(fmaxf(readlane_f32(v, 0), readlane_f32(v, 16)),
-                 fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
+// Maxima of four values over the 64 lanes (results uniform).  The four reductions are
+// interleaved so that every DPP instruction is at least three instructions away from the
+// write of its source, which covers the two wait states the DPP read needs; steps: two
+// quad permutes, half-row mirror, row mirror, then the row broadcasts that leave the
+// maximum of all rows in lane 63.
+__device__ __forceinline__ void wave_max4(float (&v)[4]) {
+    float a = v[0], b = v[1], c = v[2], d = v[3];
+    asm volatile(
+        "s_nop 1\n"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_max_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_max_f32_dpp %2, %2, %2 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_max_f32_dpp %3, %3, %3 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_max_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_max_f32_dpp %2, %2, %2 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_max_f32_dpp %3, %3, %3 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "s_nop 1\n"
+        : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    v[0] = readlane_f32(a, 63);
+    v[1] = readlane_f32(b, 63);
+    v[2] = readlane_f32(c, 63);
+    v[3] = readlane_f32(d, 63);
 }
 // low 32 bits of entry i of an int32 (sh=2) or int64 (sh=3) table
 __device__ __forceinline__ int table_lo(const void* t, int64_t i, int sh) {
@@ -128,26 +162,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
     const float c_log2e = 1.4426950408889634f;
-
-    // ---- A operands: 4*q of head j%4 for this lane's 32-channel quarter ---------------
-    // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
-    // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
-    u32x4 aq_pair[4], aq_nat[4];
-    {
-        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(kvh * 4 + (j & 3)) * a.q_sh + 32 * kq;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
-                const float lo = 4.0f * bf16_to_f32(qh[cl]), hi = 4.0f * bf16_to_f32(qh[cl + 8]);
-                aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
-                const float n0 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr]);
-                const float n1 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr + 1]);
-                aq_nat[ks][rr] = pack_f16x2(n0, n1);
-            }
-        }
-    }
 
     if (OUTLIERS) {   // the outlier tile starts out all zero; readers clear what they consume
         u32x4* dt = reinterpret_cast<u32x4*>(sm + OFF_DT);
@@ -235,6 +249,38 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         fetch_tables(n_begin + 64);
     }
 
+    // ---- A operands: 4*q of head j%4 for this lane's 32-channel quarter ---------------
+    // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
+    // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
+    u32x4 aq_pair[4], aq_nat[4];
+    {
+        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(kvh * 4 + (j & 3)) * a.q_sh + 32 * kq;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
+                const float lo = 4.0f * bf16_to_f32(qh[cl]), hi = 4.0f * bf16_to_f32(qh[cl + 8]);
+                aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
+                const float n0 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr]);
+                const float n1 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr + 1]);
+                aq_nat[ks][rr] = pack_f16x2(n0, n1);
+            }
+        }
+    }
+    // the same 4*q for the channel pass: heads 0..3 of channels 2*lane, 2*lane+1 (fp32)
+    float q4[2][4];
+    if (OUTLIERS) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(
+                a.q + b * a.q_sb + (int64_t)(kvh * 4 + r) * a.q_sh + 2 * lane);
+            q4[0][r] = 4.0f * __uint_as_float(w << 16);
+            q4[1][r] = 4.0f * __uint_as_float(w & 0xFFFF0000u);
+        }
+    }
+
+
     for (int n0 = n_begin; n0 < n_end; n0 += 64) {
         const bool tok_ok = n0 + lane < n_end;
         const bool more = n0 + 64 < n_end;
@@ -280,21 +326,98 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 }
             }
         }
+        if (OUTLIERS)
+            *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * lane) = u32x4{0, 0, 0, 0};
         lds_fence();
+        if (more) fetch_kv();             // K/V registers are staged: start the next rows
 
-        // ---------------------------------------------------------------- QK base
+        // ---------------------------------------------------------------- QK
+        // per group: channel pass (clear outlier codes, scatter deltas), then the token
+        // blocks of the group take tile and base terms in one accumulation chain
         f32x4 dq[4];
 #pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-            const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + (tb >> 1) * 256 + kq * 64);
+        for (int g = 0; g < 2; ++g) {
+            if (OUTLIERS) {
+                // RES = false: the walk every group takes.  RES = true: a second walk that only
+                // adds f16 rounding residuals of large deltas onto the logits.
+                float dl_max = 0.0f;
+                auto walk = [&](auto RES) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int c = 2 * lane + u;
+                        const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
+                        const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
+                        const float mc = __uint_as_float(u ? (g_mc[g] & 0xFFFF0000u) : (g_mc[g] << 16));
+                        // tile value (outlier - zp)/4 = level * a1 + b1
+                        const float a1 = 0.25f * __builtin_amdgcn_rcpf(ms);
+                        const float b1 = 0.25f * (mc - zp);
+                        uint32_t bm = g_bm[g][u];
+                        // 6 nibbles of this channel: bytes 3c..3c+2 of the block
+                        const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
+                        const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
+                        const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                        const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
+                        const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
+                        const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
+                        // code dword of channel c in a K row, and the mask that clears its 2 bits
+                        uint32_t* kt = reinterpret_cast<uint32_t*>(sm + OFF_KT + g * 1024) + (c >> 4);
+                        const uint32_t keep = ~(3u << (2 * (c & 15)));
+                        uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
+                        float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 128;
+#pragma unroll
+                        for (int sidx = 0; sidx < 6; ++sidx) {
+                            const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32
+                            bm &= bm - 1;
+                            const float dl = fmaf(lv[sidx], a1, b1);
+                            const _Float16 hi = static_cast<_Float16>(dl);
+                            if constexpr (!decltype(RES)::value) {
+                                dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
+                                __hip_atomic_fetch_and(kt + pos * 8, keep, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
+                                dl_max = fmaxf(dl_max, fabsf(dl));
+                            } else {
+                                if (fabsf(dl) >= BIG_DELTA) {
+                                    const float lo = dl - static_cast<float>(hi);
+#pragma unroll
+                                    for (int r = 0; r < 4; ++r)
+                                        __hip_atomic_fetch_add(lc + pos * 4 + r, lo * q4[u][r], __ATOMIC_RELAXED,
+                                                               __HIP_MEMORY_SCOPE_WAVEFRONT);
+                                }
+                            }
+                        }
+                    }
+                };
+                walk(std::false_type{});
+                // One f16 carries 11 bits: below |delta/4| = 8 its rounding error is at most
+                // 2^-9 (8e-3 in K units, a relative logit error far inside the tolerance).
+                // Groups holding a larger delta (rare) take the residual walk.
+                if (__any(dl_max >= BIG_DELTA)) walk(std::true_type{});
+                lds_fence();
+            }
+            const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + g * 256 + kq * 64);
             const u32x4 m0 = mg[0], m1 = mg[1], m2 = mg[2], m3 = mg[3];
-            const uint32_t w0 = kw[tb][0], w1 = kw[tb][1];
-            f32x4 d = {0, 0, 0, 0};
-            d = mfma_bf16(aq_pair[0], u32x4{k_pair<0>(w0, m0[0]), k_pair<1>(w0, m0[1]), k_pair<2>(w0, m0[2]), k_pair<3>(w0, m0[3])}, d);
-            d = mfma_bf16(aq_pair[1], u32x4{k_pair<4>(w0, m1[0]), k_pair<5>(w0, m1[1]), k_pair<6>(w0, m1[2]), k_pair<7>(w0, m1[3])}, d);
-            d = mfma_bf16(aq_pair[2], u32x4{k_pair<0>(w1, m2[0]), k_pair<1>(w1, m2[1]), k_pair<2>(w1, m2[2]), k_pair<3>(w1, m2[3])}, d);
-            d = mfma_bf16(aq_pair[3], u32x4{k_pair<4>(w1, m3[0]), k_pair<5>(w1, m3[1]), k_pair<6>(w1, m3[2]), k_pair<7>(w1, m3[3])}, d);
-            dq[tb] = d;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const int tb = 2 * g + t2;
+                f32x4 d = {0, 0, 0, 0};
+                if (OUTLIERS) {   // tile rows of this token block: read, clear, accumulate
+                    u32x4* row = reinterpret_cast<u32x4*>(sm + OFF_DT + (16 * t2 + j) * DT_ROW + 64 * kq);
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+                        const u32x4 bt = row[ks];
+                        row[ks] = u32x4{0, 0, 0, 0};
+                        d = mfma_f16(aq_nat[ks], bt, d);
+                    }
+                }
+                const u32x2 kw2 = *reinterpret_cast<const u32x2*>(sm + OFF_KT + (16 * tb + j) * 32 + 8 * kq);
+                const uint32_t w0 = kw2[0], w1 = kw2[1];
+                d = mfma_bf16(aq_pair[0], u32x4{k_pair<0>(w0, m0[0]), k_pair<1>(w0, m0[1]), k_pair<2>(w0, m0[2]), k_pair<3>(w0, m0[3])}, d);
+                d = mfma_bf16(aq_pair[1], u32x4{k_pair<4>(w0, m1[0]), k_pair<5>(w0, m1[1]), k_pair<6>(w0, m1[2]), k_pair<7>(w0, m1[3])}, d);
+                d = mfma_bf16(aq_pair[2], u32x4{k_pair<0>(w1, m2[0]), k_pair<1>(w1, m2[1]), k_pair<2>(w1, m2[2]), k_pair<3>(w1, m2[3])}, d);
+                d = mfma_bf16(aq_pair[3], u32x4{k_pair<4>(w1, m3[0]), k_pair<5>(w1, m3[1]), k_pair<6>(w1, m3[2]), k_pair<7>(w1, m3[3])}, d);
+                dq[tb] = d;
+            }
+            if (OUTLIERS) lds_fence();        // the tile is zero again before the next scatter
         }
         // bias columns: 0 zp(g0) 1 zp(g1) 2 2^e(g0) 3 2^e(g1); other columns repeat them
         f32x4 dbias = {0, 0, 0, 0};
@@ -303,98 +426,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             const u32x4* bp = reinterpret_cast<const u32x4*>(sm + src);
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) dbias = mfma_bf16(aq_pair[ks], bp[ks], dbias);
-        }
-        if (more) fetch_kv();             // K/V registers are free again: start the next rows
-
-        // ---------------------------------------------------------------- outliers
-        // delta = (outlier - base)/4 goes through the tile twice: its f16 rounding first,
-        // then the f16 rounding of what the first pass left over, so that the pair carries
-        // ~22 significant bits (a single f16 is not enough for outliers of magnitude 100+).
-        if (OUTLIERS) {
-#pragma unroll
-            for (int g = 0; g < 2; ++g) {
-                uint32_t lo_pk[2][3];     // residuals, two f16 per register
-                uint32_t pos_pk[2];       // six 5-bit token positions per channel
-                bool big = false;         // some |delta/4| of this lane needs the second term
-                // channel pass: lane owns channels 2*lane, 2*lane+1 of group g
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int c = 2 * lane + u;
-                    const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
-                    const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-                    const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
-                    const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
-                    const float mc = __uint_as_float(u ? (g_mc[g] & 0xFFFF0000u) : (g_mc[g] << 16));
-                    const float inv_ms = __builtin_amdgcn_rcpf(ms);
-                    uint32_t bm = g_bm[g][u];
-                    // 6 nibbles of this channel: bytes 3c..3c+2 of the block
-                    const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
-                    const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
-                    const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
-                    const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
-                    const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
-                    const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
-                    const uint8_t* kt = sm + OFF_KT + g * 1024 + (c >> 2);
-                    uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
-                    float lo[6];
-                    uint32_t pp = 0;
-#pragma unroll
-                    for (int sidx = 0; sidx < 6; ++sidx) {
-                        {
-                            const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32 (32 for an empty mask)
-                            bm &= bm - 1;
-                            pp |= static_cast<uint32_t>(pos) << (5 * sidx);
-                            const float val = fmaf(lv[sidx], inv_ms, mc);
-                            const uint32_t code = (static_cast<uint32_t>(kt[pos * 32]) >> (2 * (c & 3))) & 3u;
-                            const float base = fmaf(static_cast<float>(code), s, zp);
-                            const float dl = (val - base) * 0.25f;
-                            const _Float16 hi = static_cast<_Float16>(dl);
-                            lo[sidx] = dl - static_cast<float>(hi);
-                            big = big || fabsf(dl) >= 4.0f;
-                            dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
-                        }
-                    }
-                    pos_pk[u] = pp;
-                    lo_pk[u][0] = pack_f16x2(lo[0], lo[1]);
-                    lo_pk[u][1] = pack_f16x2(lo[2], lo[3]);
-                    lo_pk[u][2] = pack_f16x2(lo[4], lo[5]);
-                }
-                // Below |delta| = 16 the f16 rounding error of the first term (at most 2^-12
-                // relative, i.e. < 4e-3 in K units) is far inside the tolerance, so the second
-                // term is only scattered when some lane of the wave holds a larger delta.
-                const int passes = __any(big) ? 2 : 1;
-                for (int pass = 0; pass < passes; ++pass) {
-                    if (pass == 1) {
-                        // the tile is all zero again: scatter the residuals to the same places
-#pragma unroll
-                        for (int u = 0; u < 2; ++u) {
-                            uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + 2 * lane + u;
-#pragma unroll
-                            for (int sidx = 0; sidx < 6; ++sidx) {
-                                const int pos = (pos_pk[u] >> (5 * sidx)) & 31;
-                                const uint32_t w = lo_pk[u][sidx >> 1];
-                                const uint16_t hw = static_cast<uint16_t>((sidx & 1) ? (w >> 16) : (w & 0xFFFFu));
-                                if (hw != 0) dt[pos * (DT_ROW / 2)] = hw;
-                            }
-                        }
-                    }
-                    lds_fence();
-                    // token blocks 2g, 2g+1 read their rows of the tile and clear them
-#pragma unroll
-                    for (int t2 = 0; t2 < 2; ++t2) {
-                        u32x4* row = reinterpret_cast<u32x4*>(sm + OFF_DT + (16 * t2 + j) * DT_ROW + 64 * kq);
-                        f32x4 d = dq[2 * g + t2];
-#pragma unroll
-                        for (int ks = 0; ks < 4; ++ks) {
-                            const u32x4 bt = row[ks];
-                            row[ks] = u32x4{0, 0, 0, 0};
-                            d = mfma_f16(aq_nat[ks], bt, d);
-                        }
-                        dq[2 * g + t2] = d;
-                    }
-                    lds_fence();
-                }
-            }
         }
 
         if (more) {                        // group parameters and the tables after them
@@ -408,21 +439,23 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         {
             const f32x4 dsel = kq == 0 ? dq[0] : (kq == 1 ? dq[1] : (kq == 2 ? dq[2] : dq[3]));
             const int gsel = lane >> 5;
+            f32x4 corr = {0, 0, 0, 0};
+            if (OUTLIERS) corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * lane);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float zpv = __shfl(dbias[r], gsel);          // column gsel, rows 0..3
                 const float s1v = __shfl(dbias[r], 2 + gsel);
-                const float raw = dsel[r] + (0.25f * zpv - s1v);
+                const float raw = dsel[r] + corr[r] + (0.25f * zpv - s1v);
                 float x = raw * a.sm_scale;
                 x = apply_cap(x, a.cap) * c_log2e;
                 logit[r] = tok_ok ? x : -INFINITY;
             }
         }
-        float alpha[4], p[4];
+        float alpha[4], p[4], mxs[4] = {logit[0], logit[1], logit[2], logit[3]};
+        wave_max4(mxs);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float mx = wave_max(logit[r]);
-            const float m_new = fmaxf(m_run[r], mx);
+            const float m_new = fmaxf(m_run[r], mxs[r]);
             alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
             p[r] = tok_ok ? __builtin_amdgcn_exp2f(logit[r] - m_new) : 0.0f;
             m_run[r] = m_new;
@@ -511,6 +544,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 // Returns 0 when launched, 1 when the shape is not covered by the tuned kernel.
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     if (Dh != 128 || R != 4 || !(a.kout == 6 || a.kout == 0)) return 1;
+    // the kernel reads q two channels at a time
+    if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
     const size_t shm = (size_t)waves * WAVE_LDS;
