@@ -36,6 +36,8 @@ extern "C" {
 #define OMMX_ERR_NONFINITE_V   2   /* pack.py:605-607 */
 #define OMMX_ERR_UNDERFILLED   4   /* fewer than k distinct outlier lanes, pack.py:520-538 */
 #define OMMX_ERR_EXP_RANGE     8   /* scale exponent does not fit the int8 plane */
+/* error bit OR-ed into *err_flag by ommx_ring_write / ommx_tail_gather */
+#define OMMX_ERR_RING_RANGE   16   /* row outside the history (kv_store_ops.py:33-34,52-53) */
 
 int ommx_abi_version(void);
 const char* ommx_last_error(void);
@@ -152,6 +154,53 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
                         float* lse, int64_t lse_stride_b,
                         int B, int Hq, int Hkv, int D, int num_splits,
                         float sm_scale, float logit_cap, void* stream);
+
+/*
+ * bf16 residual ring, write side: one new K/V row per request.
+ * Replaces ommx_gpu_serve/attention/kv_store_ops.py:22-40,63-68 (_kv_write_token /
+ * write_token) and the batched scatter of attention/kv_pool.py:407-419.
+ *   k, v          bf16 [B,H,D] with strides k_stride_b/h (D contiguous)
+ *   k_hist,v_hist bf16 [num_slots, hist_rows, H, D] dense rows; hist_stride_req elements
+ *                 between two slots (single-sequence store: num_slots = 1)
+ *   slots         NULL (request b lives in slot b) or int64[B]
+ *   pos           int64[B] absolute token position of the new row (device)
+ *   pos_next      NULL, or int64[B] that receives pos+1 (may alias pos: the device-side
+ *                 sequence counter of kv_pool.py:1037-1046 advanced by the same launch)
+ * Ring slot of position p (kv_store.py:301-327): p < sink_rows ? p
+ * : sink_rows + (p - sink_rows) % ring_span; ring_span == 0 keeps the whole history
+ * (slot = position).  A slot outside [0,hist_rows) sets OMMX_ERR_RING_RANGE and the row is
+ * not written.
+ */
+int ommx_ring_write(const uint16_t* k, const uint16_t* v, int64_t k_stride_b, int64_t k_stride_h,
+                    int64_t v_stride_b, int64_t v_stride_h,
+                    uint16_t* k_hist, uint16_t* v_hist, int64_t hist_stride_req, int hist_rows,
+                    const int64_t* slots, const int64_t* pos, int64_t* pos_next,
+                    int B, int H, int D, int sink_rows, int ring_span,
+                    int32_t* err_flag, void* stream);
+
+/*
+ * bf16 residual ring, read side: the sink + recent rows of every request into the fixed
+ * tail buffers k_tail, v_tail bf16 [B,T,H,D] (dense).
+ * Two modes:
+ *   seq != NULL       int64[B] absolute sequence lengths on the device.  The kernel does
+ *                     the window arithmetic of attention/kv_pool.py:1048-1105
+ *                     (decode_inputs_device): boundary = seq-sink-recent <= 0 ?
+ *                     min(sink,seq) : sink + ((seq-sink-recent)/gt)*gt; rows = positions
+ *                     [0,min(sink,seq)) ++ [boundary,seq); and writes
+ *                     b_tail_len[b] = min(rows, T), b_seq_len[b] = max(boundary-sink, 0)
+ *                     (either may be NULL).  Rows past the count repeat position 0; the
+ *                     decode kernels mask them by b_tail_len.
+ *   tail_idx != NULL  int64[B,T] explicit absolute positions (kv_store_ops.py:42-61,71-76
+ *                     _kv_gather_tail / gather_tail); the length outputs are not written.
+ * Positions map to history rows as in ommx_ring_write; a row outside the history sets
+ * OMMX_ERR_RING_RANGE and yields zeros.
+ */
+int ommx_tail_gather(const uint16_t* k_hist, const uint16_t* v_hist, int64_t hist_stride_req,
+                     int hist_rows, const int64_t* slots, const int64_t* seq,
+                     const int64_t* tail_idx,
+                     uint16_t* k_tail, uint16_t* v_tail, int32_t* b_tail_len, int32_t* b_seq_len,
+                     int B, int T, int H, int D, int sink_rows, int recent_rows, int group_tokens,
+                     int ring_span, int32_t* err_flag, void* stream);
 
 #ifdef __cplusplus
 }

@@ -2,6 +2,9 @@
 
 The public names mirror ``ommx_gpu_serve.attention`` of the reference.
 """
+from .kv_pool import MultiSeqKVPool
+from .kv_store import CanonicalKVStore
+from .kv_store_ops import gather_tail, gather_tails, ring_slot, write_token, write_tokens
 from .kv_window import WindowSpec, packed_boundary, tail_token_indices
 from .pack import (CANONICAL_GROUP_CHANNELS, CANONICAL_GROUP_TOKENS, alloc_planes,
                    ommx_pack_kv_canonical_block, store_pack_into)
@@ -12,4 +15,6 @@ __all__ = [
     "ommx_paged_decode_attention_canonical", "ommx_pack_kv_canonical_block", "store_pack_into",
     "alloc_planes", "auto_num_kv_splits", "make_attn_logits", "WindowSpec", "packed_boundary",
     "tail_token_indices", "CANONICAL_GROUP_TOKENS", "CANONICAL_GROUP_CHANNELS",
+    "MultiSeqKVPool", "CanonicalKVStore", "write_token", "write_tokens", "gather_tail",
+    "gather_tails", "ring_slot",
 ]

@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
-ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE = 1, 2, 4, 8
+ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -41,6 +41,10 @@ _SIGNATURES = {
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),
     "ommx_decode_combine": (_I, [_P, _L, _L, _L, _P, _L, _L, _P, _P, _L, _L, _L, _L, _L, _L,
                                  _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _F, _F, _P]),
+    "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
+                             _I, _I, _I, _I, _I, _P, _P]),
+    "ommx_tail_gather": (_I, [_P, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P,
+                              _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
 }
 
 

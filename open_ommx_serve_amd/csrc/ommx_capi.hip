@@ -3,6 +3,7 @@
 #include <string>
 
 #include "ommx_decode_args.h"
+#include "ommx_ring_args.h"
 
 namespace ommx {
 
@@ -149,5 +150,60 @@ extern "C" int ommx_decode_combine(
         return -1;
     }
     if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_combine: launch failed"); return -2; }
+    return 0;
+}
+
+// bf16 residual ring: one new K/V row per request (kv_store_ops.py:63-68, kv_pool.py:407-419).
+extern "C" int ommx_ring_write(
+    const uint16_t* k, const uint16_t* v, int64_t k_stride_b, int64_t k_stride_h,
+    int64_t v_stride_b, int64_t v_stride_h,
+    uint16_t* k_hist, uint16_t* v_hist, int64_t hist_stride_req, int hist_rows,
+    const int64_t* slots, const int64_t* pos, int64_t* pos_next,
+    int B, int H, int D, int sink_rows, int ring_span, int32_t* err_flag, void* stream) {
+    using namespace ommx;
+    if (B <= 0 || H <= 0 || D <= 0 || hist_rows <= 0 || sink_rows < 0 || ring_span < 0) {
+        set_error("ommx_ring_write: bad shape");
+        return -1;
+    }
+    if (!k || !v || !k_hist || !v_hist || !pos) { set_error("ommx_ring_write: null pointer"); return -1; }
+    if (ring_span > 0 && sink_rows + ring_span > hist_rows) {
+        set_error("ommx_ring_write: sink_rows + ring_span exceeds the history rows");
+        return -1;
+    }
+    RingArgs a{k_hist, v_hist, hist_stride_req, hist_rows, sink_rows, ring_span, H, D, slots, err_flag};
+    launch_ring_write(a, k, v, k_stride_b, k_stride_h, v_stride_b, v_stride_h, pos, pos_next, B,
+                      static_cast<hipStream_t>(stream));
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_ring_write: launch failed"); return -2; }
+    return 0;
+}
+
+// Tail rows (sink + recent) of every request into the fixed tail buffers, plus the packed /
+// tail lengths of the decode call (kv_pool.py:1048-1105, kv_store_ops.py:71-76).
+extern "C" int ommx_tail_gather(
+    const uint16_t* k_hist, const uint16_t* v_hist, int64_t hist_stride_req, int hist_rows,
+    const int64_t* slots, const int64_t* seq, const int64_t* tail_idx,
+    uint16_t* k_tail, uint16_t* v_tail, int32_t* b_tail_len, int32_t* b_seq_len,
+    int B, int T, int H, int D, int sink_rows, int recent_rows, int group_tokens, int ring_span,
+    int32_t* err_flag, void* stream) {
+    using namespace ommx;
+    if (B <= 0 || T <= 0 || H <= 0 || D <= 0 || hist_rows <= 0 || sink_rows < 0 || ring_span < 0 ||
+        recent_rows < 0 || group_tokens <= 0) {
+        set_error("ommx_tail_gather: bad shape");
+        return -1;
+    }
+    if (!k_hist || !v_hist || !k_tail || !v_tail || (!seq && !tail_idx)) {
+        set_error("ommx_tail_gather: null pointer (one of seq, tail_idx is required)");
+        return -1;
+    }
+    if (seq && tail_idx) { set_error("ommx_tail_gather: pass seq or tail_idx, not both"); return -1; }
+    if (ring_span > 0 && sink_rows + ring_span > hist_rows) {
+        set_error("ommx_tail_gather: sink_rows + ring_span exceeds the history rows");
+        return -1;
+    }
+    RingArgs a{const_cast<uint16_t*>(k_hist), const_cast<uint16_t*>(v_hist), hist_stride_req,
+               hist_rows, sink_rows, ring_span, H, D, slots, err_flag};
+    launch_tail_gather(a, seq, tail_idx, k_tail, v_tail, B, T, recent_rows, group_tokens,
+                       b_tail_len, b_seq_len, static_cast<hipStream_t>(stream));
+    if (hipGetLastError() != hipSuccess) { set_error("ommx_tail_gather: launch failed"); return -2; }
     return 0;
 }

@@ -180,3 +180,56 @@ def test_missing_library_is_a_loud_error(monkeypatch):
     monkeypatch.setattr(_hip, "_LIB_PATH", "/nonexistent/libommx_hip.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _hip.load()
+
+
+# ── KV store host logic ──────────────────────────────────────────────────────────────────
+
+def test_ring_slot_pins_the_sink_and_never_aliases_live_rows():
+    """Ring map of kv_store.py:301-313.  At every length the rows that can still be read
+    (sink, and [boundary - group, seq)) must land on distinct ring rows."""
+    from open_ommx_serve_amd.attention.kv_store_ops import ring_slot
+    win = kv_window.WindowSpec()
+    sink, span = win.sink_tokens, win.recent_window + 2 * win.group_tokens
+    assert [ring_slot(p, sink, span) for p in range(sink)] == list(range(sink))
+    assert ring_slot(sink, sink, span) == sink and ring_slot(sink + span, sink, span) == sink
+    assert ring_slot(12345, sink, 0) == 12345
+    for n in range(1, 700):
+        edge = win.boundary(n)
+        live = list(range(min(sink, n))) + list(range(max(sink, edge - win.group_tokens), n))
+        slots = [ring_slot(p, sink, span) for p in live]
+        assert len(set(slots)) == len(slots) and max(slots) < sink + span, n
+
+
+def test_store_classes_refuse_other_recipes_and_the_cpu():
+    from open_ommx_serve_amd.attention import CanonicalKVStore, MultiSeqKVPool
+    from open_ommx_serve_amd.attention.kv_pool import check_serving_recipe
+    good = dict(k_format="i2f4", outliers_per_vector=6, outlier_select="signed",
+                outlier_repr="bitmap", use_pow2=True)
+    check_serving_recipe(**good, kv_outlier_map=True, kv_int8_scale=True, group_tokens=32,
+                         group_channels=32, scale_dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="relidx7"):
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "outlier_repr": "relidx7"})
+    with pytest.raises(NotImplementedError, match="use_pow2"):
+        CanonicalKVStore(128, 8, 256, device="cpu", **{**good, "use_pow2": False})
+    with pytest.raises(ValueError, match="k_format"):
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "k_format": "i3"})
+    with pytest.raises(ValueError, match="multiple of 32"):
+        CanonicalKVStore(100, 8, 256, device="cpu", **good)
+    with pytest.raises(ValueError, match="multiple of page_size"):
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu", window=kv_window.WindowSpec(page_size=24), **good)
+    # the serving recipe on a CPU device: there is no CPU path
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **good)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        CanonicalKVStore(128, 8, 256, device="cpu", **good)
+
+
+def test_ring_ops_validate_before_touching_the_device():
+    from open_ommx_serve_amd.attention import gather_tails, write_tokens
+    kh = torch.zeros(1, 16, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        write_tokens(kh, kh.clone(), torch.zeros(1, dtype=torch.int64), kh[0, :1], kh[0, :1], 0, 0)
+    with pytest.raises(ValueError, match="bfloat16"):
+        write_tokens(kh.float(), kh.float(), torch.zeros(1, dtype=torch.int64), kh[0, :1], kh[0, :1], 0, 0)
+    with pytest.raises(ValueError, match="num_slots"):
+        gather_tails(kh[0], kh[0], kh, kh, 0, 0, seq=torch.zeros(1, dtype=torch.int64))

@@ -1,0 +1,332 @@
+"""KV store write seams on the GPU: ring copies, incremental packing, decode through the pool.
+
+What pins what:
+* ring copies are pure row moves: compared with torch indexing of the same history;
+* the window arithmetic done inside the gather kernel is compared with the host closed forms
+  (``WindowSpec``), which the CPU suite pins against brute force;
+* incremental packing must equal, bit for bit, the oracle packer run once over the whole
+  packed prefix (32-token groups are packed independently, reference kv_pool.py:563-566);
+* decode through the pool's argument bundle is compared with the oracle's
+  dequantise-then-attend result on the full token history (tolerance: max-abs 2e-3,
+  mean-abs 2e-4).
+"""
+import math
+
+import pytest
+import torch
+
+import oracle.ommx_oracle as O
+from conftest import PLANE_NAMES
+from open_ommx_serve_amd.attention import (CanonicalKVStore, MultiSeqKVPool, WindowSpec,
+                                           gather_tails, ommx_paged_decode_attention_canonical,
+                                           write_tokens)
+from open_ommx_serve_amd.attention.kv_store_ops import ring_slot
+from open_ommx_serve_amd.synth import synth_kv, synth_q
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-3, 2e-4
+RECIPE = dict(k_format="i2f4", outliers_per_vector=6, outlier_select="signed",
+              outlier_repr="bitmap", use_pow2=True)
+DEV = "cuda"
+
+
+def _rows(n, H, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, H, D, generator=g).to(torch.bfloat16)
+
+
+# ── ring copies ────────────────────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("span", [0, 96])
+def test_write_tokens_matches_indexing_and_advances_the_counter(span):
+    N, H, D, sink = 5, 8, 128, 8
+    rows = sink + span if span else 300
+    kh = torch.zeros(N, rows, H, D, dtype=torch.bfloat16, device=DEV)
+    vh = torch.zeros_like(kh)
+    want_k, want_v = kh.cpu().clone(), vh.cpu().clone()
+    slots = torch.tensor([3, 0, 4], dtype=torch.int64, device=DEV)
+    pos = torch.tensor([5, 150, 299], dtype=torch.int64, device=DEV)
+    for step in range(3):
+        k, v = _rows(3, H, D, 10 + step), _rows(3, H, D, 20 + step)
+        p_host = pos.cpu().tolist()
+        write_tokens(kh, vh, pos, k.to(DEV), v.to(DEV), sink if span else 0, span, slots=slots,
+                     pos_next=pos)
+        for b, s in enumerate(slots.cpu().tolist()):
+            r = ring_slot(p_host[b], sink, span) if span else p_host[b]
+            if r < rows:
+                want_k[s, r], want_v[s, r] = k[b], v[b]
+        assert pos.cpu().tolist() == [p + 1 for p in p_host]
+    assert torch.equal(kh.cpu(), want_k) and torch.equal(vh.cpu(), want_v)
+
+
+def test_write_outside_the_history_sets_the_error_bit_and_writes_nothing():
+    kh = torch.zeros(1, 16, 2, 64, dtype=torch.bfloat16, device=DEV)
+    vh = torch.zeros_like(kh)
+    err = torch.zeros(1, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([16], dtype=torch.int64, device=DEV)
+    write_tokens(kh, vh, pos, _rows(1, 2, 64, 1).to(DEV), _rows(1, 2, 64, 2).to(DEV), 0, 0, err_flag=err)
+    assert int(err.item()) == 16 and not kh.any() and not vh.any()
+
+
+def test_strided_source_rows_take_the_elementwise_path():
+    H, D = 4, 64
+    kh = torch.zeros(2, 40, H, D, dtype=torch.bfloat16, device=DEV)
+    vh = torch.zeros_like(kh)
+    big = _rows(2, H, D + 3, 5).to(DEV)          # rows are not 16-byte aligned
+    k, v = big[:, :, 1:D + 1], big[:, :, 2:D + 2]
+    pos = torch.tensor([7, 39], dtype=torch.int64, device=DEV)
+    write_tokens(kh, vh, pos, k, v, 0, 0)
+    assert torch.equal(kh[0, 7], k[0]) and torch.equal(kh[1, 39], k[1])
+    assert torch.equal(vh[0, 7], v[0]) and torch.equal(vh[1, 39], v[1])
+
+
+@pytest.mark.parametrize("ring", [False, True])
+def test_gather_window_arithmetic_matches_the_host_closed_forms(ring):
+    win = WindowSpec()
+    sink, recent, gt = win.sink_tokens, win.recent_window, win.group_tokens
+    span = recent + 2 * gt if ring else 0
+    seqs = [0, 1, 5, 8, 9, 39, 40, 41, 71, 72, 73, 103, 104, 105, 135, 1000, 4096, 4097, 4135]
+    N, H, D = len(seqs), 2, 64
+    rows = sink + span if ring else max(seqs) + 1
+    T = win.max_tail_len()
+    # history row r of slot s holds the value that identifies (s, r)
+    kh = (torch.arange(N * rows, dtype=torch.float32).reshape(N, rows, 1, 1) % 251).expand(
+        N, rows, H, D).to(torch.bfloat16).contiguous().to(DEV)
+    vh = (kh.float() + 1).to(torch.bfloat16)
+    kt = torch.full((N, T, H, D), -1.0, dtype=torch.bfloat16, device=DEV)
+    vt = torch.full_like(kt, -1.0)
+    b_tail = torch.full((N,), -1, dtype=torch.int32, device=DEV)
+    b_seq = torch.full((N,), -1, dtype=torch.int32, device=DEV)
+    seq = torch.tensor(seqs, dtype=torch.int64, device=DEV)
+    gather_tails(kh, vh, kt, vt, sink if ring else 0, span, seq=seq, b_tail_len=b_tail, b_seq_len=b_seq,
+                 window_sink=sink, window_recent=recent, group_tokens=gt)
+    kt, vt, khc, vhc = kt.cpu(), vt.cpu(), kh.cpu(), vh.cpu()
+    for b, n in enumerate(seqs):
+        idx = win.tail_indices(n)
+        assert int(b_tail[b]) == min(len(idx), T), (n, int(b_tail[b]))
+        assert int(b_seq[b]) == win.packed_len(n), (n, int(b_seq[b]))
+        for t in range(T):
+            p = idx[t] if t < len(idx) else 0
+            r = ring_slot(p, sink, span) if ring else p
+            assert torch.equal(kt[b, t], khc[b, r]) and torch.equal(vt[b, t], vhc[b, r]), (n, t)
+
+
+def test_gather_explicit_positions_through_slots():
+    N, rows, H, D, T = 3, 50, 2, 64, 6
+    kh = _rows(N * rows, H, D, 3).reshape(N, rows, H, D).to(DEV)
+    vh = _rows(N * rows, H, D, 4).reshape(N, rows, H, D).to(DEV)
+    slots = torch.tensor([2, 0], dtype=torch.int64, device=DEV)
+    idx = torch.tensor([[0, 1, 49, 7, 0, 0], [3, 3, 3, 10, 11, 12]], dtype=torch.int64, device=DEV)
+    kt = torch.empty(2, T, H, D, dtype=torch.bfloat16, device=DEV)
+    vt = torch.empty_like(kt)
+    gather_tails(kh, vh, kt, vt, 0, 0, tail_idx=idx, slots=slots)
+    for b in range(2):
+        assert torch.equal(kt[b], kh[slots[b]].index_select(0, idx[b]))
+        assert torch.equal(vt[b], vh[slots[b]].index_select(0, idx[b]))
+
+
+# ── pool: incremental packing and decode ─────────────────────────────────────────────────
+
+def _decode_bundle(q, bundle, sm_scale, k):
+    pl = bundle["planes"]
+    B, Hq, D = q.shape
+    o = torch.full((B, Hq, D), float("nan"), dtype=torch.float32, device=q.device)
+    lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=q.device)
+    ommx_paged_decode_attention_canonical(
+        q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"],
+        pl["v_main"], pl["v_scale"], pl["v_zp"], bundle["k_tail"], bundle["v_tail"],
+        bundle["b_tail_len"], o, lse, bundle.get("req_to_token", pl["req_to_token"]),
+        bundle.get("req_to_group", pl["req_to_group"]), bundle["b_seq_len"],
+        sm_scale=sm_scale, page_size=pl["page_size"], k_outliers_per_vector=k,
+        bitmap_read=True, k_obmp=pl["k_obmp"], k_fp4_mapscale=pl["k_fp4_mapscale"],
+        k_fp4_mapcenter=pl["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
+        max_seq_len=bundle["max_seq_len"], max_tail_len=bundle["max_tail_len"],
+        packed_start_offset=bundle["packed_start_offset"])
+    torch.cuda.synchronize()
+    return o.cpu(), lse.cpu()
+
+
+def _oracle_decode(q, K_hist, V_hist, win, sm_scale):
+    """Dequantise-then-attend over the full history of every request (fp64)."""
+    outs, lses = [], []
+    for b, (K, V) in enumerate(zip(K_hist, V_hist)):
+        n = int(K.shape[0])
+        edge = win.boundary(n)
+        Kf = [K[i].float() for i in win.tail_indices(n)]
+        Vf = [V[i].float() for i in win.tail_indices(n)]
+        Kd = torch.stack(Kf) if Kf else torch.zeros(0, *K.shape[1:])
+        Vd = torch.stack(Vf) if Vf else torch.zeros(0, *V.shape[1:])
+        if edge > win.sink_tokens:
+            planes = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size)
+            Kp, Vp = O.dequant_kv(planes)
+            Kd, Vd = torch.cat([Kp, Kd]), torch.cat([Vp, Vd])
+        o, lse = O.attend(q[b].cpu(), Kd, Vd, sm_scale, dtype=torch.float64)
+        outs.append(o)
+        lses.append(lse)
+    return torch.stack(outs), torch.stack(lses)
+
+
+def _assert_planes_equal_oracle(got: dict, K, V, win, what):
+    n = int(K.shape[0])
+    edge = win.boundary(n)
+    assert got["num_tokens"] == max(0, edge - win.sink_tokens), what
+    if edge <= win.sink_tokens:
+        return
+    want = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size)
+    for name in PLANE_NAMES:
+        a, b = got[name].cpu(), want[name]
+        assert a.shape == b.shape and a.dtype == b.dtype, (what, name)
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{what}: plane {name} differs"
+
+
+def _check_out(got, want, what):
+    (o, lse), (wo, wl) = got, want
+    err = (o.double() - wo).abs()
+    assert torch.isfinite(o).all(), what
+    assert err.max().item() <= MAX_ABS, f"{what}: max-abs {err.max().item():.3e}"
+    assert err.mean().item() <= MEAN_ABS, f"{what}: mean-abs {err.mean().item():.3e}"
+    assert (lse.double() - wl).abs().max().item() <= 2e-3, f"{what}: lse"
+
+
+@pytest.mark.parametrize("ring", [False, True])
+@pytest.mark.parametrize("q_heads", [32, 64])
+def test_pool_prefill_then_decode_steps(ring, q_heads):
+    """Ragged prefill, then 70 appended tokens per request: every request crosses two group
+    boundaries.  Planes are compared after every pack, decode output every 9th step."""
+    H, D, B = 8, 128, 3
+    win = WindowSpec()
+    prefill = [700, 1029, 37]
+    steps = 70
+    sm_scale = 1.0 / math.sqrt(D)
+    Ks, Vs = zip(*[synth_kv(n + steps, H, D, seed=100 + i, sparse_frac=0.005) for i, n in enumerate(prefill)])
+    pool = MultiSeqKVPool(D, H, num_seqs=4, max_seq_len=1200, window=win, device=DEV, kv_ring=ring, **RECIPE)
+    slot_of = [2, 0, 3]                       # requests do not sit in batch order
+    for i, r in enumerate(slot_of):
+        n_packed = pool.append_block(r, Ks[i][:prefill[i]].to(DEV), Vs[i][:prefill[i]].to(DEV))
+        assert n_packed == win.num_groups(prefill[i])
+        _assert_planes_equal_oracle(pool.request_planes(r), Ks[i][:prefill[i]], Vs[i][:prefill[i]], win,
+                                    f"prefill req {i}")
+    q_all = synth_q(steps, B * q_heads, D, seed=5).reshape(steps, B, q_heads, D)
+    for s in range(steps):
+        newK = torch.stack([Ks[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        newV = torch.stack([Vs[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        packed = pool.append_decode_batched(slot_of, newK, newV)
+        cur = [prefill[i] + s + 1 for i in range(B)]
+        if packed:
+            for i, r in enumerate(slot_of):
+                _assert_planes_equal_oracle(pool.request_planes(r), Ks[i][:cur[i]], Vs[i][:cur[i]], win,
+                                            f"step {s} req {i}")
+        if s % 9 == 0 or s == steps - 1:
+            bundle = pool.decode_inputs_batched(slot_of)
+            assert bundle["b_seq_len"].tolist() == [win.packed_len(n) for n in cur]
+            assert bundle["b_tail_len"].tolist() == [len(win.tail_indices(n)) for n in cur]
+            q = q_all[s].to(DEV)
+            got = _decode_bundle(q, bundle, sm_scale, 6)
+            want = _oracle_decode(q, [Ks[i][:cur[i]] for i in range(B)], [Vs[i][:cur[i]] for i in range(B)],
+                                  win, sm_scale)
+            _check_out(got, want, f"ring={ring} Hq={q_heads} step {s}")
+    pool.check_errors()
+
+
+def test_pool_device_counter_path_equals_the_host_path():
+    """append_decode_device / decode_inputs_device (device sequence counter) against
+    append_decode_batched / decode_inputs_batched on a second pool fed the same rows."""
+    H, D, B, steps = 2, 64, 3, 40
+    win = WindowSpec()
+    prefill = [45, 72, 100]
+    Ks, Vs = zip(*[synth_kv(n + steps, H, D, seed=300 + i) for i, n in enumerate(prefill)])
+    pools = [MultiSeqKVPool(D, H, num_seqs=B, max_seq_len=200, window=win, device=DEV, kv_ring=True, **RECIPE)
+             for _ in range(2)]
+    for p in pools:
+        for i in range(B):
+            p.append_block(i, Ks[i][:prefill[i]].to(DEV), Vs[i][:prefill[i]].to(DEV))
+    pools[0].decode_seed_seq_device(range(B))
+    for s in range(steps):
+        newK = torch.stack([Ks[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        newV = torch.stack([Vs[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        n0 = pools[0].append_decode_device(newK, newV, B)
+        n1 = pools[1].append_decode_batched(range(B), newK, newV)
+        assert n0 == n1
+        a = pools[0].decode_inputs_device(B, 200)
+        b = pools[1].decode_inputs_batched(range(B))
+        assert torch.equal(a["b_seq_len"], b["b_seq_len"]) and torch.equal(a["b_tail_len"], b["b_tail_len"])
+        for i in range(B):
+            n = int(a["b_tail_len"][i])
+            assert torch.equal(a["k_tail"][i, :n], b["k_tail"][i, :n])
+            assert torch.equal(a["v_tail"][i, :n], b["v_tail"][i, :n])
+    for name in PLANE_NAMES:
+        assert torch.equal(getattr(pools[0], name), getattr(pools[1], name)), name
+    assert pools[0]._dbuf["seq_dev"][:B].tolist() == [prefill[i] + steps for i in range(B)]
+    pools[0].check_errors()
+
+
+def test_pool_reports_non_finite_rows_lazily():
+    H, D = 2, 64
+    pool = MultiSeqKVPool(D, H, num_seqs=1, max_seq_len=200, device=DEV, kv_ring=False, **RECIPE)
+    K, V = synth_kv(80, H, D, seed=1)
+    K[20, 1, 5] = float("nan")
+    pool.append_block(0, K.to(DEV), V.to(DEV))
+    with pytest.raises((ValueError, IndexError)):
+        pool.check_errors()
+    pool.check_errors()                      # the flag was cleared by the first read
+
+
+# ── single-sequence store ───────────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("ring", [False, True])
+def test_store_prefill_write_token_advance_and_decode(ring):
+    H, D, Hq = 8, 128, 32
+    win = WindowSpec()
+    prefill, steps = 300, 40
+    K, V = synth_kv(prefill + steps, H, D, seed=77, sparse_frac=0.005)
+    st = CanonicalKVStore(D, H, max_seq_len=512, window=win, device=DEV, kv_ring=ring, **RECIPE)
+    st.append_block(K[:prefill].to(DEV), V[:prefill].to(DEV))
+    pos = torch.zeros(1, dtype=torch.int64, device=DEV)
+    sm_scale = 1.0 / math.sqrt(D)
+    qs = synth_q(steps, Hq, D, seed=9)
+    for s in range(steps):
+        n = prefill + s + 1
+        pos.fill_(n - 1)
+        st.write_token(pos, K[n - 1].to(DEV), V[n - 1].to(DEV))
+        packed = st.advance_to(n)
+        assert packed == win.newly_completed_groups(n - 1, n)
+        if packed or s == 0:
+            got = st.decode_planes()
+            _assert_planes_equal_oracle(got, K[:n], V[:n], win, f"store step {s}")
+        # fixed-buffer gather (the graph path) and the allocating one agree
+        idx = win.tail_indices(n)
+        tidx = torch.zeros(st.tail_cap, dtype=torch.int64, device=DEV)
+        tidx[:len(idx)] = torch.tensor(idx)
+        st.gather_tail_into(tidx, st.k_tail_buf, st.v_tail_buf, len(idx))
+        kt, vt, nt = st.tail_bf16()
+        assert nt == len(idx)
+        assert torch.equal(st.k_tail_buf[0, :nt], kt[0]) and torch.equal(kt[0].cpu(), K[idx])
+        assert torch.equal(st.v_tail_buf[0, :nt], vt[0]) and torch.equal(vt[0].cpu(), V[idx])
+        if s % 13 == 0 or s == steps - 1:
+            bundle = st.decode_inputs()
+            q = qs[s:s + 1].to(DEV)
+            got = _decode_bundle(q, bundle, sm_scale, 6)
+            want = _oracle_decode(q, [K[:n]], [V[:n]], win, sm_scale)
+            _check_out(got, want, f"store ring={ring} step {s}")
+    st.check_errors()
+    st.reset_inplace()
+    assert st.seq_len == 0 and st.packed_groups == 0
+
+
+def test_eager_append_matches_write_token():
+    H, D = 2, 64
+    K, V = synth_kv(120, H, D, seed=3)
+    a = CanonicalKVStore(D, H, max_seq_len=128, device=DEV, kv_ring=True, **RECIPE)
+    b = CanonicalKVStore(D, H, max_seq_len=128, device=DEV, kv_ring=True, **RECIPE)
+    pos = torch.zeros(1, dtype=torch.int64, device=DEV)
+    for n in range(120):
+        a.append(K[n].to(DEV), V[n].to(DEV))
+        a.maybe_regroup()
+        pos.fill_(n)
+        b.write_token(pos, K[n].to(DEV), V[n].to(DEV))
+        b.advance_to(n + 1)
+    assert a.packed_groups == b.packed_groups == WindowSpec().num_groups(120)
+    assert torch.equal(a.k_hist, b.k_hist) and torch.equal(a.v_hist, b.v_hist)
+    for name in PLANE_NAMES:
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
