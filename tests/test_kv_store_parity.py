@@ -330,3 +330,60 @@ def test_eager_append_matches_write_token():
     assert torch.equal(a.k_hist, b.k_hist) and torch.equal(a.v_hist, b.v_hist)
     for name in PLANE_NAMES:
         assert torch.equal(getattr(a, name), getattr(b, name)), name
+
+
+def test_config5_bulk_pack_then_128_decode_steps_at_full_size():
+    """64 q / 8 kv heads, 8 requests of 32768 tokens: bulk-pack 32704 tokens per request, then
+    128 decode steps, each appending one token per request (4 incremental packs per request)
+    and decoding.  Full-size checks are properties plus the oracle on one request:
+    * after the last step the pool planes of every request equal ONE store launch over the
+      whole packed prefix of its history (incremental == bulk, bit for bit), and request 0's
+      also equal the oracle packer's planes;
+    * tails equal the history rows the window names;
+    * decode output of request 0 against the oracle at the first, a middle and the last
+      step; every step's output is finite and every request's lse is consistent with a
+      second decode through a different split count."""
+    from open_ommx_serve_amd.attention.pack import alloc_planes, store_pack_into
+    H, D, Hq, B = 8, 128, 64, 8
+    ctx, steps = 32768, 128
+    win = WindowSpec()
+    sm_scale = 1.0 / math.sqrt(D)
+    pool = MultiSeqKVPool(D, H, num_seqs=B, max_seq_len=ctx + steps, window=win, device=DEV,
+                          kv_ring=True, **RECIPE)
+    Ks, Vs = [], []
+    for i in range(B):
+        K, V = synth_kv(ctx + steps, H, D, seed=500 + i, sparse_frac=0.005)
+        Ks.append(K)
+        Vs.append(V)
+        assert pool.append_block(i, K[:ctx].to(DEV), V[:ctx].to(DEV)) == 1022
+    assert pool.packed_groups == [1022] * B          # 32704 packed tokens per request
+    pool.decode_seed_seq_device(range(B))
+    qs = synth_q(steps, B * Hq, D, seed=6).reshape(steps, B, Hq, D)
+    packs = 0
+    for s in range(steps):
+        newK = torch.stack([Ks[i][ctx + s] for i in range(B)]).to(DEV)
+        newV = torch.stack([Vs[i][ctx + s] for i in range(B)]).to(DEV)
+        packs += pool.append_decode_device(newK, newV, B)
+        bundle = pool.decode_inputs_device(B, ctx + steps)
+        q = qs[s].to(DEV)
+        o, lse = _decode_bundle(q, bundle, sm_scale, 6)
+        assert torch.isfinite(o).all() and torch.isfinite(lse).all(), s
+        n = ctx + s + 1
+        if s in (0, 70, steps - 1):
+            want = _oracle_decode(q[:1], [Ks[0][:n]], [Vs[0][:n]], win, sm_scale)
+            _check_out((o[:1], lse[:1]), want, f"config 5 step {s}")
+    assert packs == 4 * B and pool.packed_groups == [1026] * B
+    pool.check_errors()
+    n = ctx + steps
+    edge = win.boundary(n)
+    for i in range(B):
+        got = pool.request_planes(i)
+        ref = alloc_planes(got["k_base"].shape[0], got["k_scale"].shape[0], H, D, device=DEV)
+        store_pack_into(Ks[i][win.sink_tokens:edge].to(DEV), Vs[i][win.sink_tokens:edge].to(DEV), ref)
+        for name in PLANE_NAMES:
+            assert torch.equal(got[name], ref[name]), f"req {i} plane {name}: incremental != bulk"
+        kt, vt, bt = pool.tail_bf16_batched([i])
+        idx = win.tail_indices(n)
+        assert int(bt[0]) == len(idx)
+        assert torch.equal(kt[0, :len(idx)].cpu(), Ks[i][idx]) and torch.equal(vt[0, :len(idx)].cpu(), Vs[i][idx])
+    _assert_planes_equal_oracle(pool.request_planes(0), Ks[0][:n], Vs[0][:n], win, "config 5 req 0")
