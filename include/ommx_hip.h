@@ -95,8 +95,8 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 lse=-inf (paged_decode.py:2262-2284)
  * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
  * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64;
- * num_splits <= 256; planes 8-byte aligned.  head_dim 128 with r = 4 and 6 (or 0) outliers
- * runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
+ * num_splits <= 256; planes 8-byte aligned.  head_dim 128 with r = 4 or 8 and 6 (or 0)
+ * outliers runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,

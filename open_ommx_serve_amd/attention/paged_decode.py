@@ -30,12 +30,14 @@ def _cu_count(device: torch.device) -> int:
     return _CU_COUNT[key]
 
 
-def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256) -> int:
-    """Split count that gives every compute unit two workgroups (a workgroup covers four kv
-    heads of one split) of at least four 64-token steps each; at most 256, the number of
-    partial states the combine kernel keeps on chip."""
+def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256,
+                       q_per_kv: int = 4) -> int:
+    """Split count that gives every compute unit two workgroups (a workgroup is four waves of
+    one split; a wave covers one kv head and four of its q heads) of at least four 64-token
+    steps each; at most 256, the number of partial states the combine kernel keeps on chip."""
     steps = max(1, (int(max_seq_len) + 63) // 64)
-    wgs_per_split = max(1, int(batch) * max(1, int(kv_heads) // 4))
+    waves_per_split = int(kv_heads) * max(1, int(q_per_kv) // 4)
+    wgs_per_split = max(1, int(batch) * max(1, waves_per_split // 4))
     want = max(1, (2 * int(n_cu)) // wgs_per_split)
     return int(max(1, min(256, want, max(1, steps // 4))))
 
@@ -178,7 +180,7 @@ def ommx_paged_decode_attention_canonical(
     else:
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
     if num_kv_splits is None:
-        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device))
+        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv)
     S = max(1, int(num_kv_splits))
     if attn_logits is None:
         attn_logits = make_attn_logits(B, Hq, S, D, q.device)

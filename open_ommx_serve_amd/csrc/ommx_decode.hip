@@ -1,10 +1,11 @@
-// Tuned split-KV decode kernel for gfx950: head_dim 128, 4 q heads per kv head, 6 (or 0)
+// Tuned split-KV decode kernel for gfx950: head_dim 128, 4 or 8 q heads per kv head, 6 (or 0)
 // outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
 //
-// Work decomposition.  A wavefront owns one kv head of one split and walks it 64 tokens
-// (two 32-token K groups) at a time; waves never synchronise with each other.  A
-// workgroup is 4 waves = 4 neighbouring kv heads, so together they consume whole 128-byte
-// lines of the token-major k_base / v_main rows.
+// Work decomposition.  A wavefront owns one kv head (and 4 of its q heads) of one split and
+// walks it 64 tokens (two 32-token K groups) at a time; waves never synchronise with each
+// other.  A workgroup is 4 waves = 4 neighbouring kv heads (2 kv heads x 2 q-head groups
+// when a kv head serves 8 q heads), so together they consume whole 128-byte (64-byte) pieces
+// of the token-major k_base / v_main rows.
 //
 // Arithmetic.  All dot products run on the matrix pipe (v_mfma_f32_16x16x32, fp32
 // accumulate) with operands that are EXACT in their 16-bit type:
@@ -155,7 +156,12 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int j = lane & 15, kq = lane >> 4;
     const int Hkv = a.Hkv;
     const int waves = blockDim.x >> 6;
-    const int kvh = blockIdx.y * waves + wave;
+    // 8 q heads per kv head run as two waves of 4 heads on the same kv head (the second
+    // read of the K/V lines hits the caches; HBM traffic stays one pass)
+    const int qgroups = a.Hq / (Hkv * 4);
+    const int vhead = blockIdx.y * waves + wave;
+    const int kvh = qgroups == 2 ? (vhead >> 1) : vhead;
+    const int qh0 = qgroups == 2 ? kvh * 8 + 4 * (vhead & 1) : kvh * 4;      // first of this wave's 4 q heads
     const int b = blockIdx.z, sp = blockIdx.x;
     const int L = a.seq[b];
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
@@ -254,7 +260,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
     u32x4 aq_pair[4], aq_nat[4];
     {
-        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(kvh * 4 + (j & 3)) * a.q_sh + 32 * kq;
+        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(qh0 + (j & 3)) * a.q_sh + 32 * kq;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
@@ -274,7 +280,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const uint32_t w = *reinterpret_cast<const uint32_t*>(
-                a.q + b * a.q_sb + (int64_t)(kvh * 4 + r) * a.q_sh + 2 * lane);
+                a.q + b * a.q_sb + (int64_t)(qh0 + r) * a.q_sh + 2 * lane);
             q4[0][r] = 4.0f * __uint_as_float(w << 16);
             q4[1][r] = 4.0f * __uint_as_float(w & 0xFFFF0000u);
         }
@@ -524,7 +530,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         const int ch0 = 16 * (j & 7) + 8 * (j >> 3);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float* dst = a.al + b * a.al_b + (int64_t)(kvh * 4 + r) * a.al_h + (int64_t)sp * a.al_s;
+            float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
             const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
 #pragma unroll
             for (int y = 0; y < 8; ++y)
@@ -532,7 +538,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         }
     }
     if (lane < 4) {
-        float* dst = a.al + b * a.al_b + (int64_t)(kvh * 4 + lane) * a.al_h + (int64_t)sp * a.al_s;
+        float* dst = a.al + b * a.al_b + (int64_t)(qh0 + lane) * a.al_h + (int64_t)sp * a.al_s;
         const float lt = lane == 0 ? l_tot[0] : (lane == 1 ? l_tot[1] : (lane == 2 ? l_tot[2] : l_tot[3]));
         const float mt = lane == 0 ? m_run[0] : (lane == 1 ? m_run[1] : (lane == 2 ? m_run[2] : m_run[3]));
         dst[D] = lt > 0.0f ? (mt + log2f(lt)) * 0.6931471805599453f : -INFINITY;
@@ -543,11 +549,12 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 
 // Returns 0 when launched, 1 when the shape is not covered by the tuned kernel.
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
-    if (Dh != 128 || R != 4 || !(a.kout == 6 || a.kout == 0)) return 1;
+    if (Dh != 128 || !(R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
-    const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
-    const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
+    const int vheads = a.Hkv * (R / 4);            // waves per (split, request)
+    const int waves = (vheads % 4 == 0) ? 4 : ((vheads % 2 == 0) ? 2 : 1);
+    const dim3 grid(a.S, vheads / waves, a.B), block(64 * waves);
     const size_t shm = (size_t)waves * WAVE_LDS;
     if (a.kout == 6)
         hipLaunchKernelGGL(decode_splitkv_mfma_kernel<true>, grid, block, shm, st, a);
