@@ -45,18 +45,23 @@ namespace {
 
 constexpr int D = 128;
 // per-wave LDS map (bytes)
-constexpr int OFF_MAGIC = 0;       // [2 groups][64 pairs] bf16x2: 2^e of channels (p, p+8)
-constexpr int OFF_ZPP = 512;       // same order, bf16 zero points
-constexpr int OFF_KT = 1024;       // [64 tokens][32 B] K code rows
-constexpr int OFF_VT = 3072;       // [8 dword columns][64 tokens] V code dwords
-constexpr int OFF_PT = 5120;       // [4 heads][64 tokens] f16 softmax weights
-constexpr int OFF_VS = 5632;       // [4 channel groups][64 tokens] f16 2^e_v
-constexpr int OFF_VZ = 6144;       // [4 channel groups][64 tokens] f16 v zero points
-constexpr int OFF_DT = 6656;       // [32 tokens][DT_ROW B] f16 outlier deltas of one group
+// Row strides are padded so that the lanes of one access spread over all LDS banks.
+constexpr int KT_ROW = 40;          // bytes per K code row (32 used)
+constexpr int VT_COL = 68;          // dwords per V dword column (64 used)
+constexpr int PT_ROW = 96;          // halfwords per row of the [4][64] f16 arrays (64 used)
+constexpr int OFF_MAGIC = 0;        // [2 groups][64 pairs] bf16x2: 2^e of channels (p, p+8)
+constexpr int OFF_ZPP = 512;        // same order, bf16 zero points
+constexpr int OFF_KT = 1024;        // [64 tokens][KT_ROW] K code rows
+constexpr int OFF_VT = OFF_KT + 64 * KT_ROW;        // [8 dword columns][VT_COL] V code dwords
+constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [4 heads][PT_ROW] f16 softmax weights
+constexpr int OFF_VS = OFF_PT + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 2^e_v
+constexpr int OFF_VZ = OFF_VS + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 v zero points
+constexpr int OFF_DT = OFF_VZ + 4 * PT_ROW * 2;     // [32 tokens][DT_ROW B] f16 outlier deltas of one group
 constexpr int DT_ROW = 272;
-constexpr float BIG_DELTA = 8.0f;   // |outlier delta|/4 from which one f16 is not enough
 constexpr int OFF_LC = OFF_DT + 32 * DT_ROW;        // [64 tokens][4 heads] f32 logit corrections
-constexpr int WAVE_LDS = OFF_LC + 1024;             // 16384
+constexpr int WAVE_LDS = OFF_LC + 1024;             // 17792
+static_assert(OFF_DT % 16 == 0 && OFF_VT % 16 == 0 && OFF_PT % 16 == 0, "b128 alignment");
+constexpr float BIG_DELTA = 8.0f;   // |outlier delta|/4 from which one f16 is not enough
 
 __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
@@ -295,10 +300,10 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         // K code rows (for the outlier pass), transposed V dwords
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
-            *reinterpret_cast<u32x2*>(sm + OFF_KT + (16 * tb + j) * 32 + 8 * kq) = kw[tb];
+            *reinterpret_cast<u32x2*>(sm + OFF_KT + (16 * tb + j) * KT_ROW + 8 * kq) = kw[tb];
             uint32_t* vt = reinterpret_cast<uint32_t*>(sm + OFF_VT);
-            vt[(2 * kq) * 64 + 16 * tb + j] = vw[tb][0];
-            vt[(2 * kq + 1) * 64 + 16 * tb + j] = vw[tb][1];
+            vt[(2 * kq) * VT_COL + 16 * tb + j] = vw[tb][0];
+            vt[(2 * kq + 1) * VT_COL + 16 * tb + j] = vw[tb][1];
         }
         // V scales / zero points of this lane's token as f16, [group][token]
         {
@@ -311,8 +316,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 const uint32_t zb = (g4 & 1) ? (vzp[g4 >> 1] & 0xFFFF0000u) : (vzp[g4 >> 1] << 16);
                 float z = __uint_as_float(zb);
                 if (!tok_ok) { s = 0.0f; z = 0.0f; }
-                vs16[g4 * 64 + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(s));
-                vz16[g4 * 64 + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
+                vs16[g4 * PT_ROW + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(s));
+                vz16[g4 * PT_ROW + lane] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(z));
             }
         }
         // per-channel 2^e and zp in pair order
@@ -366,7 +371,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
                         const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
                         // code dword of channel c in a K row, and the mask that clears its 2 bits
-                        uint32_t* kt = reinterpret_cast<uint32_t*>(sm + OFF_KT + g * 1024) + (c >> 4);
+                        uint32_t* kt = reinterpret_cast<uint32_t*>(sm + OFF_KT + g * 32 * KT_ROW) + (c >> 4);
                         const uint32_t keep = ~(3u << (2 * (c & 15)));
                         uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
                         float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 128;
@@ -378,7 +383,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                             const _Float16 hi = static_cast<_Float16>(dl);
                             if constexpr (!decltype(RES)::value) {
                                 dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
-                                __hip_atomic_fetch_and(kt + pos * 8, keep, __ATOMIC_RELAXED,
+                                __hip_atomic_fetch_and(kt + pos * (KT_ROW / 4), keep, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
                                 dl_max = fmaxf(dl_max, fabsf(dl));
                             } else {
@@ -415,7 +420,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         d = mfma_f16(aq_nat[ks], bt, d);
                     }
                 }
-                const u32x2 kw2 = *reinterpret_cast<const u32x2*>(sm + OFF_KT + (16 * tb + j) * 32 + 8 * kq);
+                const u32x2 kw2 = *reinterpret_cast<const u32x2*>(sm + OFF_KT + (16 * tb + j) * KT_ROW + 8 * kq);
                 const uint32_t w0 = kw2[0], w1 = kw2[1];
                 d = mfma_bf16(aq_pair[0], u32x4{k_pair<0>(w0, m0[0]), k_pair<1>(w0, m0[1]), k_pair<2>(w0, m0[2]), k_pair<3>(w0, m0[3])}, d);
                 d = mfma_bf16(aq_pair[1], u32x4{k_pair<4>(w0, m1[0]), k_pair<5>(w0, m1[1]), k_pair<6>(w0, m1[2]), k_pair<7>(w0, m1[3])}, d);
@@ -473,7 +478,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 const _Float16 ph = static_cast<_Float16>(p[r]);
                 // accumulate the weight that P.V really uses (the f16-rounded one)
                 l_run[r] = l_run[r] * alpha[r] + static_cast<float>(ph);
-                pt[r * 64 + lane] = __builtin_bit_cast(uint16_t, ph);
+                pt[r * PT_ROW + lane] = __builtin_bit_cast(uint16_t, ph);
             }
         }
         // the running maxima seldom move after the first steps: rescale only when one did
@@ -491,16 +496,16 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             const int t0 = 32 * kb + 8 * kq;
-            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & 3) * 64 + t0) * 2);
-            const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * 64 + t0) * 2);
+            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & 3) * PT_ROW + t0) * 2);
+            const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * PT_ROW + t0) * 2);
             const u32x4 apv = {pk_mul_f16(pw[0], sw[0]), pk_mul_f16(pw[1], sw[1]),
                                pk_mul_f16(pw[2], sw[2]), pk_mul_f16(pw[3], sw[3])};
             // columns 0..3: vz of channel group j, columns 4..7: vs; others repeat
             const u32x4 bz = *reinterpret_cast<const u32x4*>(
-                sm + ((j & 4) ? OFF_VS : OFF_VZ) + ((j & 3) * 64 + t0) * 2);
+                sm + ((j & 4) ? OFF_VS : OFF_VZ) + ((j & 3) * PT_ROW + t0) * 2);
             accz = mfma_f16(pw, bz, accz);
             // V codes: dword column j%8, half j/8, tokens t0..t0+7
-            const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (j & 7) * 64 + t0;
+            const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (j & 7) * VT_COL + t0;
             const u32x4 va = *reinterpret_cast<const u32x4*>(vt);
             const u32x4 vb = *reinterpret_cast<const u32x4*>(vt + 4);
             const uint32_t sel = (j & 8) ? 0x07060302u : 0x05040100u;
