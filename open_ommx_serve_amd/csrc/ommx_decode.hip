@@ -14,9 +14,9 @@
 //            exponent field already holds the group's power-of-two scale;
 //            A = 4*q (bf16).  sum A*B = sum q*code*s + 4*sum q*s, the second term and
 //            sum q*zp come out of one small "bias" MFMA per 64 tokens.
-//   outliers a channel-major pass (one lane = two channels) clears the base code of every
-//            outlier position in the staged K rows (LDS and), so that the base term of
-//            such an element is exactly covered by the bias terms, and scatters (outlier - zp)/4 as f16
+//   outliers a channel-major pass (one lane = two channels) overwrites the base code of every
+//            outlier position in the staged K rows by 0 or 3 (ds_mskor_b32), so that the base
+//            term of such an element is known, and scatters (outlier - zp - code*2^e)/4 as f16
 //            into a per-group tile [32 tokens][128 channels] that is consumed as the B
 //            operand of an f16 MFMA against A = 4*q (f16).  Deltas too large for one f16
 //            (|delta/4| >= 4, rare) add their rounding residual times q straight onto the
@@ -158,6 +158,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint8_t* const sm = smem_all + wave * WAVE_LDS;
+    // the same place as an LDS byte address (for LDS instructions issued by hand)
+    const uint32_t sm_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint8_t*)sm));
     const int j = lane & 15, kq = lane >> 4;
     const int Hkv = a.Hkv;
     const int waves = blockDim.x >> 6;
@@ -370,21 +373,30 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
                         const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
                         const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
-                        // code dword of channel c in a K row, and the mask that clears its 2 bits
-                        uint32_t* kt = reinterpret_cast<uint32_t*>(sm + OFF_KT + g * 32 * KT_ROW) + (c >> 4);
-                        const uint32_t keep = ~(3u << (2 * (c & 15)));
+                        // The 2-bit base code of an outlier position is overwritten (in the staged
+                        // K row) by 0 or 3, whichever base value is nearer to the outlier, so the
+                        // delta left for the tile is small; the bias terms account for the rest.
+                        const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
+                        const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                        const float thr = 0.375f * s, s34 = 0.75f * s;
+                        const uint32_t field = 3u << (2 * (c & 15));
+                        const uint32_t kt = sm_lds + OFF_KT + g * 32 * KT_ROW + 4 * (c >> 4);
                         uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
                         float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 128;
 #pragma unroll
                         for (int sidx = 0; sidx < 6; ++sidx) {
                             const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32
                             bm &= bm - 1;
-                            const float dl = fmaf(lv[sidx], a1, b1);
+                            const float dl0 = fmaf(lv[sidx], a1, b1);
+                            const bool top = dl0 > thr;
+                            const float dl = top ? dl0 - s34 : dl0;
                             const _Float16 hi = static_cast<_Float16>(dl);
                             if constexpr (!decltype(RES)::value) {
                                 dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
-                                __hip_atomic_fetch_and(kt + pos * (KT_ROW / 4), keep, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
+                                // K row dword = (dword & ~field) | (top ? field : 0)
+                                asm volatile("ds_mskor_b32 %0, %1, %2"
+                                             :: "v"(kt + pos * KT_ROW), "v"(field), "v"(top ? field : 0u)
+                                             : "memory");
                                 dl_max = fmaxf(dl_max, fabsf(dl));
                             } else {
                                 if (fabsf(dl) >= BIG_DELTA) {
