@@ -20,39 +20,48 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
     constexpr int PER = ROWS / 8;        // tail rows per thread in the P.V step
     constexpr int NSP = MAXS / 8;        // split partials per thread, upper bound
     __shared__ float s_q[D];
-    __shared__ float s_lse[MAXS];
     __shared__ __attribute__((aligned(16))) float s_logit[ROWS];
     __shared__ float s_acc[8][D];        // per-sg sums of the split part
     __shared__ float s_tacc[8][D];       // per-sg sums of the tail part
     __shared__ float s_w[8], s_tl[8], s_wmax[MAXS / 64];
+    __shared__ __attribute__((aligned(16))) float s_wT[8][NSP];   // weight of split sg + 8*i at [sg][i]
     const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int d = tid % D, sg = tid / D;
     const int kvh = h / (a.Hq / a.Hkv);
-    const int L = a.seq[b];
-    const int tail = a.tail ? a.tail[b] : 0;
-    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
     const float* base = a.al + b * a.al_b + (int64_t)h * a.al_h;
 
     // ---- all loads of the split part --------------------------------------------------
-    // (clamped addresses and a uniform trip count keep the loads free of per-lane branches,
-    // so they are all in flight together)
+    // They depend on the arguments only, so they go out before anything is read from
+    // memory; one pointer per thread, advanced by 8 split slots per load.  (A uniform trip
+    // count and a clamped last address keep the loads free of per-lane branches, so they
+    // are all in flight together.)
     float pv[NSP];
     const int n_i = (a.S + 7) >> 3;
+    {
+        const float* p = base + (int64_t)sg * a.al_s + d;
+        const int64_t step = 8 * a.al_s;
 #pragma unroll
-    for (int i = 0; i < NSP; ++i) {
-        pv[i] = 0.0f;
-        if (i < n_i) pv[i] = base[(int64_t)min(sg + 8 * i, a.S - 1) * a.al_s + d];
+        for (int i = 0; i < NSP; ++i) {
+            pv[i] = 0.0f;
+            if (i < n_i) {
+                const bool inside = sg + 8 * i < a.S;          // only the last trip can fall outside
+                pv[i] = *(inside ? p : base + (int64_t)(a.S - 1) * a.al_s + d);
+                p += step;
+            }
+        }
     }
+    const uint32_t q_raw = a.q ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + d] : 0u;
+    const int L = a.seq[b];
+    const int tail = a.tail ? a.tail[b] : 0;
+    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
     float my_lse = -INFINITY;
     if (tid < MAXS) {
         const bool valid = tid < a.S && min(per * tid + per, L) > per * tid;
         if (valid) my_lse = base[(int64_t)tid * a.al_s + D];
     }
-    const uint32_t q_raw = a.q[b * a.q_sb + (int64_t)h * a.q_sh + d];
 
     if (tid < D) s_q[tid] = __uint_as_float(q_raw << 16);
     if (tid < MAXS) {
-        s_lse[tid] = my_lse;
         float wm = my_lse;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) wm = fmaxf(wm, __shfl_xor(wm, o));
@@ -109,24 +118,26 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
         }
         t_m = m_new;
     }
-    __syncthreads();                                  // s_lse ready
+    __syncthreads();                                  // s_wmax ready
 
     // ---- split part: weights from the lse column -----------------------------------------
+    // One thread per split turns its lse into a weight; the weights are laid out so that
+    // thread (d, sg) reads the ones of its splits sg, sg+8, ... as float4.
     float g_max = s_wmax[0];
 #pragma unroll
     for (int w = 1; w < MAXS / 64; ++w) g_max = fmaxf(g_max, s_wmax[w]);
     const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
+    if (tid < MAXS) s_wT[tid & 7][tid >> 3] = my_lse == -INFINITY ? 0.0f : __expf(my_lse - g_safe);
+    __syncthreads();
     float acc = 0.0f, wsum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < NSP; ++i) {
-        const int s = sg + 8 * i;
-        if (s < a.S) {
-            const float ls = s_lse[s];
-            if (ls != -INFINITY) {
-                const float w = __expf(ls - g_safe);
-                wsum += w;
-                acc = fmaf(w, pv[i], acc);
-            }
+    for (int i4 = 0; i4 < NSP / 4; ++i4) {
+        const float4 w4 = reinterpret_cast<const float4*>(s_wT[sg])[i4];
+        const float w[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {          // absent splits have weight zero; their slot
+            wsum += w[k];                      // may hold anything, so it is not multiplied
+            acc = w[k] > 0.0f ? fmaf(w[k], pv[4 * i4 + k], acc) : acc;
         }
     }
     s_acc[sg][d] = acc;
