@@ -9,6 +9,8 @@
 //   V: thread x owns the vector "token x/(D/32), channels 32*(x%(D/32))..+31".
 // The K codes of 4 neighbouring channels share a byte of k_base, so they are transposed
 // through LDS and written as 8-byte pieces of the token-major rows.
+#include <limits.h>
+
 #include "ommx_common.h"
 
 namespace ommx {
@@ -33,6 +35,7 @@ struct StoreArgs {
     uint16_t* v_zp;
     int32_t* err;
     int H, D, ps, kout;
+    int v_vec;              // V rows allow 16-byte loads
 };
 
 template <bool F32>
@@ -60,9 +63,30 @@ __device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict_
     return ((m < 0.0f) ? 8u : 0u) | idx;
 }
 
-template <bool F32>
+// x / 2^e as a multiplication: 2^-e is exact for e in [-126,126] (the product and the
+// quotient are then the same real number, so they round alike, denormal results included).
+__device__ __forceinline__ float div_pow2(float x, float scale, float inv_scale, bool inv_ok) {
+    return inv_ok ? x * inv_scale : __fdiv_rn(x, scale);
+}
+
+// Order-preserving integer image of a bf16 value held as fp32 bits, low 16 bits cleared.
+// -0 must have been turned into +0 before (they tie in the reference's sorts).
+__device__ __forceinline__ int ordered_bits(float x) {
+    const int b = __float_as_int(x);
+    return (b ^ ((b >> 31) & 0x7FFFFFFF)) & static_cast<int>(0xFFFF0000u);
+}
+__device__ __forceinline__ float from_ordered_bits(int k) {
+    const int s = k & static_cast<int>(0xFFFF0000u);
+    // negative images had their low 16 bits set before the clearing; restore them
+    return __int_as_float(s < 0 ? ((s | 0xFFFF) ^ 0x7FFFFFFF) : s);
+}
+__device__ __forceinline__ int med3_i32(int a, int b, int c) {
+    return max(min(a, b), min(max(a, b), c));          // v_med3_i32
+}
+
+template <bool F32, bool FAST6>
 __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
-    extern __shared__ uint8_t smem[];
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int D = a.D;
     uint8_t* s_codes = smem;                       // [32][D] one code per byte
     uint8_t* s_oval = smem + 32 * D;               // [D][4] nibble bytes (3 used at k=6)
@@ -83,34 +107,73 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         for (int i = 0; i < 32; ++i) {
             const int64_t row = a.src_rows ? a.src_rows[g * 32 + i] : (int64_t)g * 32 + i;
             w[i] = load_elem<F32>(a.K, row * a.k_ts + (int64_t)h * a.k_hs + d);
-            fin = fin && is_finite_f32(w[i]);
+            if (!FAST6) fin = fin && is_finite_f32(w[i]);
+        }
+
+        uint32_t top = 0, bot = 0;
+        int key_hi[3] = {0, 0, 0}, key_lo[3] = {0, 0, 0};    // FAST6: sorted keys of the chosen lanes
+        auto select_generic = [&]() {
+            // signed select (pack.py:436-445): kt largest, ties to the lower index ...
+            top = 0;
+            for (int r = 0; r < kt; ++r) {
+                float best = 0.0f; int bi = -1;
+    #pragma unroll
+                for (int i = 0; i < 32; ++i) {
+                    const bool free_lane = !((top >> i) & 1u);
+                    if (free_lane && (bi < 0 || w[i] > best)) { best = w[i]; bi = i; }
+                }
+                if (bi >= 0) top |= 1u << bi;
+            }
+            // ... then kb smallest of the vector with chosen lanes replaced by +1e9.
+            bot = 0;
+            for (int r = 0; r < kb; ++r) {
+                float best = 0.0f; int bi = -1;
+    #pragma unroll
+                for (int i = 0; i < 32; ++i) {
+                    const float v = ((top >> i) & 1u) ? 1e9f : w[i];
+                    const bool free_lane = !((bot >> i) & 1u);
+                    if (free_lane && (bi < 0 || v < best)) { best = v; bi = i; }
+                }
+                if (bi >= 0) bot |= 1u << bi;
+            }
+        };
+        bool fast_done = false;
+        if (FAST6) {
+            // bf16 inputs leave 16 free bits under the value: key = ordered value bits | tie
+            // breaker.  Largest three: tie breaker 31-i with max (equal values: lower index
+            // first, the stable descending sort).  Smallest three: tie breaker i with min.
+            // One pass each through a three-deep max / median network.
+            int t1 = INT_MIN, t2 = INT_MIN, t3 = INT_MIN;
+            int b1 = INT_MAX, b2 = INT_MAX, b3 = INT_MAX;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const int kt_i = ordered_bits(w[i] + 0.0f) | (31 - i);
+                const int kb_i = kt_i ^ 31;
+                const int n3 = med3_i32(t2, t3, kt_i), n2 = med3_i32(t1, t2, kt_i);
+                t1 = max(t1, kt_i); t2 = n2; t3 = n3;
+                const int m3 = med3_i32(b2, b3, kb_i), m2 = med3_i32(b1, b2, kb_i);
+                b1 = min(b1, kb_i); b2 = m2; b3 = m3;
+            }
+            top = (1u << (31 - (t1 & 31))) | (1u << (31 - (t2 & 31))) | (1u << (31 - (t3 & 31)));
+            bot = (1u << (b1 & 31)) | (1u << (b2 & 31)) | (1u << (b3 & 31));
+            key_hi[0] = t1; key_hi[1] = t2; key_hi[2] = t3;
+            key_lo[0] = b1; key_lo[1] = b2; key_lo[2] = b3;
+            // The reference takes the smallest three of the vector with the top lanes moved
+            // to +1e9.  That is the same set unless a top lane is among the overall smallest
+            // three (heavy ties): then redo the selection the slow way.
+            fast_done = (top & bot) == 0u;
+        }
+        if (!fast_done) select_generic();
+        const uint32_t om = top | bot;
+        if (FAST6 && fast_done) {
+            // NaN / Inf sort to the ends of the ordered keys: the largest and the smallest
+            // chosen value tell whether the whole vector is finite
+            fin = is_finite_f32(from_ordered_bits(key_hi[0])) && is_finite_f32(from_ordered_bits(key_lo[0]));
+        } else if (FAST6) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) fin = fin && is_finite_f32(w[i]);
         }
         if (!fin) err |= OMMX_ERR_NONFINITE_K;
-
-        // signed select (pack.py:436-445): kt largest, ties to the lower index ...
-        uint32_t top = 0;
-        for (int r = 0; r < kt; ++r) {
-            float best = 0.0f; int bi = -1;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const bool free_lane = !((top >> i) & 1u);
-                if (free_lane && (bi < 0 || w[i] > best)) { best = w[i]; bi = i; }
-            }
-            if (bi >= 0) top |= 1u << bi;
-        }
-        // ... then kb smallest of the vector with chosen lanes replaced by +1e9.
-        uint32_t bot = 0;
-        for (int r = 0; r < kb; ++r) {
-            float best = 0.0f; int bi = -1;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const float v = ((top >> i) & 1u) ? 1e9f : w[i];
-                const bool free_lane = !((bot >> i) & 1u);
-                if (free_lane && (bi < 0 || v < best)) { best = v; bi = i; }
-            }
-            if (bi >= 0) bot |= 1u << bi;
-        }
-        const uint32_t om = top | bot;
         if (__popc(om) != kout) err |= OMMX_ERR_UNDERFILLED;
 
         // affine base over the non-outlier lanes (pack.py:455-465)
@@ -144,20 +207,42 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             ms = bf16_to_f32(ms_b);
         }
 
+        const bool inv_ok = e >= -126 && e <= 126;
+        const float inv_scale = exp2_int(inv_ok ? -e : 0);
         uint32_t nib = 0;
-        int slot = 0;
         bool mfin = true;
+        if (FAST6 && fast_done) {
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            float c = rintf(__fdiv_rn(w[i] - zp, scale));
-            c = fminf(fmaxf(c, 0.0f), 3.0f);
-            s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
-            if (kout > 0) {
-                const float mapped = (w[i] - mc) * ms;
+            for (int i = 0; i < 32; ++i) {
+                float c = rintf(div_pow2(w[i] - zp, scale, inv_scale, inv_ok));
+                c = fminf(fmaxf(c, 0.0f), 3.0f);
+                s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
+            }
+            // |(w - mc) * ms| is largest at the extreme lanes, which are outliers: they decide
+            // whether every mapped value is finite (codec.py:55-57 checks all of them)
+#pragma unroll
+            for (int r = 0; r < 6; ++r) {
+                const int key = r < 3 ? key_hi[r] : key_lo[r - 3];
+                const int pos = r < 3 ? 31 - (key & 31) : (key & 31);
+                const float mapped = (from_ordered_bits(key) - mc) * ms;
                 mfin = mfin && is_finite_f32(mapped);
-                if ((om >> i) & 1u) {
-                    nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
-                    ++slot;
+                const int slot = __popc(om & ((1u << pos) - 1u));
+                nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
+            }
+        } else {
+            int slot = 0;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                float c = rintf(div_pow2(w[i] - zp, scale, inv_scale, inv_ok));
+                c = fminf(fmaxf(c, 0.0f), 3.0f);
+                s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
+                if (kout > 0) {
+                    const float mapped = (w[i] - mc) * ms;
+                    mfin = mfin && is_finite_f32(mapped);
+                    if ((om >> i) & 1u) {
+                        nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
+                        ++slot;
+                    }
                 }
             }
         }
@@ -190,20 +275,46 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const int64_t page = a.dst_pages ? a.dst_pages[lp] : lp;
         const int64_t prow = page * a.ps + (tok % a.ps);  // physical token row
 
+        // 32 code bytes -> 64 bits: four codes of a dword fold into its low byte
         uint64_t kb8 = 0;
-        const uint8_t* cr = s_codes + t * D + 32 * j;
+        const uint4* cr = reinterpret_cast<const uint4*>(s_codes + t * D + 32 * j);
 #pragma unroll
-        for (int c = 0; c < 32; ++c) kb8 |= static_cast<uint64_t>(cr[c] & 3u) << (2 * c);
+        for (int q4 = 0; q4 < 2; ++q4) {
+            const uint4 u = cr[q4];
+            const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uint32_t x = uw[k] & 0x03030303u;
+                x |= x >> 6;
+                x |= x >> 12;
+                kb8 |= static_cast<uint64_t>(x & 0xFFu) << (8 * (4 * q4 + k));
+            }
+        }
         reinterpret_cast<uint64_t*>(a.k_base)[(prow * a.H + h) * NGV + j] = kb8;
 
         const int64_t row = a.src_rows ? a.src_rows[tok] : tok;
         const int64_t vbase = row * a.v_ts + (int64_t)h * a.v_hs + 32 * j;
         float v[32];
+        if (!F32 && a.v_vec) {                    // 64 contiguous bytes: four 16-byte loads
+            const uint4* vp = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.V) + vbase);
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const uint4 u = vp[q4];
+                const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v[8 * q4 + 2 * k] = __uint_as_float(uw[k] << 16);
+                    v[8 * q4 + 2 * k + 1] = __uint_as_float(uw[k] & 0xFFFF0000u);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 32; ++c) v[c] = load_elem<F32>(a.V, vbase + c);
+        }
         bool fin = true;
         float mn = 0.0f, mx = 0.0f;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
-            v[c] = load_elem<F32>(a.V, vbase + c);
             fin = fin && is_finite_f32(v[c]);
             mn = c == 0 ? v[c] : fminf(mn, v[c]);
             mx = c == 0 ? v[c] : fmaxf(mx, v[c]);
@@ -215,10 +326,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const float scale = exp2_int(e);
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
+        const bool inv_ok = e >= -126 && e <= 126;
+        const float inv_scale = exp2_int(inv_ok ? -e : 0);
         uint64_t vb8 = 0;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
-            float q = rintf(__fdiv_rn(v[c] - zp, scale));
+            float q = rintf(div_pow2(v[c] - zp, scale, inv_scale, inv_ok));
             q = fminf(fmaxf(q, 0.0f), 3.0f);
             vb8 |= static_cast<uint64_t>(static_cast<int>(q)) << (2 * c);
         }
@@ -283,14 +396,17 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
     if (T == 0) return 0;
     StoreArgs a{K, V, k_ts, k_hs, v_ts, v_hs, src_rows, dst_pages, dst_groups, table,
                 k_base, k_scale, k_zp, k_ms, k_mc, k_obmp, k_oval, v_main, v_scale, v_zp,
-                err_flag, H, D, page_size, k_outliers};
+                err_flag, H, D, page_size, k_outliers,
+                (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0};
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (in_dtype == 1)
-        hipLaunchKernelGGL(store_pack_kernel<true>, grid, block, shm, st, a);
+        hipLaunchKernelGGL((store_pack_kernel<true, false>), grid, block, shm, st, a);
+    else if (k_outliers == 6)
+        hipLaunchKernelGGL((store_pack_kernel<false, true>), grid, block, shm, st, a);
     else
-        hipLaunchKernelGGL(store_pack_kernel<false>, grid, block, shm, st, a);
+        hipLaunchKernelGGL((store_pack_kernel<false, false>), grid, block, shm, st, a);
     if (hipGetLastError() != hipSuccess) { set_error("ommx_store_pack: launch failed"); return -2; }
     return 0;
 }
