@@ -354,10 +354,10 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             if (OUTLIERS) {
                 // RES = false: the walk every group takes.  RES = true: a second walk that only
                 // adds f16 rounding residuals of large deltas onto the logits.
-                float dl_max = 0.0f;
-                auto walk = [&](auto RES) {
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) {
+                float dl_max[2] = {0.0f, 0.0f};
+                auto walk = [&](auto RES, auto U) {
+                    constexpr int u = decltype(U)::value;
+                    {
                         const int c = 2 * lane + u;
                         const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
                         const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
@@ -397,7 +397,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                                 asm volatile("ds_mskor_b32 %0, %1, %2"
                                              :: "v"(kt + pos * KT_ROW), "v"(field), "v"(top ? field : 0u)
                                              : "memory");
-                                dl_max = fmaxf(dl_max, fabsf(dl));
+                                dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
                             } else {
                                 if (fabsf(dl) >= BIG_DELTA) {
                                     const float lo = dl - static_cast<float>(hi);
@@ -410,12 +410,14 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         }
                     }
                 };
-                walk(std::false_type{});
+                walk(std::false_type{}, std::integral_constant<int, 0>{});
+                walk(std::false_type{}, std::integral_constant<int, 1>{});
                 // One f16 carries 11 bits: below |delta/4| = 4 its rounding error is at most
                 // 2^-10 (4e-3 in K units; times |q| * sm_scale that stays under 1.5e-3 on a
                 // logit for |q| <= 4, inside the output tolerance even for a two-token context).
-                // Groups holding a larger delta (rare) take the residual walk.
-                if (__any(dl_max >= BIG_DELTA)) walk(std::true_type{});
+                // Channel halves holding a larger delta take the residual walk.
+                if (__any(dl_max[0] >= BIG_DELTA)) walk(std::true_type{}, std::integral_constant<int, 0>{});
+                if (__any(dl_max[1] >= BIG_DELTA)) walk(std::true_type{}, std::integral_constant<int, 1>{});
                 lds_fence();
             }
             const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + g * 256 + kq * 64);
