@@ -61,7 +61,10 @@ constexpr int DT_ROW = 272;
 constexpr int OFF_LC = OFF_DT + 32 * DT_ROW;        // [64 tokens][4 heads] f32 logit corrections
 constexpr int WAVE_LDS = OFF_LC + 1024;             // 17792
 static_assert(OFF_DT % 16 == 0 && OFF_VT % 16 == 0 && OFF_PT % 16 == 0, "b128 alignment");
-constexpr float BIG_DELTA = 4.0f;   // |outlier delta|/4 from which one f16 is not enough
+// One f16 carries 11 bits.  An outlier delta d (in units of 4) whose f16 rounding error times
+// the largest |4q| of its channel could move a logit by more than ~1.5e-3 gets its residual
+// added exactly; the bound is |d| * max|4q| >= BIG_DELTA * 16, i.e. |d| >= 4 at |q| = 4.
+constexpr float BIG_DELTA = 4.0f;
 
 __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
@@ -293,6 +296,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             q4[1][r] = 4.0f * __uint_as_float(w & 0xFFFF0000u);
         }
     }
+    // per channel: the |delta/4| from which the residual matters (infinite for q = 0)
+    float big_thr[2] = {0.0f, 0.0f};
+    if (OUTLIERS) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const float qm = fmaxf(fmaxf(fabsf(q4[u][0]), fabsf(q4[u][1])), fmaxf(fabsf(q4[u][2]), fabsf(q4[u][3])));
+            big_thr[u] = (BIG_DELTA * 16.0f) * __builtin_amdgcn_rcpf(qm);
+        }
+    }
 
 
     for (int n0 = n_begin; n0 < n_end; n0 += 64) {
@@ -399,7 +411,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                                              : "memory");
                                 dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
                             } else {
-                                if (fabsf(dl) >= BIG_DELTA) {
+                                if (fabsf(dl) >= big_thr[u]) {
                                     const float lo = dl - static_cast<float>(hi);
 #pragma unroll
                                     for (int r = 0; r < 4; ++r)
@@ -412,12 +424,10 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 };
                 walk(std::false_type{}, std::integral_constant<int, 0>{});
                 walk(std::false_type{}, std::integral_constant<int, 1>{});
-                // One f16 carries 11 bits: below |delta/4| = 4 its rounding error is at most
-                // 2^-10 (4e-3 in K units; times |q| * sm_scale that stays under 1.5e-3 on a
-                // logit for |q| <= 4, inside the output tolerance even for a two-token context).
+                // (see BIG_DELTA)
                 // Channel halves holding a larger delta take the residual walk.
-                if (__any(dl_max[0] >= BIG_DELTA)) walk(std::true_type{}, std::integral_constant<int, 0>{});
-                if (__any(dl_max[1] >= BIG_DELTA)) walk(std::true_type{}, std::integral_constant<int, 1>{});
+                if (__any(dl_max[0] >= big_thr[0])) walk(std::true_type{}, std::integral_constant<int, 0>{});
+                if (__any(dl_max[1] >= big_thr[1])) walk(std::true_type{}, std::integral_constant<int, 1>{});
                 lds_fence();
             }
             const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + g * 256 + kq * 64);
