@@ -202,6 +202,22 @@ int ommx_tail_gather(const uint16_t* k_hist, const uint16_t* v_hist, int64_t his
                      int B, int T, int H, int D, int sink_rows, int recent_rows, int group_tokens,
                      int ring_span, int32_t* err_flag, void* stream);
 
+/*
+ * Merge of partial attention states over disjoint KV segments (cascade / context-parallel /
+ * chunked composition).  Replaces merge_attention_states,
+ * ommx_gpu_serve/attention/paged_decode.py:3556-3624 (kernel :2650-2690).
+ *   o_parts    f32 [P,R,D] with strides op_stride_p / op_stride_r (D contiguous)
+ *   lse_parts  f32 [P,R] with stride lp_stride_p (R contiguous)
+ *   valid_lens NULL, or int32[R]: row r uses its first valid_lens[r] parts (negative = all)
+ *   o          f32 [R,D] row stride o_stride_r;  lse f32 [R]
+ * m = max lse_p, w_p = exp(lse_p - m), o = sum w_p o_p / sum w_p, lse = m + ln sum w_p;
+ * a part with lse = -inf weighs nothing; no attended part gives o = 0, lse = -inf.
+ */
+int ommx_merge_states(const float* o_parts, const float* lse_parts, const int32_t* valid_lens,
+                      float* o, float* lse, int P, int R, int D,
+                      int64_t op_stride_p, int64_t op_stride_r, int64_t lp_stride_p,
+                      int64_t o_stride_r, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,7 +8,7 @@ from .kv_store_ops import gather_tail, gather_tails, ring_slot, write_token, wri
 from .kv_window import WindowSpec, packed_boundary, tail_token_indices
 from .pack import (CANONICAL_GROUP_CHANNELS, CANONICAL_GROUP_TOKENS, alloc_planes,
                    ommx_pack_kv_canonical_block, store_pack_into)
-from .paged_decode import (auto_num_kv_splits, make_attn_logits,
+from .paged_decode import (auto_num_kv_splits, make_attn_logits, merge_attention_states,
                            ommx_paged_decode_attention_canonical)
 
 __all__ = [
@@ -16,5 +16,5 @@ __all__ = [
     "alloc_planes", "auto_num_kv_splits", "make_attn_logits", "WindowSpec", "packed_boundary",
     "tail_token_indices", "CANONICAL_GROUP_TOKENS", "CANONICAL_GROUP_CHANNELS",
     "MultiSeqKVPool", "CanonicalKVStore", "write_token", "write_tokens", "gather_tail",
-    "gather_tails", "ring_slot",
+    "gather_tails", "ring_slot", "merge_attention_states",
 ]

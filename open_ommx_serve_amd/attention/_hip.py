@@ -43,6 +43,7 @@ _SIGNATURES = {
                                  _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _F, _F, _P]),
     "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
                              _I, _I, _I, _I, _I, _P, _P]),
+    "ommx_merge_states": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P]),
     "ommx_tail_gather": (_I, [_P, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P,
                               _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
 }

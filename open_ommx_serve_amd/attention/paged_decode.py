@@ -169,7 +169,7 @@ def ommx_paged_decode_attention_canonical(
         raise ValueError("req_to_token / req_to_group must both be int32 or both int64")
     if req_to_token.stride(-1) != 1 or req_to_group.stride(-1) != 1:
         raise ValueError("page / group tables must be contiguous along their last axis")
-    if b_seq_len.dtype != torch.int32 or b_tail_len.dtype != torch.int32:
+    if b_seq_len.dtype != torch.int32 or (b_tail_len is not None and b_tail_len.dtype != torch.int32):
         raise ValueError("b_seq_len / b_tail_len must be int32")
     if o.dtype != torch.float32 or lse.dtype != torch.float32 or o.stride(-1) != 1 or lse.stride(-1) != 1:
         raise ValueError("o / lse must be fp32 with unit inner stride")
@@ -190,7 +190,8 @@ def ommx_paged_decode_attention_canonical(
                 or int(attn_logits.shape[3]) < D + 1 or attn_logits.stride(-1) != 1:
             raise ValueError(f"attn_logits must be fp32 [B={B}, Hq={Hq}, >= {S}, >= {D + 1}] "
                              f"with unit inner stride; got {tuple(attn_logits.shape)}")
-    has_tail = gbase == 0 and k_tail is not None and int(k_tail.shape[1]) > 0 \
+    has_tail = gbase == 0 and k_tail is not None and v_tail is not None and b_tail_len is not None \
+        and int(k_tail.shape[1]) > 0 \
         and (max_tail_len is None or int(max_tail_len) > 0)
     if has_tail:
         if k_tail.dtype != torch.bfloat16 or v_tail.dtype != torch.bfloat16 \
@@ -226,4 +227,53 @@ def ommx_paged_decode_attention_canonical(
         _hip.check(rc, "ommx_decode_combine")
 
 
-__all__ = ["ommx_paged_decode_attention_canonical", "auto_num_kv_splits", "make_attn_logits"]
+def merge_attention_states(o_parts: torch.Tensor, lse_parts: torch.Tensor, *, valid_lens=None,
+                           out=None, lse_out=None):
+    """Merge ``P`` partial attention states of the same query rows, computed over disjoint KV
+    segments, into the state over their union (reference ``paged_decode.py:3556-3624``):
+    ``m = max lse_p; w_p = exp(lse_p - m); o = sum w_p o_p / sum w_p; lse = m + log sum w_p``.
+
+    ``o_parts [P, R, D]``, ``lse_parts [P, R]``; ``valid_lens [R]`` (optional) is the number of
+    leading parts each row uses.  Returns ``(o [R, D] in o_parts' dtype, lse [R] fp32)``;
+    ``out`` / ``lse_out`` are written in place when given.  One HIP launch, fp32 arithmetic.
+    """
+    if o_parts.dim() != 3:
+        raise ValueError(
+            f"o_parts must be [P, R, D]; got shape {tuple(o_parts.shape)}. "
+            "Reshape any [P, ..., D] structure to a flat row axis R first.")
+    if lse_parts.dim() != 2 or tuple(lse_parts.shape) != tuple(o_parts.shape[:2]):
+        raise ValueError(
+            f"lse_parts must be [P, R] matching o_parts[:2]; got "
+            f"{tuple(lse_parts.shape)} vs {tuple(o_parts.shape[:2])}.")
+    P, R, D = (int(x) for x in o_parts.shape)
+    dev = o_parts.device
+    if valid_lens is not None and int(valid_lens.numel()) != R:
+        raise ValueError(f"valid_lens must have R={R} entries; got {valid_lens.numel()}.")
+    _hip.require_gpu(dev)
+    op = o_parts if (o_parts.dtype == torch.float32 and o_parts.stride(-1) == 1) \
+        else o_parts.to(torch.float32).contiguous()
+    lp = lse_parts if (lse_parts.dtype == torch.float32 and lse_parts.stride(-1) == 1
+                       and lse_parts.device == dev) else lse_parts.to(dev, torch.float32).contiguous()
+    valid = None if valid_lens is None else valid_lens.to(device=dev, dtype=torch.int32).contiguous()
+    if out is None:
+        out = torch.empty(R, D, dtype=o_parts.dtype, device=dev)
+    if lse_out is None:
+        lse_out = torch.empty(R, dtype=torch.float32, device=dev)
+    direct = out.dtype == torch.float32 and out.stride(-1) == 1 and lse_out.dtype == torch.float32 \
+        and lse_out.is_contiguous()
+    o32 = out if direct else torch.empty(R, D, dtype=torch.float32, device=dev)
+    l32 = lse_out if direct else torch.empty(R, dtype=torch.float32, device=dev)
+    lib = _hip.load()
+    with torch.cuda.device(dev):
+        _hip.check(lib.ommx_merge_states(
+            op.data_ptr(), lp.data_ptr(), _hip.ptr(valid), o32.data_ptr(), l32.data_ptr(),
+            P, R, D, op.stride(0), op.stride(1), lp.stride(0), o32.stride(0),
+            _hip.current_stream_ptr(dev)), "ommx_merge_states")
+    if not direct:
+        out.copy_(o32)
+        lse_out.copy_(l32)
+    return out, lse_out
+
+
+__all__ = ["ommx_paged_decode_attention_canonical", "merge_attention_states", "auto_num_kv_splits",
+           "make_attn_logits"]
