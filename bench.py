@@ -85,7 +85,7 @@ def _make_runner(case, splits=None):
     dev = case.q.device
     kw = case.decode_kwargs()
     n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
-    S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu)
+    S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu, Hq // case.kv_heads)
     ws = make_attn_logits(B, Hq, S, D, dev)
     o = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
