@@ -9,11 +9,12 @@
 //
 // Arithmetic.  All dot products run on the matrix pipe (v_mfma_f32_16x16x32, fp32
 // accumulate) with operands that are EXACT in their 16-bit type:
-//   K base   B = (1 + code/4) * 2^e   bf16, built with one shift and one and-or per channel
-//            pair: the 2-bit code lands in the two top mantissa bits of a bf16 whose
-//            exponent field already holds the group's power-of-two scale;
-//            A = 4*q (bf16).  sum A*B = sum q*code*s + 4*sum q*s, the second term and
-//            sum q*zp come out of one small "bias" MFMA per 64 tokens.
+//   K base   B = (1 + code*2^(2k-7)) * 2^e   bf16, built with one and-or per channel pair (and
+//            a shift shared by two pairs): the 2-bit code lands at mantissa bits [2k+1:2k]
+//            (k = 1 or 2, fixed per pair) of a bf16 whose exponent field already holds the
+//            group's power-of-two scale; A = q * 2^(7-2k) (bf16, exact).
+//            sum A*B = sum q*code*s + sum A*s; the second term and sum q*zp come out of one
+//            small "bias" MFMA per 64 tokens.
 //   outliers a channel-major pass (one lane = two channels) overwrites the base code of every
 //            outlier position in the staged K rows by 0 or 3 (ds_mskor_b32), so that the base
 //            term of such an element is known, and scatters (outlier - zp - code*2^e)/4 as f16
@@ -21,8 +22,8 @@
 //            operand of an f16 MFMA against A = 4*q (f16).  Deltas too large for one f16
 //            (|delta/4| >= 4, rare) add their rounding residual times q straight onto the
 //            logits through LDS float atomics.
-//   P.V      B = (1 + code/4) f16 for 8 tokens of one channel (V rows are transposed
-//            through LDS at dword granularity), A = p * 2^e_v (f16, exact scaling);
+//   P.V      B = (1 + code/4) or (1 + code/16) f16 for 8 tokens of one channel (V rows are
+//            transposed through LDS at dword granularity), A = p * 2^e_v (f16, exact scaling);
 //            sum_t p*vs and sum_t p*vz come from one extra MFMA per 32 tokens.
 // MFMA row groups are used as selectors: rows 4x..4x+3 carry the 4 q heads for token
 // block x (QK) or for V channel group x (P.V); a lane keeps the row group that matches
@@ -141,19 +142,24 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// K pair p of a code dword: channels p (low half) and p+8 (high half) as bf16 (1+c/4)*2^e.
+// K pair p of a code dword: channels p (low half) and p+8 (high half) as bf16.  The 2-bit code
+// may sit anywhere in the mantissa: at bits [2k+1:2k] the element reads (1 + c*2^(2k-7))*2^e, and
+// the matching A operand carries q*2^(7-2k), so the product is still q*c*2^e plus a constant
+// that the bias MFMA removes.  Using two positions (k = 1, 2) lets neighbouring pairs share a
+// shift, or need none.
+__host__ __device__ constexpr int k_class(int p) { return (p == 2 || p == 4 || p == 6) ? 2 : 1; }
 template <int P>
 __device__ __forceinline__ uint32_t k_pair(uint32_t w, uint32_t magic) {
-    const uint32_t sh = (2 * P >= 5) ? (w >> (2 * P - 5 < 0 ? 0 : 2 * P - 5))
-                                     : (w << (5 - 2 * P < 0 ? 0 : 5 - 2 * P));
-    return (sh & 0x00600060u) | magic;
+    const uint32_t sh = P == 0 ? (w << 2) : P <= 2 ? w : P <= 4 ? (w >> 4) : P <= 6 ? (w >> 8) : (w >> 12);
+    return (sh & (k_class(P) == 1 ? 0x000C000Cu : 0x00300030u)) | magic;
 }
-// V channel y of a merged dword (token a in the low 16 bits, token b in the high 16 bits).
+// V channel y of a merged dword (token a in the low 16 bits, token b in the high 16 bits) as
+// f16 1 + c/16 (even y, code at mantissa bits [7:6]) or 1 + c/4 (odd y, bits [9:8]); channels
+// y and y+1 share their shift.
 template <int Y>
 __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
-    const uint32_t sh = (2 * Y >= 8) ? (m >> (2 * Y - 8 < 0 ? 0 : 2 * Y - 8))
-                                     : (m << (8 - 2 * Y < 0 ? 0 : 8 - 2 * Y));
-    return (sh & 0x03000300u) | one_f16x2;      // one v_and_or_b32 when the constant is a VGPR
+    const uint32_t sh = Y <= 1 ? (m << 6) : Y <= 3 ? (m << 2) : Y <= 5 ? (m >> 2) : (m >> 6);
+    return (sh & ((Y & 1) ? 0x03000300u : 0x00C000C0u)) | one_f16x2;
 }
 
 template <bool OUTLIERS>
@@ -266,7 +272,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         fetch_tables(n_begin + 64);
     }
 
-    // ---- A operands: 4*q of head j%4 for this lane's 32-channel quarter ---------------
+    // ---- A operands: scaled q of head j%4 for this lane's 32-channel quarter ------------
+    // (pair order: q * 2^(7-2k) with k the code position of the pair, see k_pair; natural
+    // order: 4*q)
     // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
     // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
     u32x4 aq_pair[4], aq_nat[4];
@@ -277,7 +285,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
-                const float lo = 4.0f * bf16_to_f32(qh[cl]), hi = 4.0f * bf16_to_f32(qh[cl + 8]);
+                const float qs = k_class(4 * (ks & 1) + rr) == 1 ? 32.0f : 8.0f;    // 2^(7-2k)
+                const float lo = qs * bf16_to_f32(qh[cl]), hi = qs * bf16_to_f32(qh[cl + 8]);
                 aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
                 const float n0 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr]);
                 const float n1 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr + 1]);
@@ -348,7 +357,12 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                     const int hw = (((c >> 4) * 8) + (y & 7)) * 2 + (y >> 3);
                     const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
                     mg[g * 128 + hw] = static_cast<uint16_t>((e + 127) << 7);
-                    zp[g * 128 + hw] = static_cast<uint16_t>(u ? (g_zp[g] >> 16) : (g_zp[g] & 0xFFFFu));
+                    // zero point divided by the channel's A scale 2^(7-2k), so that the bias
+                    // MFMA returns sum q*zp (exact: a shift of the exponent field)
+                    const uint32_t zb = u ? (g_zp[g] >> 16) : (g_zp[g] & 0xFFFFu);
+                    const uint32_t zsh = k_class(y & 7) == 1 ? 5u : 3u;
+                    zp[g * 128 + hw] = static_cast<uint16_t>(
+                        ((zb >> 7) & 0xFFu) > zsh ? zb - (zsh << 7) : (zb & 0x8000u));
                 }
             }
         }
@@ -470,7 +484,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         }
 
         // ---------------------------------------------------------------- softmax
-        // bias of (group, head r): 0.25*ZP' - S1' ; columns 0..3 live in lanes 0..3 (kq 0)
+        // bias of (group, head r): sum q*zp - sum A*2^e ; columns 0..3 live in lanes 0..3 (kq 0)
         float logit[4];
         {
             const f32x4 dsel = kq == 0 ? dq[0] : (kq == 1 ? dq[1] : (kq == 2 ? dq[2] : dq[3]));
@@ -481,7 +495,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             for (int r = 0; r < 4; ++r) {
                 const float zpv = __shfl(dbias[r], gsel);          // column gsel, rows 0..3
                 const float s1v = __shfl(dbias[r], 2 + gsel);
-                const float raw = dsel[r] + corr[r] + (0.25f * zpv - s1v);
+                const float raw = dsel[r] + corr[r] + (zpv - s1v);
                 float x = raw * a.sm_scale;
                 x = apply_cap(x, a.cap) * c_log2e;
                 logit[r] = tok_ok ? x : -INFINITY;
@@ -545,7 +559,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         lds_fence();
     }
 
-    // ---- epilogue: o = (4*(acc - PVS) + PVZ) / l, lse = m + ln l -------------------------
+    // ---- epilogue: o = (f*(acc - PVS) + PVZ) / l with f = 4 or 16, lse = m + ln l ----------
     float l_tot[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) l_tot[r] = wave_sum(l_run[r]);
@@ -564,7 +578,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
 #pragma unroll
             for (int y = 0; y < 8; ++y)
-                dst[ch0 + y] = (4.0f * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
+                dst[ch0 + y] = (((y & 1) ? 4.0f : 16.0f) * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
         }
     }
     if (lane < 4) {
