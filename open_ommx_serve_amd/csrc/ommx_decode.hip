@@ -249,9 +249,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // channel pair (2*lane, 2*lane+1) parameters of both groups
     uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
     u32x2 g_bm[2], g_ov[2];
-    auto fetch_params = [&]() {
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
+    auto fetch_params_g = [&](int g) {
+        {
             const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);   // same for every lane
             const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + (uint32_t)kvh) * D;
             g_sc[g] = *reinterpret_cast<const uint16_t*>(a.k_scale + gidx + 2 * lane);
@@ -265,6 +264,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             }
         }
     };
+    auto fetch_params = [&]() { fetch_params_g(0); fetch_params_g(1); };
     if (n_begin < n_end) {
         fetch_tables(n_begin);
         fetch_kv();
@@ -444,6 +444,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 if (__any(dl_max[1] >= big_thr[1])) walk(std::true_type{}, std::integral_constant<int, 1>{});
                 lds_fence();
             }
+            // this group's parameter registers are free: start the next iteration's loads
+            if (more) fetch_params_g(g);
             const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAGIC + g * 256 + kq * 64);
             const u32x4 m0 = mg[0], m1 = mg[1], m2 = mg[2], m3 = mg[3];
 #pragma unroll
@@ -478,10 +480,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             for (int ks = 0; ks < 4; ++ks) dbias = mfma_bf16(aq_pair[ks], bp[ks], dbias);
         }
 
-        if (more) {                        // group parameters and the tables after them
-            fetch_params();
-            fetch_tables(n0 + 128);
-        }
+        if (more) fetch_tables(n0 + 128);  // after the parameter loads, which used the group slots
 
         // ---------------------------------------------------------------- softmax
         // bias of (group, head r): sum q*zp - sum A*2^e ; columns 0..3 live in lanes 0..3 (kq 0)
