@@ -319,6 +319,16 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     for (int n0 = n_begin; n0 < n_end; n0 += 64) {
         const bool tok_ok = n0 + lane < n_end;
         const bool more = n0 + 64 < n_end;
+        // Waves that share a SIMD should finish together (a wave running alone leaves issue
+        // slots empty), but the arbiter favours the older wave: give the wave with more work
+        // left the higher priority.
+        {
+            const int left = (n_end - n0 + 63) >> 6;
+            if (left >= 4) __builtin_amdgcn_s_setprio(3);
+            else if (left == 3) __builtin_amdgcn_s_setprio(2);
+            else if (left == 2) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
 
         // ---------------------------------------------------------------- stage to LDS
         // K code rows (for the outlier pass), transposed V dwords
