@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the split-KV kernel at the default workload (ctx 65536, 255
 # splits), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
 # (profiles/decode_ctx64k_hbm_traffic.txt); counters cannot be read from inside this script.
-TRAFFIC_BYTES_CTX64K = 80.36e6
+TRAFFIC_BYTES_CTX64K = 74.03e6
 STAGE1_REP = 20
 LAYERS = 32                  # decode steps (layers) per graph replay
 H200_P50_US_64K = 563.0      # reference Triton kernel, H200 NVL, B=1 ctx 65536 (other hardware)
