@@ -136,10 +136,41 @@ __device__ __forceinline__ void wave_max4(float (&v)[4]) {
 __device__ __forceinline__ int table_lo(const void* t, int64_t i, int sh) {
     return *reinterpret_cast<const int*>(static_cast<const char*>(t) + (i << sh));
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+// Sums of four values over the 64 lanes (results uniform); same interleaving as wave_max4.
+__device__ __forceinline__ void wave_sum4(float (&v)[4]) {
+    float a = v[0], b = v[1], c = v[2], d = v[3];
+    asm volatile(
+        "s_nop 1\n"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_add_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_add_f32_dpp %2, %2, %2 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_add_f32_dpp %3, %3, %3 row_bcast:15 row_mask:0xa bank_mask:0xf\n"
+        "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_add_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_add_f32_dpp %2, %2, %2 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "v_add_f32_dpp %3, %3, %3 row_bcast:31 row_mask:0xc bank_mask:0xf\n"
+        "s_nop 1\n"
+        : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    v[0] = readlane_f32(a, 63);
+    v[1] = readlane_f32(b, 63);
+    v[2] = readlane_f32(c, 63);
+    v[3] = readlane_f32(d, 63);
 }
 
 // K pair p of a code dword: channels p (low half) and p+8 (high half) as bf16.  The 2-bit code
@@ -279,18 +310,24 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
     u32x4 aq_pair[4], aq_nat[4];
     {
-        const uint16_t* qh = a.q + b * a.q_sb + (int64_t)(qh0 + (j & 3)) * a.q_sh + 32 * kq;
+        // this lane's 32 channels of q: 16 dwords, channel 2i in the low half of dword i
+        const uint32_t* qh = reinterpret_cast<const uint32_t*>(
+            a.q + b * a.q_sb + (int64_t)(qh0 + (j & 3)) * a.q_sh + 32 * kq);
+        uint32_t qw[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) qw[i] = qh[i];
+        auto q_at = [&](int c) {          // channel c of the quarter as fp32 (exact)
+            return __uint_as_float((c & 1) ? (qw[c >> 1] & 0xFFFF0000u) : (qw[c >> 1] << 16));
+        };
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
                 const float qs = k_class(4 * (ks & 1) + rr) == 1 ? 32.0f : 8.0f;    // 2^(7-2k)
-                const float lo = qs * bf16_to_f32(qh[cl]), hi = qs * bf16_to_f32(qh[cl + 8]);
+                const float lo = qs * q_at(cl), hi = qs * q_at(cl + 8);
                 aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
-                const float n0 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr]);
-                const float n1 = 4.0f * bf16_to_f32(qh[8 * ks + 2 * rr + 1]);
-                aq_nat[ks][rr] = pack_f16x2(n0, n1);
+                aq_nat[ks][rr] = pack_f16x2(4.0f * q_at(8 * ks + 2 * rr), 4.0f * q_at(8 * ks + 2 * rr + 1));
             }
         }
     }
@@ -569,9 +606,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     }
 
     // ---- epilogue: o = (f*(acc - PVS) + PVZ) / l with f = 4 or 16, lse = m + ln l ----------
-    float l_tot[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) l_tot[r] = wave_sum(l_run[r]);
+    float l_tot[4] = {l_run[0], l_run[1], l_run[2], l_run[3]};
+    wave_sum4(l_tot);
     const int jg = (j & 7) >> 1;
     float pvz[4], pvs[4];
 #pragma unroll
