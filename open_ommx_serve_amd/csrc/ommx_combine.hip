@@ -29,6 +29,9 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
     const int d = tid % D, sg = tid / D;
     const int kvh = h / (a.Hq / a.Hkv);
     const float* base = a.al + b * a.al_b + (int64_t)h * a.al_h;
+    // the two scalars that everything after the split loads waits for: requested first
+    const int L = a.seq[b];
+    const int tail = a.tail ? a.tail[b] : 0;
 
     // ---- all loads of the split part --------------------------------------------------
     // They depend on the arguments only, so they go out before anything is read from
@@ -51,8 +54,6 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
         }
     }
     const uint32_t q_raw = a.q ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + d] : 0u;
-    const int L = a.seq[b];
-    const int tail = a.tail ? a.tail[b] : 0;
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
     float my_lse = -INFINITY;
     if (tid < MAXS) {
