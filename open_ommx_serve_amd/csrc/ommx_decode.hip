@@ -422,8 +422,14 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         // per group: channel pass (clear outlier codes, scatter deltas), then the token
         // blocks of the group take tile and base terms in one accumulation chain
         f32x4 dq[4];
+        const bool g1_live = n0 + 32 < n_end;     // a last step of one group skips the second
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
+            if (g == 1 && !g1_live) {
+                dq[2] = f32x4{0, 0, 0, 0};
+                dq[3] = f32x4{0, 0, 0, 0};
+                break;
+            }
             if (OUTLIERS) {
                 // RES = false: the walk every group takes.  RES = true: a second walk that only
                 // adds f16 rounding residuals of large deltas onto the logits.
@@ -580,6 +586,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         // ---------------------------------------------------------------- P.V
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
+            if (kb == 1 && !g1_live) break;       // their weights are zero
             const int t0 = 32 * kb + 8 * kq;
             const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & 3) * PT_ROW + t0) * 2);
             const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * PT_ROW + t0) * 2);
