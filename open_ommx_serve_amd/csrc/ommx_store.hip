@@ -63,10 +63,14 @@ __device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict_
     return ((m < 0.0f) ? 8u : 0u) | idx;
 }
 
-// x / 2^e as a multiplication: 2^-e is exact for e in [-126,126] (the product and the
-// quotient are then the same real number, so they round alike, denormal results included).
-__device__ __forceinline__ float div_pow2(float x, float scale, float inv_scale, bool inv_ok) {
-    return inv_ok ? x * inv_scale : __fdiv_rn(x, scale);
+// x / 2^e is computed as x * 2^-e: 2^-e is exact for e in [-126,126], the product and the
+// quotient are then the same real number, so they round alike, denormal results included.
+// INT2 code clamp(rint(x / 2^e), 0, 3) of a finite x.  v_cvt_pk_u8_f32 rounds to nearest even
+// and saturates below at 0; the upper clamp commutes with the rounding.
+__device__ __forceinline__ uint32_t int2_code(float x, float scale, float inv_scale, bool inv_ok) {
+    if (inv_ok) return __builtin_amdgcn_cvt_pk_u8_f32(fminf(x * inv_scale, 3.0f), 0u, 0u);
+    const float c = fminf(fmaxf(rintf(__fdiv_rn(x, scale)), 0.0f), 3.0f);
+    return static_cast<uint32_t>(static_cast<int>(c));
 }
 
 // Order-preserving integer image of a bf16 value held as fp32 bits, low 16 bits cleared.
@@ -214,9 +218,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (FAST6 && fast_done) {
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                float c = rintf(div_pow2(w[i] - zp, scale, inv_scale, inv_ok));
-                c = fminf(fmaxf(c, 0.0f), 3.0f);
-                s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
+                s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, inv_ok));
             }
             // |(w - mc) * ms| is largest at the extreme lanes, which are outliers: they decide
             // whether every mapped value is finite (codec.py:55-57 checks all of them)
@@ -233,9 +235,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             int slot = 0;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                float c = rintf(div_pow2(w[i] - zp, scale, inv_scale, inv_ok));
-                c = fminf(fmaxf(c, 0.0f), 3.0f);
-                s_codes[i * D + d] = static_cast<uint8_t>(static_cast<int>(c));
+                s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, inv_ok));
                 if (kout > 0) {
                     const float mapped = (w[i] - mc) * ms;
                     mfin = mfin && is_finite_f32(mapped);
@@ -331,9 +331,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         uint64_t vb8 = 0;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
-            float q = rintf(div_pow2(v[c] - zp, scale, inv_scale, inv_ok));
-            q = fminf(fmaxf(q, 0.0f), 3.0f);
-            vb8 |= static_cast<uint64_t>(static_cast<int>(q)) << (2 * c);
+            vb8 |= static_cast<uint64_t>(int2_code(v[c] - zp, scale, inv_scale, inv_ok)) << (2 * c);
         }
         const int64_t vidx = (prow * a.H + h) * NGV + j;
         reinterpret_cast<uint64_t*>(a.v_main)[vidx] = vb8;
