@@ -102,8 +102,8 @@ def _make_runner(case, splits=None):
         rc = lib.ommx_decode_splitkv(
             case.q.data_ptr(), case.q.stride(0), case.q.stride(1),
             p["k_base"].data_ptr(), p["k_scale"].data_ptr(), p["k_zp"].data_ptr(),
-            p["k_fp4_mapscale"].data_ptr(), p["k_fp4_mapcenter"].data_ptr(),
-            p["k_obmp"].data_ptr(), p["k_oval"].data_ptr(),
+            _hip.ptr(p.get("k_fp4_mapscale")), _hip.ptr(p.get("k_fp4_mapcenter")),
+            _hip.ptr(p.get("k_obmp")), _hip.ptr(p.get("k_oval")),
             p["v_main"].data_ptr(), p["v_scale"].data_ptr(), p["v_zp"].data_ptr(),
             case.req_to_token.data_ptr(), case.req_to_token.stride(0),
             case.req_to_group.data_ptr(), case.req_to_group.stride(0),

@@ -197,7 +197,7 @@ template <bool OUTLIERS>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint8_t* const sm = smem_all + wave * WAVE_LDS;
+    uint8_t* const sm = smem_all + wave * (OUTLIERS ? WAVE_LDS : OFF_DT);   // no tile without outliers
     // the same place as an LDS byte address (for LDS instructions issued by hand)
     const uint32_t sm_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) uint8_t*)sm));
@@ -651,7 +651,7 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     const int vheads = a.Hkv * (R / 4);            // waves per (split, request)
     const int waves = (vheads % 4 == 0) ? 4 : ((vheads % 2 == 0) ? 2 : 1);
     const dim3 grid(a.S, vheads / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * WAVE_LDS;
+    const size_t shm = (size_t)waves * (a.kout == 6 ? WAVE_LDS : OFF_DT);
     if (a.kout == 6)
         hipLaunchKernelGGL(decode_splitkv_mfma_kernel<true>, grid, block, shm, st, a);
     else
