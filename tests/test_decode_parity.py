@@ -108,6 +108,17 @@ def test_long_context_64k_permuted_all_split_counts():
     _check(_run(case, num_kv_splits=64, ref_kernel=True), want, "ref S64")
 
 
+def test_long_context_128k_int64_tables_and_the_split_limit():
+    """ctx 131072 (the longest the reference serves), int64 tables, 256 splits (the limit) and
+    odd split counts that leave the last splits short or empty."""
+    case = build_decode_case([131072], seed=43, permute_tables=True, sparse_frac=0.005,
+                             table_dtype=torch.int64)
+    assert case.b_seq_len.tolist() == [131008]
+    want = _oracle(case, dtype=torch.float32)
+    for S in (None, 256, 255, 100, 3):
+        _check(_run(case, num_kv_splits=S), want, f"S{S}")
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_ragged_batch_shared_pool(ref_kernel):
     """Twelve requests of different lengths sharing one shuffled pool, incl. one with no
