@@ -387,3 +387,92 @@ def test_config5_bulk_pack_then_128_decode_steps_at_full_size():
         assert int(bt[0]) == len(idx)
         assert torch.equal(kt[0, :len(idx)].cpu(), Ks[i][idx]) and torch.equal(vt[0, :len(idx)].cpu(), Vs[i][idx])
     _assert_planes_equal_oracle(pool.request_planes(0), Ks[0][:n], Vs[0][:n], win, "config 5 req 0")
+
+
+def test_decode_step_replayed_from_a_hip_graph():
+    """One captured step = ring write (device counter advanced in the launch) + tail gather with
+    the window arithmetic + split-KV decode + combine.  Replayed 40 times while the host packs
+    completed groups between replays, and compared with an eager pool fed the same rows."""
+    H, D, Hq, B, steps = 8, 128, 32, 2, 40
+    win = WindowSpec()
+    prefill = [500, 333]
+    sm_scale = 1.0 / math.sqrt(D)
+    Ks, Vs = zip(*[synth_kv(n + steps, H, D, seed=700 + i, sparse_frac=0.005) for i, n in enumerate(prefill)])
+    pools = [MultiSeqKVPool(D, H, num_seqs=B, max_seq_len=600, window=win, device=DEV, kv_ring=True, **RECIPE)
+             for _ in range(2)]
+    for p in pools:
+        for i in range(B):
+            p.append_block(i, Ks[i][:prefill[i]].to(DEV), Vs[i][:prefill[i]].to(DEV))
+    g_pool, e_pool = pools
+    g_pool.decode_seed_seq_device(range(B))
+    d = g_pool._decode_buffers(B)
+    # fixed-address inputs and outputs of the captured step
+    newK = torch.zeros(B, H, D, dtype=torch.bfloat16, device=DEV)
+    newV = torch.zeros_like(newK)
+    q = torch.zeros(B, Hq, D, dtype=torch.bfloat16, device=DEV)
+    o = torch.zeros(B, Hq, D, dtype=torch.float32, device=DEV)
+    lse = torch.zeros(B, Hq, dtype=torch.float32, device=DEV)
+    from open_ommx_serve_amd.attention import make_attn_logits
+    S = 16
+    ws = make_attn_logits(B, Hq, S, D, DEV)
+    pl = g_pool.pool_planes()
+
+    def step():
+        write_tokens(g_pool.k_hist, g_pool.v_hist, d["seq_dev"], newK, newV, g_pool._ring_sink,
+                     g_pool._ring_rec, slots=d["rows"], pos_next=d["seq_dev"], err_flag=g_pool.err_flag)
+        gather_tails(g_pool.k_hist, g_pool.v_hist, d["kt"], d["vt"], g_pool._ring_sink, g_pool._ring_rec,
+                     seq=d["seq_dev"], slots=d["sel"], b_tail_len=d["b_tail"], b_seq_len=d["b_seq"],
+                     window_sink=win.sink_tokens, window_recent=win.recent_window, group_tokens=win.group_tokens)
+        ommx_paged_decode_attention_canonical(
+            q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"], pl["v_main"], pl["v_scale"],
+            pl["v_zp"], d["kt"], d["vt"], d["b_tail"], o, lse, pl["req_to_token"], pl["req_to_group"],
+            d["b_seq"], sm_scale=sm_scale, page_size=win.page_size, k_outliers_per_vector=6,
+            bitmap_read=True, k_obmp=pl["k_obmp"], k_fp4_mapscale=pl["k_fp4_mapscale"],
+            k_fp4_mapcenter=pl["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
+            max_seq_len=600, max_tail_len=g_pool.max_tail_len, num_kv_splits=S, attn_logits=ws)
+
+    # A token becomes visible to the decode of the step that appends it only after the host
+    # has packed the group it may complete, so the captured step decodes BEFORE the pack of
+    # its own append; the eager pool mirrors exactly that order.
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    qs = synth_q(steps, B * Hq, D, seed=8).reshape(steps, B, Hq, D)
+    with torch.cuda.stream(stream):
+        newK.copy_(torch.stack([Ks[i][prefill[i]] for i in range(B)]))
+        newV.copy_(torch.stack([Vs[i][prefill[i]] for i in range(B)]))
+        q.copy_(qs[0])
+        seq_before = d["seq_dev"].clone()
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+        d["seq_dev"].copy_(seq_before)          # capture does not run the kernels
+    torch.cuda.current_stream().wait_stream(stream)
+    for s in range(steps):
+        newK.copy_(torch.stack([Ks[i][prefill[i] + s] for i in range(B)]))
+        newV.copy_(torch.stack([Vs[i][prefill[i] + s] for i in range(B)]))
+        q.copy_(qs[s])
+        graph.replay()
+        torch.cuda.synchronize()
+        # eager mirror: same write, same decode inputs (before packing), then pack
+        write_tokens(e_pool.k_hist, e_pool.v_hist,
+                     torch.tensor([e_pool.seq_len[i] for i in range(B)], dtype=torch.int64, device=DEV),
+                     newK, newV, e_pool._ring_sink, e_pool._ring_rec)
+        cur = [prefill[i] + s + 1 for i in range(B)]
+        assert d["seq_dev"].tolist() == cur
+        # what the captured step attended: packed prefix as of the last host pack + tail as of now
+        want_o, want_l = [], []
+        for i in range(B):
+            n, packed_groups = cur[i], g_pool.packed_groups[i]
+            edge = win.sink_tokens + packed_groups * win.group_tokens
+            assert int(d["b_seq"][i]) == win.packed_len(n)
+            if win.packed_len(n) != packed_groups * win.group_tokens:
+                continue                           # the group completed by this very token: see above
+            wo, wl = _oracle_decode(q[i:i + 1], [Ks[i][:n]], [Vs[i][:n]], win, sm_scale)
+            _check_out((o[i:i + 1].cpu(), lse[i:i + 1].cpu()), (wo, wl), f"replay {s} req {i}")
+        # host seam between replays: advance the mirrors and pack what completed
+        packed = g_pool._advance_host_and_pack(range(B))
+        assert packed == e_pool._advance_host_and_pack(range(B))
+    for name in PLANE_NAMES:
+        assert torch.equal(getattr(g_pool, name), getattr(e_pool, name)), name
+    assert torch.equal(g_pool.k_hist, e_pool.k_hist) and torch.equal(g_pool.v_hist, e_pool.v_hist)
+    g_pool.check_errors()
