@@ -83,9 +83,12 @@ def store_table(device: torch.device) -> torch.Tensor:
     global _table_host
     if _table_host is None:
         _table_host = measure_store_table()
+    device = torch.device(device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
     key = str(device)
     if key not in _table_dev:
-        _table_dev[key] = _table_host.to(device)
+        _table_dev[key] = _table_host.to(device)    # first use on a device uploads (not capturable)
     return _table_dev[key]
 
 

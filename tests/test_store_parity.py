@@ -213,3 +213,36 @@ def test_decision_table_measured_on_this_host_is_monotone_and_near_the_exact_one
     ulps = (t[88:254].view(torch.int32) - d[88:254].view(torch.int32)).abs()
     assert int(ulps.max()) <= 64
     assert bool((t[257:264][1:] > t[257:264][:-1]).all())
+
+
+def test_store_replayed_from_a_hip_graph():
+    """The store launch neither allocates nor synchronises: captured once, replayed on new rows
+    (three replays with eager work between them), each time equal to the oracle's planes."""
+    T, H, D = 128, 2, 128
+    store_table_ready = hip_pack.store_table(torch.device("cuda"))     # upload outside the capture
+    assert store_table_ready.numel() == 264
+    K = torch.zeros(T, H, D, dtype=torch.bfloat16, device="cuda")
+    V = torch.zeros_like(K)
+    planes = alloc_planes(T // 16, T // 32, H, D, device="cuda")
+    err = torch.zeros(1, dtype=torch.int32, device="cuda")
+    K0, V0 = synth_kv(T, H, D, seed=90)
+    K.copy_(K0)
+    V.copy_(V0)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            store_pack_into(K, V, planes, err_flag=err)
+    torch.cuda.current_stream().wait_stream(stream)
+    for rep in range(3):
+        Kr, Vr = synth_kv(T, H, D, seed=91 + rep, sparse_frac=0.01)
+        K.copy_(Kr)
+        V.copy_(Vr)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(err.item()) == 0
+        want = O.pack_kv(Kr, Vr)
+        for name in PLANE_NAMES:
+            assert torch.equal(planes[name].cpu().view(torch.uint8), want[name].view(torch.uint8)), (rep, name)
+        (K.float().sum() + V.float().sum()).item()                      # eager work between replays
