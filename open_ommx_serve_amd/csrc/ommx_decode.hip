@@ -280,17 +280,24 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // channel pair (2*lane, 2*lane+1) parameters of both groups
     uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
     u32x2 g_bm[2], g_ov[2];
+    // (the group index is wave-uniform: base addresses are formed on the scalar unit, the lane
+    // adds a 32-bit byte offset)
+    const uint32_t kvh_s = __builtin_amdgcn_readfirstlane(kvh);
+    const uint32_t lane_b = lane;
+    auto at = [](const void* base, uint32_t byte_off) {
+        return static_cast<const char*>(base) + byte_off;
+    };
     auto fetch_params_g = [&](int g) {
         {
             const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);   // same for every lane
-            const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + (uint32_t)kvh) * D;
-            g_sc[g] = *reinterpret_cast<const uint16_t*>(a.k_scale + gidx + 2 * lane);
-            g_zp[g] = *reinterpret_cast<const uint32_t*>(a.k_zp + gidx + 2 * lane);
+            const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + kvh_s) * D;
+            g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
+            g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
             if (OUTLIERS) {
-                g_ms[g] = *reinterpret_cast<const uint32_t*>(a.k_ms + gidx + 2 * lane);
-                g_mc[g] = *reinterpret_cast<const uint32_t*>(a.k_mc + gidx + 2 * lane);
-                g_bm[g] = *reinterpret_cast<const u32x2*>(a.k_obmp + gidx * 4 + 8 * lane);
-                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(a.k_oval + gidx * 3) + (3 * lane) / 2;
+                g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
+                g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
+                g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
+                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
                 g_ov[g] = u32x2{ovp[0], ovp[1]};
             }
         }
