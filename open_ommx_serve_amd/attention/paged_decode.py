@@ -32,7 +32,8 @@ def _cu_count(device: torch.device) -> int:
 
 def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256,
                        q_per_kv: int = 4) -> int:
-    """Split count that gives every compute unit two workgroups (a workgroup is four waves of
+    """Split count that gives every compute unit four workgroups, two resident and two queued
+    behind them so that requests of different length even out (a workgroup is four waves of
     one split; a wave covers one kv head and four of its q heads), but never less than one
     64-token step per split (one 32-token group when even that leaves units idle): a wave's time
     is a fixed part plus ~5 us per step, so while compute units are idle more splits are faster;
@@ -42,7 +43,7 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
     on chip."""
     waves_per_split = int(kv_heads) * max(1, int(q_per_kv) // 4)
     wgs_per_split = max(1, int(batch) * max(1, waves_per_split // 4))
-    want = max(1, min(256, (2 * int(n_cu)) // wgs_per_split))
+    want = max(1, min(256, (4 * int(n_cu)) // wgs_per_split))
     steps = max(1, (int(max_seq_len) + 63) // 64)
     if want >= 2 * steps:          # plenty of idle units: splits of one 32-token group
         return int(min(want, max(1, (int(max_seq_len) + 31) // 32)))

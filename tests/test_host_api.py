@@ -84,7 +84,7 @@ def test_split_heuristic_bounds():
     assert auto_num_kv_splits(960, 1, 8, 256) >= 1
     assert auto_num_kv_splits(65472, 1, 8, 256) == 256
     assert auto_num_kv_splits(960, 1, 8, 256) == 30          # one 32-token group per split
-    assert auto_num_kv_splits(65472, 32, 8, 256) == 8
+    assert auto_num_kv_splits(65472, 32, 8, 256) == 16
     assert 1 <= auto_num_kv_splits(1, 1, 1, 256) <= 256
 
 
