@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 1
+#define OMMX_ABI_VERSION 2   /* 2: ring, tail-gather and state-merge entry points */
 
 /* number of floats in the store decision table: 256 pow2 thresholds + 8 FP4 slots */
 #define OMMX_STORE_TABLE_FLOATS 264

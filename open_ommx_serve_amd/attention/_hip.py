@@ -16,6 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
+ABI_VERSION = 2
 ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
@@ -67,7 +68,7 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.ommx_abi_version() != 1:
+    if lib.ommx_abi_version() != ABI_VERSION:
         raise RuntimeError("libommx_hip.so ABI version mismatch; rebuild it")
     _lib = lib
     return lib
