@@ -107,7 +107,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       permute_tables: bool = False, sparse_frac: float = 0.0,
                       outliers_per_vector: int = 6, window: Optional[WindowSpec] = None,
                       device: Any = "cuda", keep_source: bool = False,
-                      table_dtype: torch.dtype = torch.int32) -> DecodeCase:
+                      table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0) -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -142,7 +142,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     src = []
     po = go = 0
     for b, n in enumerate(int(x) for x in seq_lens):
-        K, V = synth_kv(n, H, D, seed, sparse_frac=sparse_frac, stream=b)
+        K, V = synth_kv(n, H, D, seed, sparse_frac=sparse_frac, sparse_gain=sparse_gain, stream=b)
         edge = win.boundary(n)
         ti = win.tail_indices(n)
         tails.append(len(ti))

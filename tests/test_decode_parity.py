@@ -251,3 +251,48 @@ def test_host_argument_checks_raise_before_launch():
         ommx_paged_decode_attention_canonical(*args, **{**kw, "bitmap_read": False})
     ommx_paged_decode_attention_canonical(*args, **kw)
     torch.cuda.synchronize()
+
+
+def test_randomised_shapes_two_kernels_and_the_oracle():
+    """Forty random cases (batch, lengths, GQA ratio, split count, table type, outlier mix with
+    magnitudes up to x200, partial last groups): the matrix-core kernel against the plain
+    fp32 kernel on the device (both within tolerance of each other's oracle), and against the
+    oracle itself on every fourth case."""
+    g = torch.Generator().manual_seed(2024)
+
+    def rnd(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    for it in range(40):
+        B = rnd(1, 5)
+        lens = [rnd(1, 6000) if rnd(0, 4) else rnd(1, 80) for _ in range(B)]
+        r = (4, 8)[rnd(0, 1)]
+        hkv = (1, 2, 4, 8)[rnd(0, 3)]
+        gain = (12.0, 40.0, 200.0)[rnd(0, 2)]
+        case = build_decode_case(lens, q_heads=hkv * r, kv_heads=hkv, seed=1000 + it,
+                                 permute_tables=bool(rnd(0, 1)), sparse_frac=(0.0, 0.005, 0.03)[rnd(0, 2)],
+                                 table_dtype=(torch.int32, torch.int64)[rnd(0, 1)], sparse_gain=gain)
+        if rnd(0, 2) == 0:                         # cut into the last group of every request
+            cut = torch.tensor([max(0, n - rnd(0, 31)) for n in case.b_seq_len.tolist()], dtype=torch.int32)
+            case.b_seq_len.copy_(cut)
+        S = (None, 1, 2, 5, 16, 37, 256)[rnd(0, 6)]
+        what = f"case {it}: B={B} lens={lens} r={r} hkv={hkv} gain={gain} S={S}"
+        fast = _run(case, num_kv_splits=S)
+        ref = _run(case, num_kv_splits=S, ref_kernel=True)
+        assert torch.isfinite(fast[0]).all(), what
+        err = (fast[0] - ref[0]).abs()
+        assert err.max().item() <= MAX_ABS and err.mean().item() <= MEAN_ABS, f"{what}: {err.max().item():.3e}"
+        fin = torch.isfinite(ref[1])
+        assert torch.equal(torch.isfinite(fast[1]), fin), what
+        # x200 outliers push lse into the hundreds, where 2e-3 is a few dozen fp32 ulps of the
+        # logits' own accumulation: allow 1e-5 relative on top
+        if fin.any():
+            d = (fast[1][fin] - ref[1][fin]).abs() - 1e-5 * ref[1][fin].abs()
+            assert d.max().item() <= 2e-3, what
+        if it % 4 == 0:
+            wo, wl = _oracle(case, dtype=torch.float32)
+            e = (fast[0].double() - wo).abs()
+            assert e.max().item() <= MAX_ABS and e.mean().item() <= MEAN_ABS, what
+            f2 = torch.isfinite(wl)
+            if f2.any():
+                assert ((fast[1].double()[f2] - wl[f2]).abs() - 1e-5 * wl[f2].abs()).max().item() <= 2e-3, what
