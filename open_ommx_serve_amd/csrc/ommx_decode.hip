@@ -62,10 +62,11 @@ constexpr int DT_ROW = 272;
 constexpr int OFF_LC = OFF_DT + 32 * DT_ROW;        // [64 tokens][4 heads] f32 logit corrections
 constexpr int WAVE_LDS = OFF_LC + 1024;             // 17792
 static_assert(OFF_DT % 16 == 0 && OFF_VT % 16 == 0 && OFF_PT % 16 == 0, "b128 alignment");
-// One f16 carries 11 bits.  An outlier delta d (in units of 4) whose f16 rounding error times
-// the largest |4q| of its channel could move a logit by more than ~1.5e-3 gets its residual
-// added exactly; the bound is |d| * max|4q| >= BIG_DELTA * 16, i.e. |d| >= 4 at |q| = 4.
-constexpr float BIG_DELTA = 4.0f;
+// One f16 carries 11 bits: rounding d (an outlier delta in units of 4) costs up to |d| * 2^-11,
+// i.e. up to |d| * max|4q| * 2^-11 * sm_scale on a logit.  A delta with |d| * max|4q| >=
+// BIG_DELTA * 16 (|d| >= 2 at |q| = 4; at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its
+// residual added exactly; smaller ones stay below that and average a quarter of it.
+constexpr float BIG_DELTA = 2.0f;
 
 __device__ __forceinline__ f32x4 mfma_bf16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),

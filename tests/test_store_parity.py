@@ -246,3 +246,47 @@ def test_store_replayed_from_a_hip_graph():
         for name in PLANE_NAMES:
             assert torch.equal(planes[name].cpu().view(torch.uint8), want[name].view(torch.uint8)), (rep, name)
         (K.float().sum() + V.float().sum()).item()                      # eager work between replays
+
+
+def test_store_randomised_tie_patterns_signed_zeros_and_extremes():
+    """Thirty random blocks drawn from small value sets (so that ties reach into the chosen
+    lanes in every pattern), with signed zeros, bf16 denormals, huge magnitudes and vectors that
+    are constant or constant but for one to five lanes; bf16 and fp32 input; bit-exact."""
+    g = torch.Generator().manual_seed(31337)
+
+    def rnd(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    pools = [
+        torch.tensor([-0.0, 0.0, 1.0, -1.0]),
+        torch.tensor([-0.0, 0.0]),
+        torch.tensor([3.0, 3.0, 3.0, 3.0, 3.0, -2.0, 7.0]),
+        torch.tensor([9.1835e-41, -9.1835e-41, 0.0, 1e-38, -1e-38]),          # bf16 denormals
+        torch.tensor([1e30, -1e30, 5e8, 2e9, -3e9, 1.0]),
+        torch.tensor([-4.0, -1.0, -1.0, 0.0, 0.0, 0.25, 2.0, 2.0, 8.0, 8.0, 8.0]),
+        torch.arange(-16, 17).float() * 0.5,
+    ]
+    for it in range(30):
+        H, D, T = (1, 2, 8)[rnd(0, 2)], (32, 64, 128)[rnd(0, 2)], 32 * rnd(1, 4)
+        pk = pools[rnd(0, len(pools) - 1)]
+        pv = pools[rnd(0, len(pools) - 1)]
+        K = pk[torch.randint(0, len(pk), (T, H, D), generator=g)]
+        V = pv[torch.randint(0, len(pv), (T, H, D), generator=g)]
+        # a few vectors that are constant but for n lanes
+        for _ in range(4):
+            h, d, n = rnd(0, H - 1), rnd(0, D - 1), rnd(0, 5)
+            K[:32, h, d] = float(pk[0])
+            for i in torch.randperm(32, generator=g)[:n].tolist():
+                K[i, h, d] = float(pk[rnd(0, len(pk) - 1)]) + 1.0
+        if rnd(0, 1):
+            K, V = K.to(torch.bfloat16), V.to(torch.bfloat16)
+        what = f"random block {it} {tuple(K.shape)} {K.dtype}"
+        try:
+            want = O.pack_kv(K, V)
+        except (IndexError, ValueError) as exc:
+            # magnitudes of 1e9 and more defeat the +1e9 sentinel of the selector: the
+            # reference refuses such a block, and so must the store
+            with pytest.raises(type(exc)):
+                _hip(K, V)
+            continue
+        assert_planes_equal(_hip(K, V), want, what=what, zero_sign_free=True)
