@@ -54,14 +54,18 @@ constexpr int OFF_MAGIC = 0;        // [2 groups][64 pairs] bf16x2: 2^e of chann
 constexpr int OFF_ZPP = 512;        // same order, bf16 zero points
 constexpr int OFF_KT = 1024;        // [64 tokens][KT_ROW] K code rows
 constexpr int OFF_VT = OFF_KT + 64 * KT_ROW;        // [8 dword columns][VT_COL] V code dwords
-constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [4 heads][PT_ROW] f16 softmax weights
-constexpr int OFF_VS = OFF_PT + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 2^e_v
-constexpr int OFF_VZ = OFF_VS + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 v zero points
-constexpr int OFF_DT = OFF_VZ + 4 * PT_ROW * 2;     // [32 tokens][DT_ROW B] f16 outlier deltas of one group
+constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [HR heads][PT_ROW] f16 softmax weights
 constexpr int DT_ROW = 272;
-constexpr int OFF_LC = OFF_DT + 32 * DT_ROW;        // [64 tokens][4 heads] f32 logit corrections
-constexpr int WAVE_LDS = OFF_LC + 1024;             // 17792
-static_assert(OFF_DT % 16 == 0 && OFF_VT % 16 == 0 && OFF_PT % 16 == 0, "b128 alignment");
+template <int HR>                   // the rest depends on the q heads per wave
+struct LdsMap {
+    static constexpr int VS = OFF_PT + HR * PT_ROW * 2;    // [4 channel groups][PT_ROW] f16 2^e_v
+    static constexpr int VZ = VS + 4 * PT_ROW * 2;         // [4 channel groups][PT_ROW] f16 v zero points
+    static constexpr int DT = VZ + 4 * PT_ROW * 2;         // [32 tokens][DT_ROW B] f16 outlier deltas of one group
+    static constexpr int LC = DT + 32 * DT_ROW;            // [64 tokens][HR] f32 logit corrections
+    static constexpr int END = LC + 64 * HR * 4;           // 17792 / 19584: two 4-wave workgroups fit a CU's 160 KB
+    static_assert(DT % 16 == 0 && LC % 16 == 0, "b128 alignment");
+};
+static_assert(OFF_VT % 16 == 0 && OFF_PT % 16 == 0, "b128 alignment");
 // One f16 carries 11 bits: rounding d (an outlier delta in units of 4) costs up to |d| * 2^-11,
 // i.e. up to |d| * max|4q| * 2^-11 * sm_scale on a logit.  A delta with |d| * max|4q| >=
 // BIG_DELTA * 16 (|d| >= 2 at |q| = 4; at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its
@@ -174,6 +178,73 @@ __device__ __forceinline__ void wave_sum4(float (&v)[4]) {
     v[3] = readlane_f32(d, 63);
 }
 
+// Two sets of lanes, 32 apart, hold partial results of the same quantity: both get the
+// combination.  v_permlane32_swap trades the upper half of one register with the lower half of
+// the other, which leaves (low, low) and (high, high) copies.
+__device__ __forceinline__ void halves_of(float v, float& lo, float& hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+// Maxima / sums of four values over the 32 lanes of rows {0, 2} and of rows {1, 3} separately
+// (a row = 16 lanes); every lane ends with the result of its own pair of rows.
+__device__ __forceinline__ void rowpair_max4(float (&v)[4]) {
+    float a = v[0], b = v[1], c = v[2], d = v[3];
+    asm volatile(
+        "s_nop 1\n"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %2, %2, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_max_f32_dpp %3, %3, %3 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "s_nop 1\n"
+        : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    float lo, hi;
+    halves_of(a, lo, hi); v[0] = fmaxf(lo, hi);
+    halves_of(b, lo, hi); v[1] = fmaxf(lo, hi);
+    halves_of(c, lo, hi); v[2] = fmaxf(lo, hi);
+    halves_of(d, lo, hi); v[3] = fmaxf(lo, hi);
+}
+__device__ __forceinline__ void rowpair_sum4(float (&v)[4]) {
+    float a = v[0], b = v[1], c = v[2], d = v[3];
+    asm volatile(
+        "s_nop 1\n"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %2, %2, %2 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "v_add_f32_dpp %3, %3, %3 row_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+        "s_nop 1\n"
+        : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    float lo, hi;
+    halves_of(a, lo, hi); v[0] = lo + hi;
+    halves_of(b, lo, hi); v[1] = lo + hi;
+    halves_of(c, lo, hi); v[2] = lo + hi;
+    halves_of(d, lo, hi); v[3] = lo + hi;
+}
+
 // K pair p of a code dword: channels p (low half) and p+8 (high half) as bf16.  The 2-bit code
 // may sit anywhere in the mantissa: at bits [2k+1:2k] the element reads (1 + c*2^(2k-7))*2^e, and
 // the matching A operand carries q*2^(7-2k), so the product is still q*c*2^e plus a constant
@@ -194,23 +265,24 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
     return (sh & ((Y & 1) ? 0x03000300u : 0x00C000C0u)) | one_f16x2;
 }
 
-template <bool OUTLIERS>
+template <bool OUTLIERS, int HR>          // HR: q heads per kv head (4 or 8), all on one wave
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint8_t* const sm = smem_all + wave * (OUTLIERS ? WAVE_LDS : OFF_DT);   // no tile without outliers
+    constexpr int OFF_VS = LdsMap<HR>::VS, OFF_VZ = LdsMap<HR>::VZ, OFF_DT = LdsMap<HR>::DT,
+                  OFF_LC = LdsMap<HR>::LC;
+    uint8_t* const sm = smem_all + wave * (OUTLIERS ? LdsMap<HR>::END : OFF_DT);   // no tile without outliers
     // the same place as an LDS byte address (for LDS instructions issued by hand)
     const uint32_t sm_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) uint8_t*)sm));
     const int j = lane & 15, kq = lane >> 4;
+    // With 8 heads the MFMA rows are (row group x = row / 8, head = row % 8); a lane holds rows
+    // 4kq..4kq+3 of a result, i.e. heads 4*hg + r of row group kq / 2.
+    const int hg = HR == 8 ? (kq & 1) : 0;
     const int Hkv = a.Hkv;
     const int waves = blockDim.x >> 6;
-    // 8 q heads per kv head run as two waves of 4 heads on the same kv head (the second
-    // read of the K/V lines hits the caches; HBM traffic stays one pass)
-    const int qgroups = a.Hq / (Hkv * 4);
-    const int vhead = blockIdx.y * waves + wave;
-    const int kvh = qgroups == 2 ? (vhead >> 1) : vhead;
-    const int qh0 = qgroups == 2 ? kvh * 8 + 4 * (vhead & 1) : kvh * 4;      // first of this wave's 4 q heads
+    const int kvh = blockIdx.y * waves + wave;
+    const int qh0 = kvh * HR;             // first of this wave's q heads
     const int b = blockIdx.z, sp = blockIdx.x;
     const int L = a.seq[b];
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
@@ -311,7 +383,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         fetch_tables(n_begin + 64);
     }
 
-    // ---- A operands: scaled q of head j%4 for this lane's 32-channel quarter ------------
+    // ---- A operands: scaled q of head j % HR for this lane's 32-channel quarter ---------
     // (pair order: q * 2^(7-2k) with k the code position of the pair, see k_pair; natural
     // order: 4*q)
     // pair order (QK base, bias):   k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2)
@@ -320,7 +392,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     {
         // this lane's 32 channels of q: 16 dwords, channel 2i in the low half of dword i
         const uint32_t* qh = reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + (j & 3)) * a.q_sh + 32 * kq);
+            a.q + b * a.q_sb + (int64_t)(qh0 + (j & (HR - 1))) * a.q_sh + 32 * kq);
         uint32_t qw[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) qw[i] = qh[i];
@@ -339,23 +411,34 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             }
         }
     }
-    // the same 4*q for the channel pass: heads 0..3 of channels 2*lane, 2*lane+1 (fp32)
-    float q4[2][4];
-    if (OUTLIERS) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t w = *reinterpret_cast<const uint32_t*>(
-                a.q + b * a.q_sb + (int64_t)(qh0 + r) * a.q_sh + 2 * lane);
-            q4[0][r] = 4.0f * __uint_as_float(w << 16);
-            q4[1][r] = 4.0f * __uint_as_float(w & 0xFFFF0000u);
-        }
-    }
+    // q of every head for the channel pass, channels 2*lane and 2*lane+1: as fp32 with 4
+    // heads, left as the bf16 pair with 8 (registers are short there, and the residual walk
+    // that reads them is rare)
+    uint32_t qraw[HR];
+    float qf[2][4];
+    auto q4_at = [&](int u, int r) {      // 4*q
+        if constexpr (HR == 4) return qf[u][r];
+        else return 4.0f * __uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16));
+    };
     // per channel: the |delta/4| from which the residual matters (infinite for q = 0)
     float big_thr[2] = {0.0f, 0.0f};
     if (OUTLIERS) {
 #pragma unroll
+        for (int r = 0; r < HR; ++r)
+            qraw[r] = *reinterpret_cast<const uint32_t*>(
+                a.q + b * a.q_sb + (int64_t)(qh0 + r) * a.q_sh + 2 * lane);
+        if constexpr (HR == 4) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                qf[0][r] = 4.0f * __uint_as_float(qraw[r] << 16);
+                qf[1][r] = 4.0f * __uint_as_float(qraw[r] & 0xFFFF0000u);
+            }
+        }
+#pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const float qm = fmaxf(fmaxf(fabsf(q4[u][0]), fabsf(q4[u][1])), fmaxf(fabsf(q4[u][2]), fabsf(q4[u][3])));
+            float qm = 0.0f;
+#pragma unroll
+            for (int r = 0; r < HR; ++r) qm = fmaxf(qm, fabsf(q4_at(u, r)));
             big_thr[u] = (BIG_DELTA * 16.0f) * __builtin_amdgcn_rcpf(qm);
         }
     }
@@ -421,8 +504,11 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 }
             }
         }
-        if (OUTLIERS)
-            *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * lane) = u32x4{0, 0, 0, 0};
+        if (OUTLIERS) {
+#pragma unroll
+            for (int i = 0; i < HR / 4; ++i)
+                *reinterpret_cast<u32x4*>(sm + OFF_LC + 4 * HR * lane + 16 * i) = u32x4{0, 0, 0, 0};
+        }
         lds_fence();
         if (more) fetch_kv();             // K/V registers are staged: start the next rows
 
@@ -469,7 +555,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const uint32_t field = 3u << (2 * (c & 15));
                         const uint32_t kt = sm_lds + OFF_KT + g * 32 * KT_ROW + 4 * (c >> 4);
                         uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
-                        float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 128;
+                        float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 32 * HR;
 #pragma unroll
                         for (int sidx = 0; sidx < 6; ++sidx) {
                             const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32
@@ -489,8 +575,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                                 if (fabsf(dl) >= big_thr[u]) {
                                     const float lo = dl - static_cast<float>(hi);
 #pragma unroll
-                                    for (int r = 0; r < 4; ++r)
-                                        __hip_atomic_fetch_add(lc + pos * 4 + r, lo * q4[u][r], __ATOMIC_RELAXED,
+                                    for (int r = 0; r < HR; ++r)
+                                        __hip_atomic_fetch_add(lc + pos * HR + r, lo * q4_at(u, r), __ATOMIC_RELAXED,
                                                                __HIP_MEMORY_SCOPE_WAVEFRONT);
                                 }
                             }
@@ -544,40 +630,72 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         if (more) fetch_tables(n0 + 128);  // after the parameter loads, which used the group slots
 
         // ---------------------------------------------------------------- softmax
-        // bias of (group, head r): sum q*zp - sum A*2^e ; columns 0..3 live in lanes 0..3 (kq 0)
-        float logit[4];
+        // bias of (group, head): sum q*zp - sum A*2^e, columns 0..3 of the bias result
+        // 4 heads: a lane owns token n0 + lane (block kq) and heads 0..3.
+        // 8 heads: a lane owns tokens n0 + lane and n0 + (lane ^ 16) (blocks kq and kq ^ 1, same
+        //          K group) and heads 4*hg..4*hg+3.
+        constexpr int NT = HR / 4;                  // tokens per lane
+        const bool tok_ok2[2] = {tok_ok, n0 + (lane ^ 16) < n_end};
+        float logit[NT][4];
         {
-            const f32x4 dsel = kq == 0 ? dq[0] : (kq == 1 ? dq[1] : (kq == 2 ? dq[2] : dq[3]));
+            f32x4 dsel[NT];
+            dsel[0] = kq == 0 ? dq[0] : (kq == 1 ? dq[1] : (kq == 2 ? dq[2] : dq[3]));
+            if constexpr (HR == 8) dsel[1] = kq == 0 ? dq[1] : (kq == 1 ? dq[0] : (kq == 2 ? dq[3] : dq[2]));
             const int gsel = lane >> 5;
-            f32x4 corr = {0, 0, 0, 0};
-            if (OUTLIERS) corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * lane);
+            f32x4 corr[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                corr[t] = f32x4{0, 0, 0, 0};
+                if (OUTLIERS)
+                    corr[t] = *reinterpret_cast<const f32x4*>(
+                        sm + OFF_LC + 4 * HR * (t ? (lane ^ 16) : lane) + 16 * hg);
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float zpv = __shfl(dbias[r], gsel);          // column gsel, rows 0..3
-                const float s1v = __shfl(dbias[r], 2 + gsel);
-                const float raw = dsel[r] + corr[r] + (zpv - s1v);
-                float x = raw * a.sm_scale;
-                x = apply_cap(x, a.cap) * c_log2e;
-                logit[r] = tok_ok ? x : -INFINITY;
+                // column gsel (zp) and 2 + gsel (2^e) of the rows that hold this lane's heads
+                const float zpv = __shfl(dbias[r], 16 * hg + gsel);
+                const float s1v = __shfl(dbias[r], 16 * hg + 2 + gsel);
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    logit[t][r] = (dsel[t][r] + corr[t][r] + (zpv - s1v)) * a.sm_scale;
             }
+            if (a.cap > 0.0f) {           // one uniform branch around all the tanh work
+                asm volatile("" ::: "memory");      // (keeps it a branch: never computed speculatively)
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) logit[t][r] = apply_cap(logit[t][r], a.cap);
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) logit[t][r] = tok_ok2[t] ? logit[t][r] * c_log2e : -INFINITY;
         }
-        float alpha[4], p[4], mxs[4] = {logit[0], logit[1], logit[2], logit[3]};
-        wave_max4(mxs);
+        float alpha[4], p[NT][4], mxs[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mxs[r] = HR == 8 ? fmaxf(logit[0][r], logit[NT - 1][r]) : logit[0][r];
+        if constexpr (HR == 8) rowpair_max4(mxs); else wave_max4(mxs);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float m_new = fmaxf(m_run[r], mxs[r]);
             alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
-            p[r] = tok_ok ? __builtin_amdgcn_exp2f(logit[r] - m_new) : 0.0f;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                p[t][r] = tok_ok2[t] ? __builtin_amdgcn_exp2f(logit[t][r] - m_new) : 0.0f;
             m_run[r] = m_new;
         }
         {
             uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const _Float16 ph = static_cast<_Float16>(p[r]);
                 // accumulate the weight that P.V really uses (the f16-rounded one)
-                l_run[r] = l_run[r] * alpha[r] + static_cast<float>(ph);
-                pt[r * PT_ROW + lane] = __builtin_bit_cast(uint16_t, ph);
+                l_run[r] *= alpha[r];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const _Float16 ph = static_cast<_Float16>(p[t][r]);
+                    l_run[r] += static_cast<float>(ph);
+                    pt[(4 * hg + r) * PT_ROW + (t ? (lane ^ 16) : lane)] = __builtin_bit_cast(uint16_t, ph);
+                }
             }
         }
         // the running maxima seldom move after the first steps: rescale only when one did
@@ -596,55 +714,109 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         for (int kb = 0; kb < 2; ++kb) {
             if (kb == 1 && !g1_live) break;       // their weights are zero
             const int t0 = 32 * kb + 8 * kq;
-            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & 3) * PT_ROW + t0) * 2);
-            const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * PT_ROW + t0) * 2);
-            const u32x4 apv = {pk_mul_f16(pw[0], sw[0]), pk_mul_f16(pw[1], sw[1]),
-                               pk_mul_f16(pw[2], sw[2]), pk_mul_f16(pw[3], sw[3])};
+            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + OFF_PT + ((j & (HR - 1)) * PT_ROW + t0) * 2);
             // columns 0..3: vz of channel group j, columns 4..7: vs; others repeat
             const u32x4 bz = *reinterpret_cast<const u32x4*>(
                 sm + ((j & 4) ? OFF_VS : OFF_VZ) + ((j & 3) * PT_ROW + t0) * 2);
             accz = mfma_f16(pw, bz, accz);
-            // V codes: dword column j%8, half j/8, tokens t0..t0+7
-            const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (j & 7) * VT_COL + t0;
-            const u32x4 va = *reinterpret_cast<const u32x4*>(vt);
-            const u32x4 vb = *reinterpret_cast<const u32x4*>(vt + 4);
-            const uint32_t sel = (j & 8) ? 0x07060302u : 0x05040100u;
-            const uint32_t mg0 = __builtin_amdgcn_perm(va[1], va[0], sel);
-            const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], sel);
-            const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], sel);
-            const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], sel);
+            if constexpr (HR == 4) {
+                // row group x = j / 4 carries the scales of channel group x
+                const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + OFF_VS + ((j >> 2) * PT_ROW + t0) * 2);
+                const u32x4 apv = {pk_mul_f16(pw[0], sw[0]), pk_mul_f16(pw[1], sw[1]),
+                                   pk_mul_f16(pw[2], sw[2]), pk_mul_f16(pw[3], sw[3])};
+                // V codes: dword column j%8, half j/8, tokens t0..t0+7
+                const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (j & 7) * VT_COL + t0;
+                const u32x4 va = *reinterpret_cast<const u32x4*>(vt);
+                const u32x4 vb = *reinterpret_cast<const u32x4*>(vt + 4);
+                const uint32_t sel = (j & 8) ? 0x07060302u : 0x05040100u;
+                const uint32_t mg0 = __builtin_amdgcn_perm(va[1], va[0], sel);
+                const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], sel);
+                const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], sel);
+                const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], sel);
 #define OMMX_PV(Y) acc[Y] = mfma_f16(apv, u32x4{v_pair<Y>(mg0, one2), v_pair<Y>(mg1, one2), v_pair<Y>(mg2, one2), v_pair<Y>(mg3, one2)}, acc[Y]);
-            OMMX_PV(0) OMMX_PV(1) OMMX_PV(2) OMMX_PV(3) OMMX_PV(4) OMMX_PV(5) OMMX_PV(6) OMMX_PV(7)
+                OMMX_PV(0) OMMX_PV(1) OMMX_PV(2) OMMX_PV(3) OMMX_PV(4) OMMX_PV(5) OMMX_PV(6) OMMX_PV(7)
 #undef OMMX_PV
+            } else {
+                // Two row groups only, so the channel groups go in two sets s = 0, 1: row group
+                // x = j / 8 carries the scales of channel group 2s + x, and column j reads V
+                // dword column 4s + j%4 (whose channel group is 2s + (j%4)/2), byte 2*((j/4)%2) +
+                // j/8 of it: four channels per token, taken one per result (acc[4s + y]).
+                const uint32_t bsel = 2 * ((j >> 2) & 1) + (j >> 3);
+                const uint32_t sel = bsel | 0x0C000C00u | ((4u + bsel) << 16);
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const u32x4 sw = *reinterpret_cast<const u32x4*>(
+                        sm + OFF_VS + ((2 * s + (j >> 3)) * PT_ROW + t0) * 2);
+                    const u32x4 apv = {pk_mul_f16(pw[0], sw[0]), pk_mul_f16(pw[1], sw[1]),
+                                       pk_mul_f16(pw[2], sw[2]), pk_mul_f16(pw[3], sw[3])};
+                    const uint32_t* vt = reinterpret_cast<const uint32_t*>(sm + OFF_VT) + (4 * s + (j & 3)) * VT_COL + t0;
+                    const u32x4 va = *reinterpret_cast<const u32x4*>(vt);
+                    const u32x4 vb = *reinterpret_cast<const u32x4*>(vt + 4);
+                    const uint32_t mg0 = __builtin_amdgcn_perm(va[1], va[0], sel);
+                    const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], sel);
+                    const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], sel);
+                    const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], sel);
+#define OMMX_PV(Y) acc[4 * s + Y] = mfma_f16(apv, u32x4{v_pair<Y>(mg0, one2), v_pair<Y>(mg1, one2), v_pair<Y>(mg2, one2), v_pair<Y>(mg3, one2)}, acc[4 * s + Y]);
+                    OMMX_PV(0) OMMX_PV(1) OMMX_PV(2) OMMX_PV(3)
+#undef OMMX_PV
+                }
+            }
         }
         lds_fence();
     }
 
     // ---- epilogue: o = (f*(acc - PVS) + PVZ) / l with f = 4 or 16, lse = m + ln l ----------
     float l_tot[4] = {l_run[0], l_run[1], l_run[2], l_run[3]};
-    wave_sum4(l_tot);
-    const int jg = (j & 7) >> 1;
-    float pvz[4], pvs[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        pvz[r] = __shfl(accz[r], jg);          // column jg, rows 0..3 (kq 0)
-        pvs[r] = __shfl(accz[r], 4 + jg);
-    }
-    if (kq == jg) {
-        const int ch0 = 16 * (j & 7) + 8 * (j >> 3);
+    if constexpr (HR == 8) rowpair_sum4(l_tot); else wave_sum4(l_tot);
+    if constexpr (HR == 4) {
+        const int jg = (j & 7) >> 1;
+        float pvz[4], pvs[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
-            const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+            pvz[r] = __shfl(accz[r], jg);          // column jg, rows 0..3 (kq 0)
+            pvs[r] = __shfl(accz[r], 4 + jg);
+        }
+        if (kq == jg) {
+            const int ch0 = 16 * (j & 7) + 8 * (j >> 3);
 #pragma unroll
-            for (int y = 0; y < 8; ++y)
-                dst[ch0 + y] = (((y & 1) ? 4.0f : 16.0f) * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
+            for (int r = 0; r < 4; ++r) {
+                float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
+                const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+#pragma unroll
+                for (int y = 0; y < 8; ++y)
+                    dst[ch0 + y] = (((y & 1) ? 4.0f : 16.0f) * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
+            }
+        }
+    } else {
+        const int xg = (j & 3) >> 1;               // the row group that is valid in column j
+        float pvz[2][4], pvs[2][4];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {          // columns 2s+xg / 4+2s+xg, rows of this head group
+                pvz[s][r] = __shfl(accz[r], 16 * hg + 2 * s + xg);
+                pvs[s][r] = __shfl(accz[r], 16 * hg + 4 + 2 * s + xg);
+            }
+        if ((kq >> 1) == xg) {
+            const int bsel = 2 * ((j >> 2) & 1) + (j >> 3);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* dst = a.al + b * a.al_b + (int64_t)(qh0 + 4 * hg + r) * a.al_h + (int64_t)sp * a.al_s;
+                const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int ch0 = 16 * (4 * s + (j & 3)) + 4 * bsel;
+#pragma unroll
+                    for (int y = 0; y < 4; ++y)
+                        dst[ch0 + y] = (((y & 1) ? 4.0f : 16.0f) * (acc[4 * s + y][r] - pvs[s][r]) + pvz[s][r]) * inv;
+                }
+            }
         }
     }
-    if (lane < 4) {
-        float* dst = a.al + b * a.al_b + (int64_t)(qh0 + lane) * a.al_h + (int64_t)sp * a.al_s;
-        const float lt = lane == 0 ? l_tot[0] : (lane == 1 ? l_tot[1] : (lane == 2 ? l_tot[2] : l_tot[3]));
-        const float mt = lane == 0 ? m_run[0] : (lane == 1 ? m_run[1] : (lane == 2 ? m_run[2] : m_run[3]));
+    if (j < 4 && kq < HR / 4) {                    // lane 16*hg + r holds head 4*hg + r
+        float* dst = a.al + b * a.al_b + (int64_t)(qh0 + 4 * kq + j) * a.al_h + (int64_t)sp * a.al_s;
+        const float lt = j == 0 ? l_tot[0] : (j == 1 ? l_tot[1] : (j == 2 ? l_tot[2] : l_tot[3]));
+        const float mt = j == 0 ? m_run[0] : (j == 1 ? m_run[1] : (j == 2 ? m_run[2] : m_run[3]));
         dst[D] = lt > 0.0f ? (mt + log2f(lt)) * 0.6931471805599453f : -INFINITY;
     }
 }
@@ -656,14 +828,18 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     if (Dh != 128 || !(R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
-    const int vheads = a.Hkv * (R / 4);            // waves per (split, request)
-    const int waves = (vheads % 4 == 0) ? 4 : ((vheads % 2 == 0) ? 2 : 1);
-    const dim3 grid(a.S, vheads / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * (a.kout == 6 ? WAVE_LDS : OFF_DT);
-    if (a.kout == 6)
-        hipLaunchKernelGGL(decode_splitkv_mfma_kernel<true>, grid, block, shm, st, a);
+    const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);    // one wave per kv head
+    const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
+    const size_t shm = (size_t)waves * (R == 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
+                                               : (a.kout == 6 ? LdsMap<8>::END : LdsMap<8>::DT));
+    if (a.kout == 6 && R == 4)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4>), grid, block, shm, st, a);
+    else if (a.kout == 6)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8>), grid, block, shm, st, a);
+    else if (R == 4)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4>), grid, block, shm, st, a);
     else
-        hipLaunchKernelGGL(decode_splitkv_mfma_kernel<false>, grid, block, shm, st, a);
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8>), grid, block, shm, st, a);
     return 0;
 }
 
