@@ -34,15 +34,15 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
                        q_per_kv: int = 4) -> int:
     """Split count that gives every compute unit four workgroups, two resident and two queued
     behind them so that requests of different length even out (a workgroup is four waves of
-    one split; a wave covers one kv head and four of its q heads), but never less than one
+    one split; a wave covers one kv head and all of its q heads, so ``q_per_kv`` does not
+    enter), but never less than one
     64-token step per split (one 32-token group when even that leaves units idle): a wave's time
     is a fixed part plus ~5 us per step, so while compute units are idle more splits are faster;
     and the steps are dealt out evenly (the split length
     is rounded up to whole groups by the kernel, so a careless count leaves splits empty and
     others a step longer).  At most 256, the number of partial states the combine kernel keeps
     on chip."""
-    waves_per_split = int(kv_heads) * max(1, int(q_per_kv) // 4)
-    wgs_per_split = max(1, int(batch) * max(1, waves_per_split // 4))
+    wgs_per_split = max(1, int(batch) * max(1, int(kv_heads) // 4))
     want = max(1, min(256, (4 * int(n_cu)) // wgs_per_split))
     steps = max(1, (int(max_seq_len) + 63) // 64)
     if want >= 2 * steps:          # plenty of idle units: splits of one 32-token group

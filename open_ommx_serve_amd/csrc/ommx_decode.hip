@@ -1,11 +1,10 @@
 // Tuned split-KV decode kernel for gfx950: head_dim 128, 4 or 8 q heads per kv head, 6 (or 0)
 // outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
 //
-// Work decomposition.  A wavefront owns one kv head (and 4 of its q heads) of one split and
-// walks it 64 tokens (two 32-token K groups) at a time; waves never synchronise with each
-// other.  A workgroup is 4 waves = 4 neighbouring kv heads (2 kv heads x 2 q-head groups
-// when a kv head serves 8 q heads), so together they consume whole 128-byte (64-byte) pieces
-// of the token-major k_base / v_main rows.
+// Work decomposition.  A wavefront owns one kv head (and all 4 or 8 of its q heads) of one
+// split and walks it 64 tokens (two 32-token K groups) at a time; waves never synchronise with
+// each other.  A workgroup is 4 waves = 4 neighbouring kv heads, so together they consume whole
+// 128-byte pieces of the token-major k_base / v_main rows.
 //
 // Arithmetic.  All dot products run on the matrix pipe (v_mfma_f32_16x16x32, fp32
 // accumulate) with operands that are EXACT in their 16-bit type:
@@ -19,15 +18,20 @@
 //            outlier position in the staged K rows by 0 or 3 (ds_mskor_b32), so that the base
 //            term of such an element is known, and scatters (outlier - zp - code*2^e)/4 as f16
 //            into a per-group tile [32 tokens][128 channels] that is consumed as the B
-//            operand of an f16 MFMA against A = 4*q (f16).  Deltas too large for one f16
-//            (|delta/4| >= 4, rare) add their rounding residual times q straight onto the
-//            logits through LDS float atomics.
+//            operand of an f16 MFMA against A = 4*q (f16).  Deltas whose f16 rounding could
+//            show on a logit (see BIG_DELTA) add their rounding residual times q straight
+//            onto the logits through LDS float atomics.
 //   P.V      B = (1 + code/4) or (1 + code/16) f16 for 8 tokens of one channel (V rows are
 //            transposed through LDS at dword granularity), A = p * 2^e_v (f16, exact scaling);
 //            sum_t p*vs and sum_t p*vz come from one extra MFMA per 32 tokens.
-// MFMA row groups are used as selectors: rows 4x..4x+3 carry the 4 q heads for token
-// block x (QK) or for V channel group x (P.V); a lane keeps the row group that matches
-// its column.
+// The 16 MFMA rows hold the q heads several times over, and the copies are used as selectors.
+//   4 heads: rows 4x..4x+3 carry the heads for token block x (QK) or with the scales of V
+//            channel group x (P.V); a lane keeps the row group that matches its column.
+//   8 heads: rows 8x..8x+7.  QK: a lane takes two token blocks (kq and kq^1) for the four heads
+//            its result rows hold.  P.V: two row groups cannot tell four channel groups
+//            apart, so the V columns are dealt in two sets (channel groups {0,1} and {2,3}),
+//            each with its own A operand; the MFMA count per token is the same as with 4
+//            heads, only softmax and the A operands double.
 #include <type_traits>
 
 #include "ommx_decode_args.h"
