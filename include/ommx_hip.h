@@ -26,7 +26,12 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 2   /* 2: ring, tail-gather and state-merge entry points */
+#define OMMX_ABI_VERSION 3   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments */
+
+/* outlier index plane (pack.py:23-40, `outlier_repr`) */
+#define OMMX_INDEX_BITMAP   0   /* k_index u8[G,H,D,4]: bit p of the frame = position p (codec.py:330-372) */
+#define OMMX_INDEX_RELIDX7  1   /* k_index u8[G,H,D,ceil(7k/8)]: ascending positions, 7 bits each,
+                                   least significant bit first (pack.py:128-164) */
 
 /* number of floats in the store decision table: 256 pow2 thresholds + 8 FP4 slots */
 #define OMMX_STORE_TABLE_FLOATS 264
@@ -64,8 +69,8 @@ void ommx_store_default_table(float* host_table);
  *   table         float[OMMX_STORE_TABLE_FLOATS] on the device
  *   planes        as written by pack.py:576-623:
  *                 k_base,v_main u8[P,ps,H,D/4]; k_scale i8[G,H,D]; k_zp,k_ms,k_mc bf16[G,H,D];
- *                 k_obmp u8[G,H,D,4]; k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32];
- *                 v_zp bf16[P,ps,H,D/32]
+ *                 k_index as index_repr says (k_obmp or k_oidx of the reference);
+ *                 k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32]; v_zp bf16[P,ps,H,D/32]
  *   err_flag      NULL or int32[1], OR-ed with OMMX_ERR_* (caller zeroes it)
  * k_outliers in 0..8; D a multiple of 32, at most 256; T a multiple of 32 and page_size;
  * 32 % page_size == 0.
@@ -74,18 +79,18 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
                     int64_t k_tok_stride, int64_t k_head_stride,
                     int64_t v_tok_stride, int64_t v_head_stride,
                     const int32_t* src_rows,
-                    int T, int H, int D, int page_size, int k_outliers,
+                    int T, int H, int D, int page_size, int k_outliers, int index_repr,
                     const int32_t* dst_pages, const int32_t* dst_groups,
                     const float* table,
                     uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
-                    uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_obmp, uint8_t* k_oval,
+                    uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index, uint8_t* k_oval,
                     uint8_t* v_main, int8_t* v_scale, uint16_t* v_zp,
                     int32_t* err_flag, void* stream);
 
 /*
  * Split-KV decode over the packed planes (stage 1).
  *   q             bf16 [B,Hq,D], strides q_stride_b, q_stride_h, D contiguous
- *   planes        contiguous, layouts as above; k_outliers in 0..8 with the bitmap index
+ *   planes        contiguous, layouts as above; k_outliers in 0..8 with either index
  *                 plane, dedicated FP4 map and int8 exponents (the serving recipe)
  *   req_to_token  int32 or int64 (table_i64) [B, >= ceil((L+off)/ps)], row stride rt_stride
  *   req_to_group  same type [B, >= seg_group_base + ceil(L/32)], row stride rg_stride
@@ -101,7 +106,7 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
                         const uint16_t* k_ms, const uint16_t* k_mc,
-                        const uint8_t* k_obmp, const uint8_t* k_oval,
+                        const uint8_t* k_index, const uint8_t* k_oval,
                         const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
                         const void* req_to_token, int64_t rt_stride,
                         const void* req_to_group, int64_t rg_stride, int table_i64,
@@ -109,7 +114,7 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
                         float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,
                         int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                        int num_splits, float sm_scale, float logit_cap,
+                        int index_repr, int num_splits, float sm_scale, float logit_cap,
                         int packed_start_offset, int seg_group_base, void* stream);
 
 /*
@@ -120,7 +125,7 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
 int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                             const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
                             const uint16_t* k_ms, const uint16_t* k_mc,
-                            const uint8_t* k_obmp, const uint8_t* k_oval,
+                            const uint8_t* k_index, const uint8_t* k_oval,
                             const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
                             const void* req_to_token, int64_t rt_stride,
                             const void* req_to_group, int64_t rg_stride, int table_i64,
@@ -128,7 +133,7 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
                             float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                             int64_t al_stride_s,
                             int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                            int num_splits, float sm_scale, float logit_cap,
+                            int index_repr, int num_splits, float sm_scale, float logit_cap,
                             int packed_start_offset, int seg_group_base, void* stream);
 
 /*

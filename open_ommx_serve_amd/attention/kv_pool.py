@@ -61,7 +61,7 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"k_format={k_format!r}")
     if str(v_format).lower() != "i2":
         bad.append(f"v_format={v_format!r}")
-    if k > 0 and str(outlier_repr).lower() != "bitmap":
+    if k > 0 and str(outlier_repr).lower() not in ("bitmap", "relidx7"):
         bad.append(f"outlier_repr={outlier_repr!r}")
     if k > 0 and str(outlier_select).lower() != "signed":
         bad.append(f"outlier_select={outlier_select!r}")
@@ -161,7 +161,12 @@ class MultiSeqKVPool:
         if self.k > 0:
             self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
             self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-            self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
+            # index plane of the recipe: flat bitmask, or 7-bit position streams (pack.py:128-164)
+            if self.outlier_repr == "relidx7":
+                self.k_obmp = None
+                self.k_oidx = z(self.G_cap, self.H, self.D, (7 * self.k + 7) // 8, dtype=torch.uint8, device=dev)
+            else:
+                self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             self.k_oval = z(self.G_cap, self.H, self.D, (self.k + 1) // 2, dtype=torch.uint8, device=dev)
         else:
             self.k_fp4_mapscale = self.k_fp4_mapcenter = self.k_obmp = self.k_oval = None
@@ -223,7 +228,7 @@ class MultiSeqKVPool:
     def _planes_for_store(self) -> dict:
         return {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
                 "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
-                "k_obmp": self.k_obmp, "k_oval": self.k_oval,
+                "k_obmp": self.k_obmp, "k_oidx": self.k_oidx, "k_oval": self.k_oval,
                 "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp}
 
     def _as_rows(self, t: torch.Tensor, what: str) -> torch.Tensor:
@@ -367,6 +372,7 @@ class MultiSeqKVPool:
         flat_k = self.k_hist.view(self.num_seqs * self.S_ring, self.H, self.D)
         flat_v = self.v_hist.view(self.num_seqs * self.S_ring, self.H, self.D)
         store_pack_into(flat_k, flat_v, self._planes_for_store(), outliers_per_vector=self.k,
+                        outlier_repr=self.outlier_repr,
                         page_size=self.ps, src_rows=idx[:n_s], dst_pages=idx[n_s:n_s + n_p],
                         dst_groups=idx[n_s + n_p:], err_flag=self.err_flag, num_tokens=n_s)
 
@@ -401,6 +407,7 @@ class MultiSeqKVPool:
         gp0 = r * self.G_per_seq + g0
         pp0 = r * self.P_per_seq + g0 * self.pages_per_group
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
+                        outlier_repr=self.outlier_repr,
                         page_size=self.ps,
                         dst_pages=self._req_to_token.view(-1)[pp0:pp0 + (g1 - g0) * self.pages_per_group],
                         dst_groups=self._req_to_group.view(-1)[gp0:gp0 + (g1 - g0)],
@@ -444,7 +451,7 @@ class MultiSeqKVPool:
 
         return {
             "k_base": sel(self.k_base, pidx), "k_scale": sel(self.k_scale, gidx),
-            "k_zp": sel(self.k_zp, gidx), "k_oidx": None, "k_crank": None,
+            "k_zp": sel(self.k_zp, gidx), "k_oidx": sel(self.k_oidx, gidx), "k_crank": None,
             "k_oval": sel(self.k_oval, gidx), "k_obmp": sel(self.k_obmp, gidx),
             "k_fp4_mapscale": sel(self.k_fp4_mapscale, gidx),
             "k_fp4_mapcenter": sel(self.k_fp4_mapcenter, gidx),

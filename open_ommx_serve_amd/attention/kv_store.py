@@ -98,7 +98,12 @@ class CanonicalKVStore:
         if self.k > 0:
             self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
             self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-            self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
+            # index plane of the recipe: flat bitmask, or 7-bit position streams (pack.py:128-164)
+            if self.outlier_repr == "relidx7":
+                self.k_obmp = None
+                self.k_oidx = z(self.G_cap, self.H, self.D, (7 * self.k + 7) // 8, dtype=torch.uint8, device=dev)
+            else:
+                self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             self.k_oval = z(self.G_cap, self.H, self.D, (self.k + 1) // 2, dtype=torch.uint8, device=dev)
         else:
             self.k_fp4_mapscale = self.k_fp4_mapcenter = self.k_obmp = self.k_oval = None
@@ -245,7 +250,7 @@ class CanonicalKVStore:
     def _planes_for_store(self) -> dict:
         return {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
                 "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
-                "k_obmp": self.k_obmp, "k_oval": self.k_oval,
+                "k_obmp": self.k_obmp, "k_oidx": self.k_oidx, "k_oval": self.k_oval,
                 "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp}
 
     def _regroup_pack_range(self, g0: int, g1: int) -> None:
@@ -265,6 +270,7 @@ class CanonicalKVStore:
         n_tok = (g1 - g0) * self.gt
         ppg = self.pages_per_group
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
+                        outlier_repr=self.outlier_repr,
                         page_size=self.ps, src_rows=src_rows,
                         dst_pages=self._req_to_token_full.view(-1)[g0 * ppg:g1 * ppg],
                         dst_groups=self._req_to_group_full.view(-1)[g0:g1],
@@ -289,7 +295,7 @@ class CanonicalKVStore:
             return None if t is None else t[:n]
 
         out = {"k_base": self.k_base[:P], "k_scale": self.k_scale[:G], "k_zp": self.k_zp[:G],
-               "k_oidx": None, "k_crank": None, "k_oval": cut(self.k_oval, G),
+               "k_oidx": cut(self.k_oidx, G), "k_crank": None, "k_oval": cut(self.k_oval, G),
                "k_obmp": cut(self.k_obmp, G), "k_fp4_mapscale": cut(self.k_fp4_mapscale, G),
                "k_fp4_mapcenter": cut(self.k_fp4_mapcenter, G),
                "v_main": self.v_main[:P], "v_scale": self.v_scale[:P], "v_zp": self.v_zp[:P],
@@ -302,7 +308,7 @@ class CanonicalKVStore:
     def decode_planes_full(self) -> dict:
         """Full-capacity, fixed-address plane dict (kv_store.py:651-676)."""
         out = {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
-               "k_oidx": None, "k_oval": self.k_oval, "k_crank": None, "k_obmp": self.k_obmp,
+               "k_oidx": self.k_oidx, "k_oval": self.k_oval, "k_crank": None, "k_obmp": self.k_obmp,
                "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
                "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp,
                "req_to_token": self._req_to_token_full, "req_to_group": self._req_to_group_full}

@@ -109,7 +109,8 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                     dst_pages: Optional[torch.Tensor] = None,
                     dst_groups: Optional[torch.Tensor] = None,
                     err_flag: Optional[torch.Tensor] = None,
-                    num_tokens: Optional[int] = None) -> None:
+                    num_tokens: Optional[int] = None,
+                    outlier_repr: str = "bitmap") -> None:
     """Pack ``num_tokens`` (default: all rows) tokens of ``K``/``V`` into ``planes`` in place.
 
     ``src_rows`` int32[T] picks the source row of each packed token (a ring gather);
@@ -117,7 +118,8 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
     and group slot of each logical page / group (identity when ``None``).  No host
     synchronisation happens here: non-finite input or an under-filled outlier set is
     reported by bits OR-ed into ``err_flag`` (int32[1]), which the caller reads when it
-    can afford to.  Launches on the current stream.
+    can afford to.  Launches on the current stream.  ``outlier_repr`` names the index plane
+    that is written: ``planes["k_obmp"]`` (``"bitmap"``) or ``planes["k_oidx"]`` (``"relidx7"``).
     """
     _check_rows("K", K)
     _check_rows("V", V)
@@ -132,24 +134,38 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                               or int(t.numel()) < n or t.device != K.device):
             raise ValueError("index tables must be contiguous int32 device tensors of the right length")
     k = int(outliers_per_vector)
+    index_repr, index_plane = _index_plane(planes, outlier_repr, k)
     lib = _hip.load()
     with torch.cuda.device(K.device):
         rc = lib.ommx_store_pack(
             K.data_ptr(), V.data_ptr(), 1 if K.dtype == torch.float32 else 0,
             K.stride(0), K.stride(1), V.stride(0), V.stride(1),
-            _hip.ptr(src_rows), T, H, D, int(page_size), k,
+            _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr,
             _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
             planes["k_base"].data_ptr(), planes["k_scale"].data_ptr(), planes["k_zp"].data_ptr(),
             _hip.ptr(planes.get("k_fp4_mapscale")), _hip.ptr(planes.get("k_fp4_mapcenter")),
-            _hip.ptr(planes.get("k_obmp")), _hip.ptr(planes.get("k_oval")),
+            _hip.ptr(index_plane), _hip.ptr(planes.get("k_oval")),
             planes["v_main"].data_ptr(), planes["v_scale"].data_ptr(), planes["v_zp"].data_ptr(),
             _hip.ptr(err_flag), _hip.current_stream_ptr(K.device))
     _hip.check(rc, "ommx_store_pack")
 
 
+def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int):
+    """(index_repr code of the C ABI, index plane tensor) for an ``outlier_repr`` name."""
+    repr_l = str(outlier_repr).lower()
+    if repr_l == "bitmap":
+        return _hip.INDEX_BITMAP, planes.get("k_obmp")
+    if repr_l == "relidx7":
+        t = planes.get("k_oidx")
+        if k > 0 and (t is None or int(t.shape[-1]) != (7 * k + 7) // 8):
+            raise ValueError("relidx7 needs a k_oidx plane of ceil(7k/8) bytes per frame")
+        return _hip.INDEX_RELIDX7, t
+    raise NotImplementedError(f"outlier_repr={outlier_repr!r} has no HIP kernel")
+
+
 def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim: int, *,
                  page_size: int = 16, outliers_per_vector: int = 6,
-                 device: Any = "cuda") -> Dict[str, Any]:
+                 device: Any = "cuda", outlier_repr: str = "bitmap") -> Dict[str, Any]:
     """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``."""
     P, G, H, D, ps, k = num_pages, num_group_slots, n_kv_heads, head_dim, page_size, outliers_per_vector
     dev = torch.device(device)
@@ -165,7 +181,10 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
         "k_obmp": None, "k_oval": None, "k_fp4_mapscale": None, "k_fp4_mapcenter": None,
     }
     if k > 0:
-        out["k_obmp"] = torch.empty(G, H, D, 4, dtype=u8, device=dev)
+        if str(outlier_repr).lower() == "relidx7":      # pack.py:128-164: ceil(7k/8) bytes per frame
+            out["k_oidx"] = torch.empty(G, H, D, (7 * k + 7) // 8, dtype=u8, device=dev)
+        else:
+            out["k_obmp"] = torch.empty(G, H, D, 4, dtype=u8, device=dev)
         out["k_oval"] = torch.empty(G, H, D, (k + 1) // 2, dtype=u8, device=dev)
         out["k_fp4_mapscale"] = torch.empty(G, H, D, dtype=bf, device=dev)
         out["k_fp4_mapcenter"] = torch.empty(G, H, D, dtype=bf, device=dev)
@@ -245,7 +264,7 @@ def ommx_pack_kv_canonical_block(
     unsupported = []
     if gt != 32 or gc != 32:
         unsupported.append("group_tokens/group_channels other than 32")
-    if k > 0 and repr_l != "bitmap":
+    if k > 0 and repr_l not in ("bitmap", "relidx7"):
         unsupported.append(f"outlier_repr={repr_l!r}")
     if k > 0 and str(outlier_select).lower() != "signed":
         unsupported.append(f"outlier_select={outlier_select!r}")
@@ -281,10 +300,12 @@ def ommx_pack_kv_canonical_block(
     if Vd.stride(-1) != 1:
         Vd = Vd.contiguous()
     G, pages = T // gt, T // int(page_size)
-    planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev)
+    planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev,
+                          outlier_repr=repr_l)
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
-        store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err)
+        store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,
+                        outlier_repr=repr_l)
     raise_for_store_errors(int(err.item()))
 
     def _to(t):
@@ -293,7 +314,7 @@ def ommx_pack_kv_canonical_block(
     out = {name: _to(planes[name]) for name in (
         "k_base", "k_scale", "k_zp", "k_oidx", "k_oval", "k_crank", "k_obmp",
         "k_fp4_mapscale", "k_fp4_mapcenter")}
-    out["k_field_bytes"] = (gt + 7) // 8 if k > 0 else 0
+    out["k_field_bytes"] = (gt + 7) // 8 if (k > 0 and repr_l == "bitmap") else 0    # pack.py:468,568
     out.update({name: _to(planes[name]) for name in ("v_main", "v_scale", "v_zp")})
     out.update(
         req_to_token=torch.arange(pages, dtype=torch.int32, device=device).reshape(1, pages),

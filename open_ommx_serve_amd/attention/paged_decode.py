@@ -157,8 +157,10 @@ def ommx_paged_decode_attention_canonical(
     unsupported = []
     if group_tokens != 32 or group_channels != 32:
         unsupported.append("group sizes other than 32")
-    if k > 0 and not bitmap_read:
-        unsupported.append("relidx7 / combinadic outlier index planes")
+    if k > 0 and combinadic_read:
+        unsupported.append("combinadic outlier index plane")
+    if k > 8:
+        unsupported.append("more than 8 outliers per vector")
     if k > 0 and not use_map:
         unsupported.append("base-shared outliers (kv_outlier_map=False)")
     if k_scale.dtype != torch.int8 or v_scale.dtype != torch.int8:
@@ -172,7 +174,12 @@ def ommx_paged_decode_attention_canonical(
     if unsupported:
         raise NotImplementedError(
             "the HIP decode kernel implements the serving recipe only; not: " + ", ".join(unsupported))
-    for name, t in (("k_scale", k_scale), ("k_zp", k_zp), ("k_oval", k_oval), ("k_obmp", k_obmp),
+    # which index plane the kernels read (paged_decode.py:945-968 bitmap, :843-913 relidx7)
+    k_index, index_repr = (k_obmp, _hip.INDEX_BITMAP) if bitmap_read else (k_oidx, _hip.INDEX_RELIDX7)
+    if k > 0 and (k_index.dtype != torch.uint8 or tuple(k_index.shape[:3]) != tuple(k_scale.shape)
+                  or int(k_index.shape[-1]) != (4 if bitmap_read else (7 * k + 7) // 8)):
+        raise ValueError("outlier index plane must be u8 [group_slots, Hkv, D, 4 (bitmap) or ceil(7k/8) (relidx7)]")
+    for name, t in (("k_scale", k_scale), ("k_zp", k_zp), ("k_oval", k_oval), ("k_index", k_index),
                     ("k_fp4_mapscale", k_fp4_mapscale), ("k_fp4_mapcenter", k_fp4_mapcenter)):
         if t is not None and not t.is_contiguous():
             raise ValueError(f"{name} must be contiguous")
@@ -217,14 +224,14 @@ def ommx_paged_decode_attention_canonical(
             q.data_ptr(), q.stride(0), q.stride(1),
             k_base.data_ptr(), k_scale.data_ptr(), k_zp.data_ptr(),
             _hip.ptr(k_fp4_mapscale) if k > 0 else None, _hip.ptr(k_fp4_mapcenter) if k > 0 else None,
-            _hip.ptr(k_obmp) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
+            _hip.ptr(k_index) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
             v_main.data_ptr(), v_scale.data_ptr(), v_zp.data_ptr(),
             req_to_token.data_ptr(), req_to_token.stride(0),
             req_to_group.data_ptr(), req_to_group.stride(0),
             1 if req_to_token.dtype == torch.int64 else 0,
             b_seq_len.data_ptr(),
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            B, Hq, Hkv, D, ps, k, S, float(sm_scale), float(logit_cap), off, gbase, stream)
+            B, Hq, Hkv, D, ps, k, index_repr, S, float(sm_scale), float(logit_cap), off, gbase, stream)
         _hip.check(rc, "ommx_decode_splitkv")
         rc = lib.ommx_decode_combine(
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),

@@ -269,7 +269,9 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
     return (sh & ((Y & 1) ? 0x03000300u : 0x00C000C0u)) | one_f16x2;
 }
 
-template <bool OUTLIERS, int HR>          // HR: q heads per kv head (4 or 8), all on one wave
+// HR: q heads per kv head (4 or 8), all on one wave.  IDX: 0 = outlier positions from 32-bit
+// bitmaps, 1 = from 7-bit position streams (6 bytes per channel and group at 6 outliers).
+template <bool OUTLIERS, int HR, int IDX>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -357,6 +359,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // channel pair (2*lane, 2*lane+1) parameters of both groups
     uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
     u32x2 g_bm[2], g_ov[2];
+    uint32_t g_bx[2];                     // third index dword (position streams only)
     // (the group index is wave-uniform: base addresses are formed on the scalar unit, the lane
     // adds a 32-bit byte offset)
     const uint32_t kvh_s = __builtin_amdgcn_readfirstlane(kvh);
@@ -373,7 +376,13 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             if (OUTLIERS) {
                 g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
                 g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
-                g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
+                if constexpr (IDX == 0) {
+                    g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
+                } else {          // 12 bytes: the streams of both channels
+                    const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp + gidx * 6, 12 * lane_b));
+                    g_bm[g] = u32x2{ixp[0], ixp[1]};
+                    g_bx[g] = ixp[2];
+                }
                 const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
                 g_ov[g] = u32x2{ovp[0], ovp[1]};
             }
@@ -543,6 +552,12 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const float a1 = 0.25f * __builtin_amdgcn_rcpf(ms);
                         const float b1 = 0.25f * (mc - zp);
                         uint32_t bm = g_bm[g][u];
+                        // position stream of this channel: 42 bits from bit 0 (u = 0) or bit 48
+                        uint32_t ix_lo = 0, ix_hi = 0;
+                        if constexpr (IDX == 1) {
+                            ix_lo = u ? __builtin_amdgcn_alignbit(g_bx[g], g_bm[g][1], 16) : g_bm[g][0];
+                            ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
+                        }
                         // 6 nibbles of this channel: bytes 3c..3c+2 of the block
                         const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
                         const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
@@ -562,8 +577,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 32 * HR;
 #pragma unroll
                         for (int sidx = 0; sidx < 6; ++sidx) {
-                            const int pos = __builtin_ctz(bm) & 31;     // v_ffbl_b32
-                            bm &= bm - 1;
+                            int pos;
+                            if constexpr (IDX == 0) {
+                                pos = __builtin_ctz(bm) & 31;           // v_ffbl_b32
+                                bm &= bm - 1;
+                            } else {                                    // bits [7s, 7s+5) of the stream
+                                pos = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
+                                    : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
+                                                : ((ix_hi >> 3) & 31);
+                            }
                             const float dl0 = fmaf(lv[sidx], a1, b1);
                             const bool top = dl0 > thr;
                             const float dl = top ? dl0 - s34 : dl0;
@@ -836,14 +858,18 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
     const size_t shm = (size_t)waves * (R == 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
                                                : (a.kout == 6 ? LdsMap<8>::END : LdsMap<8>::DT));
-    if (a.kout == 6 && R == 4)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4>), grid, block, shm, st, a);
+    if (a.kout == 6 && a.idx_repr == 0 && R == 4)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, 0>), grid, block, shm, st, a);
+    else if (a.kout == 6 && a.idx_repr == 0)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8, 0>), grid, block, shm, st, a);
+    else if (a.kout == 6 && R == 4)
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, 1>), grid, block, shm, st, a);
     else if (a.kout == 6)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8>), grid, block, shm, st, a);
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8, 1>), grid, block, shm, st, a);
     else if (R == 4)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4>), grid, block, shm, st, a);
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4, 0>), grid, block, shm, st, a);
     else
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8>), grid, block, shm, st, a);
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8, 0>), grid, block, shm, st, a);
     return 0;
 }
 

@@ -7,7 +7,9 @@ namespace ommx {
 struct DecodeArgs {
     const uint16_t* q; int64_t q_sb, q_sh;
     const uint8_t* k_base; const int8_t* k_scale; const uint16_t* k_zp;
-    const uint16_t* k_ms; const uint16_t* k_mc; const uint8_t* k_obmp; const uint8_t* k_oval;
+    const uint16_t* k_ms; const uint16_t* k_mc;
+    const uint8_t* k_obmp;           // index plane: 4-byte bitmaps, or 7-bit position streams (idx_repr 1)
+    const uint8_t* k_oval;
     const uint8_t* v_main; const int8_t* v_scale; const uint16_t* v_zp;
     const void* rt; int64_t rt_s; const void* rg; int64_t rg_s; int i64;
     const int32_t* seq;
@@ -15,7 +17,11 @@ struct DecodeArgs {
     int B, Hq, Hkv, ps, kout, S;
     float sm_scale, cap;
     int off, gbase;
+    int idx_repr;                    // 0 flat bitmap, 1 relidx7
 };
+
+// 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)
+__host__ __device__ constexpr int relidx7_bytes(int k) { return (7 * k + 7) / 8; }
 
 __device__ __forceinline__ int64_t table_at(const void* t, int64_t i, int i64) {
     return i64 ? static_cast<const int64_t*>(t)[i] : static_cast<const int32_t*>(t)[i];

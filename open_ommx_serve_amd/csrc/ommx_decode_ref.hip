@@ -79,7 +79,16 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
 
         if (a.kout > 0 && tid < D) {   // outlier splice: thread = channel
             const int nval = (a.kout + 1) >> 1;
-            uint32_t bm = reinterpret_cast<const uint32_t*>(a.k_obmp)[gidx0 + tid];
+            uint32_t bm = 0;
+            if (a.idx_repr == 0) {
+                bm = reinterpret_cast<const uint32_t*>(a.k_obmp)[gidx0 + tid];
+            } else {               // 7-bit position stream -> the same occupancy mask
+                const int nidx = relidx7_bytes(a.kout);
+                const uint8_t* ip = a.k_obmp + (gidx0 + tid) * nidx;
+                uint64_t stream = 0;
+                for (int j = 0; j < nidx; ++j) stream |= static_cast<uint64_t>(ip[j]) << (8 * j);
+                for (int s = 0; s < a.kout; ++s) bm |= 1u << ((stream >> (7 * s)) & 31u);
+            }
             const uint8_t* ov = a.k_oval + (gidx0 + tid) * nval;
             uint32_t nib = 0;
             for (int j = 0; j < nval; ++j) nib |= static_cast<uint32_t>(ov[j]) << (8 * j);

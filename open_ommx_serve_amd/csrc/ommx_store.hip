@@ -28,7 +28,7 @@ struct StoreArgs {
     uint16_t* k_zp;
     uint16_t* k_ms;
     uint16_t* k_mc;
-    uint8_t* k_obmp;
+    uint8_t* k_obmp;        // index plane: bitmaps [G,H,D,4], or 7-bit streams [G,H,D,ceil(7k/8)]
     uint8_t* k_oval;
     uint8_t* v_main;
     int8_t* v_scale;
@@ -36,6 +36,7 @@ struct StoreArgs {
     int32_t* err;
     int H, D, ps, kout;
     int v_vec;              // V rows allow 16-byte loads
+    int idx_repr;           // 0 flat bitmap (codec.py:330-372), 1 relidx7 (pack.py:128-164)
 };
 
 template <bool F32>
@@ -94,6 +95,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
     const int D = a.D;
     uint8_t* s_codes = smem;                       // [32][D] one code per byte
     uint8_t* s_oval = smem + 32 * D;               // [D][4] nibble bytes (3 used at k=6)
+    uint8_t* s_oidx = smem + 36 * D;               // [D][8] position stream bytes (relidx7 only)
     const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int NGV = D >> 5;
     const int kout = a.kout, kt = (kout + 1) >> 1, kb = kout - kt;
@@ -254,7 +256,17 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (kout > 0) {
             a.k_ms[gidx] = ms_b;
             a.k_mc[gidx] = mc_b;
-            reinterpret_cast<uint32_t*>(a.k_obmp)[gidx] = om;      // byte p>>3, bit p&7
+            if (a.idx_repr == 0) {
+                reinterpret_cast<uint32_t*>(a.k_obmp)[gidx] = om;  // byte p>>3, bit p&7
+            } else {               // ascending positions, 7 bits each, least significant first
+                uint64_t stream = 0;
+                uint32_t m = om;
+                for (int s = 0; s < kout; ++s) {
+                    stream |= static_cast<uint64_t>(__ffs(m) - 1) << (7 * s);
+                    m &= m - 1;
+                }
+                reinterpret_cast<uint64_t*>(s_oidx)[d] = stream;
+            }
             reinterpret_cast<uint32_t*>(s_oval)[d] = nib;
         }
     }
@@ -265,6 +277,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const int64_t obase = (gs * a.H + h) * (int64_t)D * nval;
         for (int b = tid; b < D * nval; b += D)
             a.k_oval[obase + b] = s_oval[(b / nval) * 4 + (b % nval)];
+        if (a.idx_repr != 0) {     // D frames of nidx bytes, contiguous in memory
+            const int nidx = (7 * kout + 7) / 8;
+            const int64_t ibase = (gs * a.H + h) * (int64_t)D * nidx;
+            for (int b = tid; b < D * nidx; b += D)
+                a.k_obmp[ibase + b] = s_oidx[(b / nidx) * 8 + (b % nidx)];
+        }
     }
 
     // ------------------------------------------------- k_base rows and the V vector
@@ -366,10 +384,10 @@ extern "C" void ommx_store_default_table(float* t) {
 extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                                int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
                                const int32_t* src_rows, int T, int H, int D, int page_size,
-                               int k_outliers, const int32_t* dst_pages,
+                               int k_outliers, int index_repr, const int32_t* dst_pages,
                                const int32_t* dst_groups, const float* table,
                                uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
-                               uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_obmp,
+                               uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index,
                                uint8_t* k_oval, uint8_t* v_main, int8_t* v_scale,
                                uint16_t* v_zp, int32_t* err_flag, void* stream) {
     using namespace ommx;
@@ -382,22 +400,24 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
         return -1;
     }
     if (k_outliers < 0 || k_outliers > 8) {
-        set_error("ommx_store_pack: outliers_per_vector must be in [0,8] for the bitmap plane");
+        set_error("ommx_store_pack: outliers_per_vector must be in [0,8]");
         return -1;
     }
+    if (index_repr != 0 && index_repr != 1) { set_error("ommx_store_pack: index_repr"); return -1; }
     if (in_dtype != 0 && in_dtype != 1) { set_error("ommx_store_pack: in_dtype"); return -1; }
     if (!K || !V || !table || !k_base || !k_scale || !k_zp || !v_main || !v_scale || !v_zp ||
-        (k_outliers > 0 && (!k_ms || !k_mc || !k_obmp || !k_oval))) {
+        (k_outliers > 0 && (!k_ms || !k_mc || !k_index || !k_oval))) {
         set_error("ommx_store_pack: null plane or input pointer");
         return -1;
     }
     if (T == 0) return 0;
     StoreArgs a{K, V, k_ts, k_hs, v_ts, v_hs, src_rows, dst_pages, dst_groups, table,
-                k_base, k_scale, k_zp, k_ms, k_mc, k_obmp, k_oval, v_main, v_scale, v_zp,
+                k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval, v_main, v_scale, v_zp,
                 err_flag, H, D, page_size, k_outliers,
-                (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0};
+                (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0,
+                index_repr};
     const dim3 grid(T / 32, H), block(D);
-    const size_t shm = 32 * (size_t)D + 4 * (size_t)D;
+    const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (in_dtype == 1)
         hipLaunchKernelGGL((store_pack_kernel<true, false>), grid, block, shm, st, a);

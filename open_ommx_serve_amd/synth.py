@@ -67,13 +67,15 @@ class DecodeCase:
     head_dim: int
     seq_lens: List[int]
     outliers_per_vector: int = 6
+    outlier_repr: str = "bitmap"
     extra: Dict[str, Any] = field(default_factory=dict)
 
     def decode_kwargs(self) -> Dict[str, Any]:
         p = self.planes
         return dict(sm_scale=self.sm_scale, page_size=self.page_size,
                     k_outliers_per_vector=self.outliers_per_vector, k_format="i2f4",
-                    bitmap_read=self.outliers_per_vector > 0, k_obmp=p["k_obmp"],
+                    bitmap_read=self.outliers_per_vector > 0 and self.outlier_repr == "bitmap",
+                    k_obmp=p["k_obmp"],
                     k_fp4_mapscale=p["k_fp4_mapscale"], k_fp4_mapcenter=p["k_fp4_mapcenter"],
                     kv_outlier_map=self.outliers_per_vector > 0, kv_int8_scale=True,
                     max_seq_len=max(1, int(max(self.packed_lens))),
@@ -85,7 +87,7 @@ class DecodeCase:
 
     def decode_args(self, o: torch.Tensor, lse: torch.Tensor):
         p = self.planes
-        return (self.q, p["k_base"], p["k_scale"], p["k_zp"], None, p["k_oval"],
+        return (self.q, p["k_base"], p["k_scale"], p["k_zp"], p.get("k_oidx"), p["k_oval"],
                 p["v_main"], p["v_scale"], p["v_zp"], self.k_tail, self.v_tail, self.b_tail_len,
                 o, lse, self.req_to_token, self.req_to_group, self.b_seq_len)
 
@@ -94,7 +96,8 @@ class DecodeCase:
         bf16 tail rows (K and V); q, partials and outputs are not counted."""
         D, H, k = self.head_dim, self.kv_heads, self.outliers_per_vector
         per_tok = D // 4 + D // 4 + D // 32 + 2 * (D // 32)
-        per_grp = D * (1 + 2 + (2 + 2 + 4 + (k + 1) // 2 if k > 0 else 0))
+        nidx = 4 if self.outlier_repr == "bitmap" else (7 * k + 7) // 8
+        per_grp = D * (1 + 2 + (2 + 2 + nidx + (k + 1) // 2 if k > 0 else 0))
         tails = [int(x) for x in self.b_tail_len.tolist()]
         tot = 0
         for L, tl in zip(self.packed_lens, tails):
@@ -107,7 +110,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       permute_tables: bool = False, sparse_frac: float = 0.0,
                       outliers_per_vector: int = 6, window: Optional[WindowSpec] = None,
                       device: Any = "cuda", keep_source: bool = False,
-                      table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0) -> DecodeCase:
+                      table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
+                      outlier_repr: str = "bitmap") -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -127,7 +131,9 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     # group slots follow their pages only through the tables, so shuffle them separately
     group_ids = g.permutation(tot_groups) if permute_tables else np.arange(tot_groups)
     planes = alloc_planes(tot_pages, tot_groups, H, D, page_size=ps,
-                          outliers_per_vector=outliers_per_vector, device=dev)
+                          outliers_per_vector=outliers_per_vector, device=dev,
+                          outlier_repr=outlier_repr)
+    planes["outlier_repr"] = str(outlier_repr).lower()
     for t in planes.values():
         if torch.is_tensor(t):
             t.zero_()
@@ -158,7 +164,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
             store_pack_into(Kd, Vd, planes, outliers_per_vector=outliers_per_vector, page_size=ps,
                             dst_pages=torch.from_numpy(rt[b, :n_pages[b]].astype(np.int32)).to(dev),
                             dst_groups=torch.from_numpy(rg[b, :n_groups[b]].astype(np.int32)).to(dev),
-                            err_flag=err)
+                            err_flag=err, outlier_repr=outlier_repr)
         po += n_pages[b]
         go += n_groups[b]
         if keep_source:
@@ -173,6 +179,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
         b_seq_len=torch.tensor(packed, dtype=torch.int32, device=dev),
         sm_scale=1.0 / math.sqrt(D), page_size=ps, q_heads=q_heads, kv_heads=H, head_dim=D,
         seq_lens=[int(x) for x in seq_lens], outliers_per_vector=outliers_per_vector,
+        outlier_repr=str(outlier_repr).lower(),
         extra={"packed_lens": packed, "window": win})
     if keep_source:
         case.extra["source"] = src

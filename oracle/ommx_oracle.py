@@ -16,6 +16,9 @@ Parity status of each function (what pins it, besides reading):
                                nearest-in-log check            (tests/test_oracle_codec.py)
   pack_int2 / unpack_int2      closed form, round trip
   bitmap_pack / bitmap_unpack  closed form, popcount / rank-rule invariants
+  relidx7_pack / relidx7_unpack  closed form (7-bit LSB-first stream) against big-integer
+                               arithmetic and hand-computed bytes; positions equal the
+                               bitmap's for the same input     (tests/test_oracle_codec.py)
   pow2_exponent                rule 2^rint(log2(x)) incl. exact-tie vectors
   select_outliers_signed       brute-force rank counting on small vectors with ties
   pack_kv                      golden planes written by the reference packer itself
@@ -118,6 +121,40 @@ def bitmap_unpack(bmp: torch.Tensor, k: int, n: int = GROUP_TOKENS) -> torch.Ten
     return torch.where(occ, idx, torch.full_like(idx, n)).sort(-1)[0][..., :k]
 
 
+def relidx7_pack(pos: torch.Tensor) -> torch.Tensor:
+    """Ascending positions ``[..., k]`` -> ``[..., ceil(7k/8)]`` bytes: position s occupies
+    bits [7s, 7s+7) of a little-endian bit stream, least significant bit first.
+    pack.py:128-164, codec.py:91-107."""
+    p = pos.to(torch.int64)
+    if bool((p < 0).any()) or bool((p > 127).any()):
+        raise ValueError("relidx7_pack: position out of range")
+    k = int(p.shape[-1])
+    nbytes = (7 * k + 7) // 8
+    bits = ((p.unsqueeze(-1) >> torch.arange(7, dtype=torch.int64)) & 1).reshape(*p.shape[:-1], 7 * k)
+    pad = nbytes * 8 - 7 * k
+    if pad:
+        bits = torch.cat([bits, torch.zeros(*p.shape[:-1], pad, dtype=torch.int64)], dim=-1)
+    w = 1 << torch.arange(8, dtype=torch.int64)
+    return (bits.reshape(*p.shape[:-1], nbytes, 8) * w).sum(-1).to(torch.uint8)
+
+
+def relidx7_unpack(plane: torch.Tensor, k: int) -> torch.Tensor:
+    """Inverse of :func:`relidx7_pack`: ``[..., ceil(7k/8)]`` bytes -> positions ``[..., k]``.
+    pack.py:167-174, codec.py:110-121."""
+    b = plane.to(torch.int64).unsqueeze(-1)
+    bits = ((b >> torch.arange(8, dtype=torch.int64)) & 1).reshape(*plane.shape[:-1], plane.shape[-1] * 8)
+    bits = bits[..., : 7 * k].reshape(*plane.shape[:-1], k, 7)
+    return (bits * (1 << torch.arange(7, dtype=torch.int64))).sum(-1)
+
+
+def outlier_positions(planes: Dict[str, object], gsel, k: int, gt: int = GROUP_TOKENS) -> torch.Tensor:
+    """Ascending outlier positions ``[n, H, D, k]`` of the group slots ``gsel`` from whichever
+    index plane the pack carries (both decode to the same positions, pack.py:323-326)."""
+    if str(planes.get("outlier_repr", "bitmap")).lower() == "relidx7":
+        return relidx7_unpack(planes["k_oidx"][gsel], k)
+    return bitmap_unpack(planes["k_obmp"][gsel], k, gt)
+
+
 def nibbles_pack(val: torch.Tensor) -> torch.Tensor:
     """k 4-bit values ``[..., k]`` -> ``[..., ceil(k/2)]`` bytes, even slot = low nibble.
     pack.py:116-125."""
@@ -181,10 +218,10 @@ def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor,
 
 
 def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
-            outliers_per_vector: int = 6) -> Dict[str, object]:
+            outliers_per_vector: int = 6, outlier_repr: str = "bitmap") -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
-    i2f4, signed select, bitmap index plane, pow2 scales stored as int8 exponents,
-    dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
+    i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
+    exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
 
     ``K``/``V`` are ``[T, H, D]`` bf16 or fp32 with T a multiple of 32 and of
     ``page_size``.  Returns the ten planes, identity tables and the metadata keys.
@@ -210,7 +247,10 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     zp = _bf16_rt(mn)
     code = torch.round((gw - zp) / scale).clamp(0, 3).to(torch.int64)
 
-    planes: Dict[str, object] = {}
+    repr_l = str(outlier_repr).lower()
+    if repr_l not in ("bitmap", "relidx7"):
+        raise ValueError("outlier_repr must be bitmap or relidx7")
+    planes: Dict[str, object] = {"k_oidx": None}
     if k > 0:
         omn, omx = _masked_min_max(gw, omask)
         center = _bf16_rt((omx + omn) / 2.0)
@@ -225,7 +265,11 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         oval = fpc.gather(-1, pos)
         pos = pos.permute(2, 0, 1, 3).contiguous()          # [G,H,D,k]
         oval = oval.permute(2, 0, 1, 3).contiguous()
-        planes["k_obmp"] = bitmap_pack(pos, gt)
+        if repr_l == "bitmap":                              # pack.py:559-573
+            planes["k_obmp"] = bitmap_pack(pos, gt)
+        else:
+            planes["k_obmp"] = None
+            planes["k_oidx"] = relidx7_pack(pos)
         planes["k_oval"] = nibbles_pack(oval)
         planes["k_fp4_mapscale"] = mscale.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
         planes["k_fp4_mapcenter"] = center.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
@@ -254,11 +298,11 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     planes["v_zp"] = vzp.squeeze(-1).to(torch.bfloat16).reshape(pages, page_size, H, NGV).contiguous()
 
     planes.update(
-        k_oidx=None, k_crank=None, k_field_bytes=(gt + 7) // 8 if k > 0 else 0,
+        k_crank=None, k_field_bytes=(gt + 7) // 8 if (k > 0 and repr_l == "bitmap") else 0,
         req_to_token=torch.arange(pages, dtype=torch.int32).reshape(1, pages),
         req_to_group=torch.arange(G, dtype=torch.int32).reshape(1, G),
         head_dim=D, n_kv_heads=H, num_tokens=T, n_groups=G, page_size=int(page_size),
-        outliers_per_vector=k, outlier_repr="bitmap", outlier_select="signed",
+        outliers_per_vector=k, outlier_repr=repr_l, outlier_select="signed",
         group_tokens=gt, group_channels=gc, k_format="i2f4", v_format="i2",
         k_base_bits=2, oval_bits=4, use_pow2=True, kv_outlier_map=k > 0,
         kv_int8_scale=True)
@@ -286,7 +330,7 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
     zp = planes["k_zp"].to(torch.float32)[:G]
     Kd = code * scale.repeat_interleave(gt, 0) + zp.repeat_interleave(gt, 0)
     if k > 0:
-        pos = bitmap_unpack(planes["k_obmp"][:G], k, gt)                     # [G,H,D,k]
+        pos = outlier_positions(planes, slice(0, G), k, gt)                  # [G,H,D,k]
         lvl = fp4_decode(nibbles_unpack(planes["k_oval"][:G], k))
         ms = planes["k_fp4_mapscale"].to(torch.float32)[:G].unsqueeze(-1)
         mc = planes["k_fp4_mapcenter"].to(torch.float32)[:G].unsqueeze(-1)
@@ -401,7 +445,7 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
     k = int(planes["outliers_per_vector"])
     if k > 0:
         Lp = n_g * gt
-        pos = bitmap_unpack(planes["k_obmp"][gs], k, gt)
+        pos = outlier_positions(planes, gs, k, gt)
         lvl = fp4_decode(nibbles_unpack(planes["k_oval"][gs], k))
         ms = planes["k_fp4_mapscale"].to(torch.float32)[gs].unsqueeze(-1)
         mc = planes["k_fp4_mapcenter"].to(torch.float32)[gs].unsqueeze(-1)

@@ -153,6 +153,34 @@ def test_other_head_ratios(ref_kernel):
 
 
 @pytest.mark.parametrize("ref_kernel", [False, True])
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 2)])
+def test_relidx7_index_plane(hq, hkv, ref_kernel):
+    """Positions from the 7-bit streams (k_oidx, bitmap_read=False) instead of the bitmaps:
+    same tolerance against the oracle, and the same result as the bitmap pack of the same
+    cache (the two planes hold the same positions)."""
+    kw = dict(q_heads=hq, kv_heads=hkv, seed=31, permute_tables=True, sparse_frac=0.005)
+    lens = [3000, 72, 1500]
+    case = build_decode_case(lens, outlier_repr="relidx7", **kw)
+    assert case.planes["k_obmp"] is None and case.planes["k_oidx"].shape[-1] == 6
+    assert case.decode_kwargs()["bitmap_read"] is False
+    want = _oracle(case)
+    twin = _run(build_decode_case(lens, **kw), ref_kernel=ref_kernel)
+    for S in (None, 3):
+        got = _run(case, num_kv_splits=S, ref_kernel=ref_kernel)
+        _check(got, want, f"relidx7 S{S}")
+        if S is None:
+            assert (got[0] - twin[0]).abs().max().item() <= 1e-5
+
+
+def test_relidx7_other_outlier_counts_and_head_dim():
+    for k, D in ((3, 64), (8, 128), (1, 64)):
+        case = build_decode_case([700], q_heads=4, kv_heads=2, head_dim=D, seed=32 + k,
+                                 outliers_per_vector=k, outlier_repr="relidx7")
+        assert case.planes["k_oidx"].shape[-1] == (7 * k + 7) // 8
+        _check(_run(case), _oracle(case), f"relidx7 k{k} D{D}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)
     _check(_run(case, ref_kernel=ref_kernel), _oracle(case), "k0")

@@ -33,7 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     for n in names:
         assert getattr(raw, n) is not None, n
     assert set(_hip.exported_symbols()) == set(names)
-    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 2
+    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 3
 
 
 def test_default_decision_table_is_the_exact_arithmetic_one():
@@ -108,7 +108,7 @@ def test_pack_argument_errors_match_the_reference():
     with pytest.raises(ValueError):
         P(K, K, **{**good, "v_format": "fp8"})
     with pytest.raises(NotImplementedError):
-        P(K, K, **{**good, "outlier_repr": "relidx7"})
+        P(K, K, **{**good, "outlier_repr": "combinadic"})
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "use_pow2": False})
     with pytest.raises(NotImplementedError):
@@ -208,8 +208,10 @@ def test_store_classes_refuse_other_recipes_and_the_cpu():
                 outlier_repr="bitmap", use_pow2=True)
     check_serving_recipe(**good, kv_outlier_map=True, kv_int8_scale=True, group_tokens=32,
                          group_channels=32, scale_dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError, match="relidx7"):
-        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "outlier_repr": "relidx7"})
+    with pytest.raises(NotImplementedError, match="combinadic"):
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "outlier_repr": "combinadic"})
+    check_serving_recipe(**{**good, "outlier_repr": "relidx7"}, kv_outlier_map=True, kv_int8_scale=True,
+                         group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError, match="use_pow2"):
         CanonicalKVStore(128, 8, 256, device="cpu", **{**good, "use_pow2": False})
     with pytest.raises(ValueError, match="k_format"):

@@ -134,12 +134,13 @@ def _decode_bundle(q, bundle, sm_scale, k):
     o = torch.full((B, Hq, D), float("nan"), dtype=torch.float32, device=q.device)
     lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=q.device)
     ommx_paged_decode_attention_canonical(
-        q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"],
+        q, pl["k_base"], pl["k_scale"], pl["k_zp"], pl.get("k_oidx"), pl["k_oval"],
         pl["v_main"], pl["v_scale"], pl["v_zp"], bundle["k_tail"], bundle["v_tail"],
         bundle["b_tail_len"], o, lse, bundle.get("req_to_token", pl["req_to_token"]),
         bundle.get("req_to_group", pl["req_to_group"]), bundle["b_seq_len"],
         sm_scale=sm_scale, page_size=pl["page_size"], k_outliers_per_vector=k,
-        bitmap_read=True, k_obmp=pl["k_obmp"], k_fp4_mapscale=pl["k_fp4_mapscale"],
+        bitmap_read=pl.get("outlier_repr", "bitmap") == "bitmap", k_obmp=pl["k_obmp"],
+        k_fp4_mapscale=pl["k_fp4_mapscale"],
         k_fp4_mapcenter=pl["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
         max_seq_len=bundle["max_seq_len"], max_tail_len=bundle["max_tail_len"],
         packed_start_offset=bundle["packed_start_offset"])
@@ -167,14 +168,18 @@ def _oracle_decode(q, K_hist, V_hist, win, sm_scale):
     return torch.stack(outs), torch.stack(lses)
 
 
-def _assert_planes_equal_oracle(got: dict, K, V, win, what):
+def _assert_planes_equal_oracle(got: dict, K, V, win, what, outlier_repr="bitmap"):
     n = int(K.shape[0])
     edge = win.boundary(n)
     assert got["num_tokens"] == max(0, edge - win.sink_tokens), what
     if edge <= win.sink_tokens:
         return
-    want = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size)
+    want = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size,
+                     outlier_repr=outlier_repr)
     for name in PLANE_NAMES:
+        if outlier_repr == "relidx7" and name == "k_obmp":
+            assert got["k_obmp"] is None
+            name = "k_oidx"
         a, b = got[name].cpu(), want[name]
         assert a.shape == b.shape and a.dtype == b.dtype, (what, name)
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{what}: plane {name} differs"
@@ -227,6 +232,47 @@ def test_pool_prefill_then_decode_steps(ring, q_heads):
                                   win, sm_scale)
             _check_out(got, want, f"ring={ring} Hq={q_heads} step {s}")
     pool.check_errors()
+
+
+@pytest.mark.parametrize("ring", [False, True])
+def test_pool_with_the_relidx7_index_plane(ring):
+    """The pool on the 7-bit position-stream recipe: prefill, 40 appended tokens (every request
+    crosses a group boundary), planes against the oracle after every pack, decode at the end
+    of each 10 steps; and a single-sequence store on the same recipe."""
+    H, D, B, q_heads = 8, 128, 2, 32
+    win = WindowSpec()
+    prefill, steps = [300, 71], 40
+    sm_scale = 1.0 / math.sqrt(D)
+    recipe = {**RECIPE, "outlier_repr": "relidx7"}
+    Ks, Vs = zip(*[synth_kv(n + steps, H, D, seed=500 + i, sparse_frac=0.005) for i, n in enumerate(prefill)])
+    pool = MultiSeqKVPool(D, H, num_seqs=2, max_seq_len=400, window=win, device=DEV, kv_ring=ring, **recipe)
+    assert pool.k_obmp is None and tuple(pool.k_oidx.shape[2:]) == (D, 6)
+    for r in range(B):
+        pool.append_block(r, Ks[r][:prefill[r]].to(DEV), Vs[r][:prefill[r]].to(DEV))
+        _assert_planes_equal_oracle(pool.request_planes(r), Ks[r][:prefill[r]], Vs[r][:prefill[r]], win,
+                                    f"prefill req {r}", "relidx7")
+    q_all = synth_q(steps, B * q_heads, D, seed=6).reshape(steps, B, q_heads, D)
+    for s in range(steps):
+        newK = torch.stack([Ks[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        newV = torch.stack([Vs[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        packed = pool.append_decode_batched(range(B), newK, newV)
+        cur = [prefill[i] + s + 1 for i in range(B)]
+        if packed:
+            for r in range(B):
+                _assert_planes_equal_oracle(pool.request_planes(r), Ks[r][:cur[r]], Vs[r][:cur[r]], win,
+                                            f"step {s} req {r}", "relidx7")
+        if s % 10 == 9:
+            bundle = pool.decode_inputs_batched(range(B))
+            assert bundle["planes"]["outlier_repr"] == "relidx7"
+            q = q_all[s].to(DEV)
+            want = _oracle_decode(q, [Ks[i][:cur[i]] for i in range(B)], [Vs[i][:cur[i]] for i in range(B)],
+                                  win, sm_scale)
+            _check_out(_decode_bundle(q, bundle, sm_scale, 6), want, f"relidx7 ring={ring} step {s}")
+    pool.check_errors()
+    store = CanonicalKVStore(D, H, max_seq_len=400, window=win, device=DEV, kv_ring=ring, **recipe)
+    store.append_block(Ks[0][:prefill[0]].to(DEV), Vs[0][:prefill[0]].to(DEV))
+    _assert_planes_equal_oracle(store.decode_planes(), Ks[0][:prefill[0]], Vs[0][:prefill[0]], win,
+                                "store", "relidx7")
 
 
 def test_pool_device_counter_path_equals_the_host_path():

@@ -127,6 +127,44 @@ def test_bitmap_layout_popcount_and_rank_rule():
         O.bitmap_unpack(torch.tensor([[0xFF, 0, 0, 0]], dtype=torch.uint8), 6)
 
 
+def test_relidx7_stream_layout_against_big_integers_and_hand_bytes():
+    # hand-computed: 1 -> bits 0..6 = 1000000, 127 -> bits 7..13 all ones
+    assert O.relidx7_pack(torch.tensor([[1, 127]])).tolist() == [[0x81, 0x3F]]
+    # positions 0..5: value sum(p << 7p) written little-endian in ceil(42/8) = 6 bytes
+    assert O.relidx7_pack(torch.tensor([[0, 1, 2, 3, 4, 5]])).tolist() == \
+        [list((sum(p << (7 * p) for p in range(6))).to_bytes(6, "little"))]
+    g = torch.Generator().manual_seed(11)
+    for k in (1, 2, 3, 5, 6, 8):
+        pos = torch.stack([torch.randperm(32, generator=g)[:k].sort()[0] for _ in range(50)])
+        plane = O.relidx7_pack(pos)
+        assert plane.shape == (50, (7 * k + 7) // 8)
+        for row, p in zip(plane.tolist(), pos.tolist()):
+            # the scalar rule of codec.py:91-107 as one big integer
+            assert int.from_bytes(bytes(row), "little") == sum(v << (7 * s) for s, v in enumerate(p))
+        assert torch.equal(O.relidx7_unpack(plane, k), pos)
+    with pytest.raises(ValueError):
+        O.relidx7_pack(torch.tensor([[0, 128]]))
+
+
+def test_relidx7_pack_carries_the_same_positions_and_values_as_the_bitmap_pack():
+    """The index planes are membership-equivalent (pack.py:323-326): same positions, every other
+    plane identical, identical dequantised K."""
+    from open_ommx_serve_amd.synth import synth_kv
+    K, V = synth_kv(128, 2, 64, 77, sparse_frac=0.02)
+    a = O.pack_kv(K, V, outlier_repr="bitmap")
+    b = O.pack_kv(K, V, outlier_repr="relidx7")
+    assert b["k_obmp"] is None and a["k_oidx"] is None
+    assert b["k_oidx"].shape == (4, 2, 64, 6) and b["k_oidx"].dtype == torch.uint8
+    assert b["k_field_bytes"] == 0 and a["k_field_bytes"] == 4          # pack.py:468,568
+    assert torch.equal(O.relidx7_unpack(b["k_oidx"], 6), O.bitmap_unpack(a["k_obmp"], 6))
+    for n in ("k_base", "k_scale", "k_zp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter",
+              "v_main", "v_scale", "v_zp"):
+        assert torch.equal(a[n], b[n]), n
+    Ka, Va = O.dequant_kv(a)
+    Kb, Vb = O.dequant_kv(b)
+    assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
+
+
 def test_nibble_stream_even_slot_low():
     v = torch.tensor([[1, 2, 3, 4, 5, 6]])
     assert O.nibbles_pack(v).tolist() == [[0x21, 0x43, 0x65]]

@@ -46,6 +46,23 @@ def test_store_matches_oracle_random_bf16(seed, T, H, D):
     assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what=f"seed{seed}")
 
 
+@pytest.mark.parametrize("k,T,H,D", [(6, 256, 8, 128), (6, 64, 2, 64), (1, 64, 2, 32), (3, 96, 1, 64),
+                                     (5, 64, 2, 128), (8, 64, 2, 256)])
+def test_store_relidx7_index_plane(k, T, H, D):
+    """The 7-bit position-stream index plane (the reference packer's default ``outlier_repr``):
+    bit-exact against the oracle, every other plane unchanged against the bitmap pack."""
+    K, V = synth_kv(T, H, D, 300 + k, outlier_channels=min(4, D // 8), sparse_frac=0.01)
+    want = O.pack_kv(K, V, outliers_per_vector=k, outlier_repr="relidx7")
+    got = _hip(K, V, outliers_per_vector=k, outlier_repr="relidx7")
+    assert got["k_obmp"] is None and got["outlier_repr"] == "relidx7" and got["k_field_bytes"] == 0
+    assert tuple(got["k_oidx"].shape) == (T // 32, H, D, (7 * k + 7) // 8)
+    for n in ("k_oidx", "k_base", "k_scale", "k_zp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter",
+              "v_main", "v_scale", "v_zp"):
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+    bm = _hip(K, V, outliers_per_vector=k)
+    assert torch.equal(O.relidx7_unpack(got["k_oidx"], k), O.bitmap_unpack(bm["k_obmp"], k))
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
@@ -174,7 +191,7 @@ def test_store_refuses_nonfinite_and_bad_arguments():
     with pytest.raises(ValueError):
         _hip(K, V, outliers_per_vector=33)
     with pytest.raises(NotImplementedError):
-        _hip(K, V, outlier_repr="relidx7")
+        _hip(K, V, outlier_repr="combinadic")
     _hip(K, V)                                     # and a good call still works afterwards
 
 
