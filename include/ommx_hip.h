@@ -71,6 +71,8 @@ void ommx_store_default_table(float* host_table);
  *                 k_base,v_main u8[P,ps,H,D/4]; k_scale i8[G,H,D]; k_zp,k_ms,k_mc bf16[G,H,D];
  *                 k_index as index_repr says (k_obmp or k_oidx of the reference);
  *                 k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32]; v_zp bf16[P,ps,H,D/32]
+ *                 k_ms and k_mc both NULL: base-shared outliers, the FP4 code is taken of
+ *                 (w - zp) / scale and no map planes exist (pack.py:502-506)
  *   err_flag      NULL or int32[1], OR-ed with OMMX_ERR_* (caller zeroes it)
  * k_outliers in 0..8; D a multiple of 32, at most 256; T a multiple of 32 and page_size;
  * 32 % page_size == 0.
@@ -91,7 +93,8 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  * Split-KV decode over the packed planes (stage 1).
  *   q             bf16 [B,Hq,D], strides q_stride_b, q_stride_h, D contiguous
  *   planes        contiguous, layouts as above; k_outliers in 0..8 with either index
- *                 plane, dedicated FP4 map and int8 exponents (the serving recipe)
+ *                 plane, int8 exponents, and the dedicated FP4 map (the serving recipe) or,
+ *                 with k_ms = k_mc = NULL, outliers on the base scale and zero point
  *   req_to_token  int32 or int64 (table_i64) [B, >= ceil((L+off)/ps)], row stride rt_stride
  *   req_to_group  same type [B, >= seg_group_base + ceil(L/32)], row stride rg_stride
  *   b_seq_len     int32[B] packed tokens per request (device; bounds the loop)

@@ -67,8 +67,6 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"outlier_select={outlier_select!r}")
     if not use_pow2:
         bad.append("use_pow2=False")
-    if kv_outlier_map is False and k > 0:
-        bad.append("kv_outlier_map=False")
     if kv_int8_scale is False:
         bad.append("kv_int8_scale=False")
     if group_tokens != 32 or group_channels != 32:
@@ -159,8 +157,11 @@ class MultiSeqKVPool:
         self.k_oidx = None
         self.k_crank = None
         if self.k > 0:
-            self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-            self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+            if self.kv_outlier_map:     # base-shared outliers carry no map planes (pack.py:502-506)
+                self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+                self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+            else:
+                self.k_fp4_mapscale = self.k_fp4_mapcenter = None
             # index plane of the recipe: flat bitmask, or 7-bit position streams (pack.py:128-164)
             if self.outlier_repr == "relidx7":
                 self.k_obmp = None

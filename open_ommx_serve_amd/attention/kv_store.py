@@ -96,8 +96,11 @@ class CanonicalKVStore:
         self.k_oidx = None
         self.k_crank = None
         if self.k > 0:
-            self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-            self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+            if self.kv_outlier_map:     # base-shared outliers carry no map planes (pack.py:502-506)
+                self.k_fp4_mapscale = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+                self.k_fp4_mapcenter = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
+            else:
+                self.k_fp4_mapscale = self.k_fp4_mapcenter = None
             # index plane of the recipe: flat bitmask, or 7-bit position streams (pack.py:128-164)
             if self.outlier_repr == "relidx7":
                 self.k_obmp = None

@@ -165,7 +165,8 @@ def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int):
 
 def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim: int, *,
                  page_size: int = 16, outliers_per_vector: int = 6,
-                 device: Any = "cuda", outlier_repr: str = "bitmap") -> Dict[str, Any]:
+                 device: Any = "cuda", outlier_repr: str = "bitmap",
+                 kv_outlier_map: bool = True) -> Dict[str, Any]:
     """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``."""
     P, G, H, D, ps, k = num_pages, num_group_slots, n_kv_heads, head_dim, page_size, outliers_per_vector
     dev = torch.device(device)
@@ -186,8 +187,9 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
         else:
             out["k_obmp"] = torch.empty(G, H, D, 4, dtype=u8, device=dev)
         out["k_oval"] = torch.empty(G, H, D, (k + 1) // 2, dtype=u8, device=dev)
-        out["k_fp4_mapscale"] = torch.empty(G, H, D, dtype=bf, device=dev)
-        out["k_fp4_mapcenter"] = torch.empty(G, H, D, dtype=bf, device=dev)
+        if kv_outlier_map:       # base-shared outliers carry no map planes (pack.py:502-506)
+            out["k_fp4_mapscale"] = torch.empty(G, H, D, dtype=bf, device=dev)
+            out["k_fp4_mapcenter"] = torch.empty(G, H, D, dtype=bf, device=dev)
     return out
 
 
@@ -270,8 +272,6 @@ def ommx_pack_kv_canonical_block(
         unsupported.append(f"outlier_select={outlier_select!r}")
     if not use_pow2 or not kv_int8_scale:
         unsupported.append("non power-of-two / non int8-exponent scales")
-    if k > 0 and not kv_outlier_map:
-        unsupported.append("kv_outlier_map=False")
     if k > 8:
         unsupported.append("more than 8 outliers per vector")
     if vfmt != "i2":
@@ -301,7 +301,7 @@ def ommx_pack_kv_canonical_block(
         Vd = Vd.contiguous()
     G, pages = T // gt, T // int(page_size)
     planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev,
-                          outlier_repr=repr_l)
+                          outlier_repr=repr_l, kv_outlier_map=bool(kv_outlier_map))
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
         store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,

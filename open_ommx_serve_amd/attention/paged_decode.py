@@ -161,8 +161,6 @@ def ommx_paged_decode_attention_canonical(
         unsupported.append("combinadic outlier index plane")
     if k > 8:
         unsupported.append("more than 8 outliers per vector")
-    if k > 0 and not use_map:
-        unsupported.append("base-shared outliers (kv_outlier_map=False)")
     if k_scale.dtype != torch.int8 or v_scale.dtype != torch.int8:
         unsupported.append("bf16 scale planes (int8 exponents only)")
     if D != Dv or D not in (64, 128) or (Hq // Hkv) not in (1, 2, 4, 8):
@@ -223,7 +221,7 @@ def ommx_paged_decode_attention_canonical(
         rc = splitkv(
             q.data_ptr(), q.stride(0), q.stride(1),
             k_base.data_ptr(), k_scale.data_ptr(), k_zp.data_ptr(),
-            _hip.ptr(k_fp4_mapscale) if k > 0 else None, _hip.ptr(k_fp4_mapcenter) if k > 0 else None,
+            _hip.ptr(k_fp4_mapscale) if use_map else None, _hip.ptr(k_fp4_mapcenter) if use_map else None,
             _hip.ptr(k_index) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
             v_main.data_ptr(), v_scale.data_ptr(), v_zp.data_ptr(),
             req_to_token.data_ptr(), req_to_token.stride(0),

@@ -64,7 +64,7 @@ extern "C" int ommx_decode_splitkv(
         set_error("ommx_decode_splitkv: null pointer");
         return -1;
     }
-    if (k_outliers > 0 && (!k_ms || !k_mc || !k_index || !k_oval)) {
+    if ((k_outliers > 0 && (!k_index || !k_oval)) || (!k_ms != !k_mc)) {
         set_error("ommx_decode_splitkv: outlier planes missing");
         return -1;
     }

@@ -271,7 +271,9 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 
 // HR: q heads per kv head (4 or 8), all on one wave.  IDX: 0 = outlier positions from 32-bit
 // bitmaps, 1 = from 7-bit position streams (6 bytes per channel and group at 6 outliers).
-template <bool OUTLIERS, int HR, int IDX>
+// OWN_MAP: outliers decode through their own (map_scale, centre) pair; false = through the
+// base scale and zero point (level * 2^e + zp), and there are no map planes.
+template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -357,7 +359,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
     };
     // channel pair (2*lane, 2*lane+1) parameters of both groups
-    uint32_t g_sc[2], g_zp[2], g_ms[2], g_mc[2];
+    uint32_t g_sc[2], g_zp[2], g_ms[2] = {0, 0}, g_mc[2] = {0, 0};
+    constexpr bool own_map = OWN_MAP;
     u32x2 g_bm[2], g_ov[2];
     uint32_t g_bx[2];                     // third index dword (position streams only)
     // (the group index is wave-uniform: base addresses are formed on the scalar unit, the lane
@@ -374,8 +377,10 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
             g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
             if (OUTLIERS) {
-                g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
-                g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
+                if (own_map) {
+                    g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
+                    g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
+                }
                 if constexpr (IDX == 0) {
                     g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
                 } else {          // 12 bytes: the streams of both channels
@@ -549,8 +554,10 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
                         const float mc = __uint_as_float(u ? (g_mc[g] & 0xFFFF0000u) : (g_mc[g] << 16));
                         // tile value (outlier - zp)/4 = level * a1 + b1
-                        const float a1 = 0.25f * __builtin_amdgcn_rcpf(ms);
-                        const float b1 = 0.25f * (mc - zp);
+                        const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
+                        const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                        const float a1 = own_map ? 0.25f * __builtin_amdgcn_rcpf(ms) : 0.25f * s;
+                        const float b1 = own_map ? 0.25f * (mc - zp) : 0.0f;
                         uint32_t bm = g_bm[g][u];
                         // position stream of this channel: 42 bits from bit 0 (u = 0) or bit 48
                         uint32_t ix_lo = 0, ix_hi = 0;
@@ -568,8 +575,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         // The 2-bit base code of an outlier position is overwritten (in the staged
                         // K row) by 0 or 3, whichever base value is nearer to the outlier, so the
                         // delta left for the tile is small; the bias terms account for the rest.
-                        const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
-                        const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
                         const float thr = 0.375f * s, s34 = 0.75f * s;
                         const uint32_t field = 3u << (2 * (c & 15));
                         const uint32_t kt = sm_lds + OFF_KT + g * 32 * KT_ROW + 4 * (c >> 4);
@@ -858,18 +863,27 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
     const size_t shm = (size_t)waves * (R == 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
                                                : (a.kout == 6 ? LdsMap<8>::END : LdsMap<8>::DT));
-    if (a.kout == 6 && a.idx_repr == 0 && R == 4)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, 0>), grid, block, shm, st, a);
-    else if (a.kout == 6 && a.idx_repr == 0)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8, 0>), grid, block, shm, st, a);
-    else if (a.kout == 6 && R == 4)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, 1>), grid, block, shm, st, a);
-    else if (a.kout == 6)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 8, 1>), grid, block, shm, st, a);
-    else if (R == 4)
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4, 0>), grid, block, shm, st, a);
-    else
-        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8, 0>), grid, block, shm, st, a);
+    const bool own_map = a.k_ms != nullptr;
+#define OMMX_LAUNCH(HR, IDX, MAP) \
+    hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a)
+    if (a.kout == 6) {
+        const int variant = (R == 8 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0);
+        switch (variant) {
+            case 0: OMMX_LAUNCH(4, 0, false); break;
+            case 1: OMMX_LAUNCH(4, 0, true); break;
+            case 2: OMMX_LAUNCH(4, 1, false); break;
+            case 3: OMMX_LAUNCH(4, 1, true); break;
+            case 4: OMMX_LAUNCH(8, 0, false); break;
+            case 5: OMMX_LAUNCH(8, 0, true); break;
+            case 6: OMMX_LAUNCH(8, 1, false); break;
+            default: OMMX_LAUNCH(8, 1, true); break;
+        }
+    } else if (R == 4) {
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4, 0, true>), grid, block, shm, st, a);
+    } else {
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8, 0, true>), grid, block, shm, st, a);
+    }
+#undef OMMX_LAUNCH
     return 0;
 }
 

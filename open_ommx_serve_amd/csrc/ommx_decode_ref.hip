@@ -92,15 +92,17 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
             const uint8_t* ov = a.k_oval + (gidx0 + tid) * nval;
             uint32_t nib = 0;
             for (int j = 0; j < nval; ++j) nib |= static_cast<uint32_t>(ov[j]) << (8 * j);
-            const float ms = bf16_to_f32(a.k_ms[gidx0 + tid]);
-            const float mc = bf16_to_f32(a.k_mc[gidx0 + tid]);
+            // dedicated map: level / map_scale + centre; else the base scale and zero point
+            const bool own_map = a.k_ms != nullptr;
+            const float ms = own_map ? bf16_to_f32(a.k_ms[gidx0 + tid]) : 0.0f;
+            const float mc = own_map ? bf16_to_f32(a.k_mc[gidx0 + tid]) : 0.0f;
             while (bm) {
                 const int pos = __ffs(bm) - 1;
                 bm &= bm - 1;
                 float lvl = fp4_level(nib & 7u);
                 if (nib & 8u) lvl = -lvl;
                 nib >>= 4;
-                s_K[pos * KS + tid] = __fdiv_rn(lvl, ms) + mc;
+                s_K[pos * KS + tid] = own_map ? __fdiv_rn(lvl, ms) + mc : lvl * s_sc[tid] + s_zp[tid];
             }
         }
         __syncthreads();

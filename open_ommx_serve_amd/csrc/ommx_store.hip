@@ -203,10 +203,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
 
-        // dedicated FP4 map over the outlier lanes (pack.py:486-498)
+        // dedicated FP4 map over the outlier lanes (pack.py:486-498); without map planes the
+        // outliers share the base scale and zero point instead (pack.py:502-506)
+        const bool own_map = a.k_ms != nullptr;
         uint16_t mc_b = 0, ms_b = 0;
         float mc = 0.0f, ms = 0.0f;
-        if (kout > 0) {
+        if (kout > 0 && own_map) {
             mc_b = f32_to_bf16_rne(__fdiv_rn(omx + omn, 2.0f));
             ms_b = f32_to_bf16_rne(__fdiv_rn(12.0f, fmaxf(omx - omn, 1e-8f)));
             mc = bf16_to_f32(mc_b);
@@ -215,6 +217,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
 
         const bool inv_ok = e >= -126 && e <= 126;
         const float inv_scale = exp2_int(inv_ok ? -e : 0);
+        // the value whose FP4 code is stored: (w - centre) * map_scale, or (w - zp) / scale
+        // (a division by a power of two: the same rounding as the exact inverse multiply)
+        auto fp4_input = [&](float wv) {
+            if (own_map) return (wv - mc) * ms;
+            return inv_ok ? (wv - zp) * inv_scale : __fdiv_rn(wv - zp, scale);
+        };
         uint32_t nib = 0;
         bool mfin = true;
         if (FAST6 && fast_done) {
@@ -228,7 +236,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             for (int r = 0; r < 6; ++r) {
                 const int key = r < 3 ? key_hi[r] : key_lo[r - 3];
                 const int pos = r < 3 ? 31 - (key & 31) : (key & 31);
-                const float mapped = (from_ordered_bits(key) - mc) * ms;
+                const float mapped = fp4_input(from_ordered_bits(key));
                 mfin = mfin && is_finite_f32(mapped);
                 const int slot = __popc(om & ((1u << pos) - 1u));
                 nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
@@ -239,7 +247,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             for (int i = 0; i < 32; ++i) {
                 s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, inv_ok));
                 if (kout > 0) {
-                    const float mapped = (w[i] - mc) * ms;
+                    const float mapped = fp4_input(w[i]);
                     mfin = mfin && is_finite_f32(mapped);
                     if ((om >> i) & 1u) {
                         nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
@@ -254,8 +262,10 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         a.k_scale[gidx] = static_cast<int8_t>(e);
         a.k_zp[gidx] = zp_b;
         if (kout > 0) {
-            a.k_ms[gidx] = ms_b;
-            a.k_mc[gidx] = mc_b;
+            if (own_map) {
+                a.k_ms[gidx] = ms_b;
+                a.k_mc[gidx] = mc_b;
+            }
             if (a.idx_repr == 0) {
                 reinterpret_cast<uint32_t*>(a.k_obmp)[gidx] = om;  // byte p>>3, bit p&7
             } else {               // ascending positions, 7 bits each, least significant first
@@ -406,7 +416,7 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
     if (index_repr != 0 && index_repr != 1) { set_error("ommx_store_pack: index_repr"); return -1; }
     if (in_dtype != 0 && in_dtype != 1) { set_error("ommx_store_pack: in_dtype"); return -1; }
     if (!K || !V || !table || !k_base || !k_scale || !k_zp || !v_main || !v_scale || !v_zp ||
-        (k_outliers > 0 && (!k_ms || !k_mc || !k_index || !k_oval))) {
+        (k_outliers > 0 && (!k_index || !k_oval)) || (!k_ms != !k_mc)) {
         set_error("ommx_store_pack: null plane or input pointer");
         return -1;
     }

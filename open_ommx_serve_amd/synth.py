@@ -77,7 +77,8 @@ class DecodeCase:
                     bitmap_read=self.outliers_per_vector > 0 and self.outlier_repr == "bitmap",
                     k_obmp=p["k_obmp"],
                     k_fp4_mapscale=p["k_fp4_mapscale"], k_fp4_mapcenter=p["k_fp4_mapcenter"],
-                    kv_outlier_map=self.outliers_per_vector > 0, kv_int8_scale=True,
+                    kv_outlier_map=self.outliers_per_vector > 0 and p["k_fp4_mapscale"] is not None,
+                    kv_int8_scale=True,
                     max_seq_len=max(1, int(max(self.packed_lens))),
                     max_tail_len=int(self.k_tail.shape[1]))
 
@@ -97,7 +98,8 @@ class DecodeCase:
         D, H, k = self.head_dim, self.kv_heads, self.outliers_per_vector
         per_tok = D // 4 + D // 4 + D // 32 + 2 * (D // 32)
         nidx = 4 if self.outlier_repr == "bitmap" else (7 * k + 7) // 8
-        per_grp = D * (1 + 2 + (2 + 2 + nidx + (k + 1) // 2 if k > 0 else 0))
+        nmap = 4 if self.planes.get("k_fp4_mapscale") is not None else 0
+        per_grp = D * (1 + 2 + (nmap + nidx + (k + 1) // 2 if k > 0 else 0))
         tails = [int(x) for x in self.b_tail_len.tolist()]
         tot = 0
         for L, tl in zip(self.packed_lens, tails):
@@ -111,7 +113,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       outliers_per_vector: int = 6, window: Optional[WindowSpec] = None,
                       device: Any = "cuda", keep_source: bool = False,
                       table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
-                      outlier_repr: str = "bitmap") -> DecodeCase:
+                      outlier_repr: str = "bitmap", kv_outlier_map: bool = True) -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -132,7 +134,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     group_ids = g.permutation(tot_groups) if permute_tables else np.arange(tot_groups)
     planes = alloc_planes(tot_pages, tot_groups, H, D, page_size=ps,
                           outliers_per_vector=outliers_per_vector, device=dev,
-                          outlier_repr=outlier_repr)
+                          outlier_repr=outlier_repr, kv_outlier_map=kv_outlier_map)
     planes["outlier_repr"] = str(outlier_repr).lower()
     for t in planes.values():
         if torch.is_tensor(t):

@@ -218,10 +218,13 @@ def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor,
 
 
 def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
-            outliers_per_vector: int = 6, outlier_repr: str = "bitmap") -> Dict[str, object]:
+            outliers_per_vector: int = 6, outlier_repr: str = "bitmap",
+            kv_outlier_map: bool = True) -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
     i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
     exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
+    ``kv_outlier_map=False`` is the base-shared outlier variant (pack.py:502-506): the FP4 code
+    is taken of ``(w - zp) / scale`` and there are no map planes.
 
     ``K``/``V`` are ``[T, H, D]`` bf16 or fp32 with T a multiple of 32 and of
     ``page_size``.  Returns the ten planes, identity tables and the metadata keys.
@@ -252,10 +255,13 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         raise ValueError("outlier_repr must be bitmap or relidx7")
     planes: Dict[str, object] = {"k_oidx": None}
     if k > 0:
-        omn, omx = _masked_min_max(gw, omask)
-        center = _bf16_rt((omx + omn) / 2.0)
-        mscale = _bf16_rt(12.0 / (omx - omn).clamp_min(1e-8))
-        mapped = (gw - center) * mscale
+        if kv_outlier_map:                                  # pack.py:486-498
+            omn, omx = _masked_min_max(gw, omask)
+            center = _bf16_rt((omx + omn) / 2.0)
+            mscale = _bf16_rt(12.0 / (omx - omn).clamp_min(1e-8))
+            mapped = (gw - center) * mscale
+        else:                                               # pack.py:502-506
+            mapped = (gw - zp) / scale
         fpc = fp4_encode(mapped).to(torch.int64)
         cols = torch.arange(gt).expand_as(gw)
         pos = torch.where(omask, cols, torch.full_like(cols, gt)).sort(-1)[0][..., :k]
@@ -271,8 +277,11 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
             planes["k_obmp"] = None
             planes["k_oidx"] = relidx7_pack(pos)
         planes["k_oval"] = nibbles_pack(oval)
-        planes["k_fp4_mapscale"] = mscale.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
-        planes["k_fp4_mapcenter"] = center.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
+        if kv_outlier_map:
+            planes["k_fp4_mapscale"] = mscale.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
+            planes["k_fp4_mapcenter"] = center.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
+        else:
+            planes["k_fp4_mapscale"] = planes["k_fp4_mapcenter"] = None
     else:
         planes["k_obmp"] = planes["k_oval"] = None
         planes["k_fp4_mapscale"] = planes["k_fp4_mapcenter"] = None
@@ -304,7 +313,7 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         head_dim=D, n_kv_heads=H, num_tokens=T, n_groups=G, page_size=int(page_size),
         outliers_per_vector=k, outlier_repr=repr_l, outlier_select="signed",
         group_tokens=gt, group_channels=gc, k_format="i2f4", v_format="i2",
-        k_base_bits=2, oval_bits=4, use_pow2=True, kv_outlier_map=k > 0,
+        k_base_bits=2, oval_bits=4, use_pow2=True, kv_outlier_map=bool(kv_outlier_map) and k > 0,
         kv_int8_scale=True)
     return planes
 
@@ -332,9 +341,12 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
     if k > 0:
         pos = outlier_positions(planes, slice(0, G), k, gt)                  # [G,H,D,k]
         lvl = fp4_decode(nibbles_unpack(planes["k_oval"][:G], k))
-        ms = planes["k_fp4_mapscale"].to(torch.float32)[:G].unsqueeze(-1)
-        mc = planes["k_fp4_mapcenter"].to(torch.float32)[:G].unsqueeze(-1)
-        dq = lvl / ms + mc
+        if planes.get("k_fp4_mapscale") is not None:                         # pack.py:749-755
+            ms = planes["k_fp4_mapscale"].to(torch.float32)[:G].unsqueeze(-1)
+            mc = planes["k_fp4_mapcenter"].to(torch.float32)[:G].unsqueeze(-1)
+            dq = lvl / ms + mc
+        else:                                                                # pack.py:756-757
+            dq = lvl * scale.unsqueeze(-1) + zp.unsqueeze(-1)
         Kg = Kd.reshape(G, gt, H, D).permute(0, 2, 3, 1).contiguous()        # [G,H,D,gt]
         Kg.scatter_(-1, pos, dq)
         Kd = Kg.permute(0, 3, 1, 2).reshape(T, H, D)
@@ -447,9 +459,13 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
         Lp = n_g * gt
         pos = outlier_positions(planes, gs, k, gt)
         lvl = fp4_decode(nibbles_unpack(planes["k_oval"][gs], k))
-        ms = planes["k_fp4_mapscale"].to(torch.float32)[gs].unsqueeze(-1)
-        mc = planes["k_fp4_mapcenter"].to(torch.float32)[gs].unsqueeze(-1)
-        dq = lvl / ms + mc
+        if planes.get("k_fp4_mapscale") is not None:
+            ms = planes["k_fp4_mapscale"].to(torch.float32)[gs].unsqueeze(-1)
+            mc = planes["k_fp4_mapcenter"].to(torch.float32)[gs].unsqueeze(-1)
+            dq = lvl / ms + mc
+        else:
+            gsc = torch.exp2(planes["k_scale"].to(torch.float32))[gs].unsqueeze(-1)
+            dq = lvl * gsc + planes["k_zp"].to(torch.float32)[gs].unsqueeze(-1)
         Kp = torch.zeros(Lp, H, D, dtype=torch.float32)
         Kp[:L] = Kd
         Kg = Kp.reshape(n_g, gt, H, D).permute(0, 2, 3, 1).contiguous()

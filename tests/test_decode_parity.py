@@ -181,6 +181,18 @@ def test_relidx7_other_outlier_counts_and_head_dim():
 
 
 @pytest.mark.parametrize("ref_kernel", [False, True])
+@pytest.mark.parametrize("hq,hkv,rep", [(32, 8, "bitmap"), (64, 8, "relidx7"), (8, 2, "bitmap")])
+def test_base_shared_outliers(hq, hkv, rep, ref_kernel):
+    """kv_outlier_map=False: outliers decode as level * 2^e + zp, no map planes."""
+    case = build_decode_case([2100, 40, 700], q_heads=hq, kv_heads=hkv, seed=41, permute_tables=True,
+                             sparse_frac=0.005, outlier_repr=rep, kv_outlier_map=False)
+    assert case.planes["k_fp4_mapscale"] is None and case.decode_kwargs()["kv_outlier_map"] is False
+    want = _oracle(case)
+    for S in (None, 4):
+        _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"base-shared S{S}")
+
+
+@pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)
     _check(_run(case, ref_kernel=ref_kernel), _oracle(case), "k0")

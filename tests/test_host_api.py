@@ -170,7 +170,8 @@ def test_decode_argument_errors_precede_any_launch():
         bad = list(args); bad[6] = args[6][:, ::2]
         D(*bad, **{**kw, "page_size": 8})
     with pytest.raises(NotImplementedError, match="serving recipe"):
-        D(*args, **{**kw, "kv_outlier_map": False, "k_fp4_mapscale": None})
+        D(*args, **{**kw, "combinadic_read": True, "bitmap_read": False,
+                    "k_crank": torch.zeros(2, 2, 64, 3, dtype=torch.uint8)})
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             D(*args, **kw)

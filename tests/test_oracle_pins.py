@@ -165,6 +165,36 @@ def test_relidx7_pack_carries_the_same_positions_and_values_as_the_bitmap_pack()
     assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
 
 
+def test_base_shared_outliers_hand_built_vector():
+    """kv_outlier_map=False (pack.py:502-506, dequant :756-757), every stored value derived on
+    paper.  Channel 0 over 32 tokens: base lanes 0, 1, 2, 3 repeating -> min 0, max 3, scale
+    2^0, zp 0.  Outliers (top three, bottom three): +6.5, +4.9, +3.4 and -6, -2.4, -0.2.
+    (w - zp) / scale = w, so the FP4 codes are those of the raw values: 6.5 -> level 6 (code 7),
+    4.9 -> nearest in log to 4 vs 6: boundary sqrt(24) = 4.899 -> 6 (code 7), 3.4 -> boundary
+    sqrt(12) = 3.46 -> 3 (code 5), -6 -> sign | 7 = 15, -2.4 -> boundary sqrt(6) = 2.449 -> 2
+    (code 4 | 8 = 12), -0.2 -> boundary sqrt(0.5e-8)... 0.2 is nearer to 0.5 than to 1e-8 in
+    log -> 0.5 (code 1 | 8 = 9).  Dequant = level * 1 + 0."""
+    w = torch.tensor([float(i % 4) for i in range(32)])
+    put = {3: 6.5, 7: 4.9, 12: 3.4, 16: -6.0, 21: -2.4, 30: -0.2}
+    for p, v in put.items():
+        w[p] = v
+    K = torch.zeros(32, 1, 32)
+    K[:, 0, 0] = w
+    K[:, 0, 1:] = torch.arange(32).float().unsqueeze(1) * 0.01      # other channels: anything finite
+    pl = O.pack_kv(K, K.clone(), kv_outlier_map=False)
+    assert pl["k_fp4_mapscale"] is None and pl["k_fp4_mapcenter"] is None and pl["kv_outlier_map"] is False
+    assert int(pl["k_scale"][0, 0, 0]) == 0 and float(pl["k_zp"][0, 0, 0]) == 0.0
+    assert O.bitmap_unpack(pl["k_obmp"], 6)[0, 0, 0].tolist() == sorted(put)
+    assert O.nibbles_unpack(pl["k_oval"], 6)[0, 0, 0].tolist() == [7, 7, 5, 15, 12, 9]
+    Kd, _ = O.dequant_kv(pl)
+    want = w.clone()
+    for p, v in zip(sorted(put), [6.0, 6.0, 3.0, -6.0, -2.0, -0.5]):
+        want[p] = v
+    assert torch.equal(Kd[:, 0, 0], want)
+    # with the dedicated map the same vector stores other nibbles and planes
+    assert O.pack_kv(K, K.clone())["k_fp4_mapscale"] is not None
+
+
 def test_nibble_stream_even_slot_low():
     v = torch.tensor([[1, 2, 3, 4, 5, 6]])
     assert O.nibbles_pack(v).tolist() == [[0x21, 0x43, 0x65]]

@@ -63,6 +63,21 @@ def test_store_relidx7_index_plane(k, T, H, D):
     assert torch.equal(O.relidx7_unpack(got["k_oidx"], k), O.bitmap_unpack(bm["k_obmp"], k))
 
 
+@pytest.mark.parametrize("k,T,H,D,rep", [(6, 256, 8, 128, "bitmap"), (6, 64, 2, 64, "relidx7"),
+                                         (3, 96, 1, 64, "bitmap"), (8, 64, 2, 256, "bitmap")])
+def test_store_base_shared_outliers(k, T, H, D, rep):
+    """kv_outlier_map=False: the FP4 code of (w - zp) / scale, no map planes (pack.py:502-506)."""
+    K, V = synth_kv(T, H, D, 400 + k, outlier_channels=min(4, D // 8), sparse_frac=0.01)
+    want = O.pack_kv(K, V, outliers_per_vector=k, outlier_repr=rep, kv_outlier_map=False)
+    got = _hip(K, V, outliers_per_vector=k, outlier_repr=rep, kv_outlier_map=False)
+    assert got["k_fp4_mapscale"] is None and got["k_fp4_mapcenter"] is None and got["kv_outlier_map"] is False
+    idx = "k_obmp" if rep == "bitmap" else "k_oidx"
+    for n in (idx, "k_base", "k_scale", "k_zp", "k_oval", "v_main", "v_scale", "v_zp"):
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+    # the nibbles differ from the dedicated-map pack of the same block: it is another code
+    assert not np.array_equal(bits_of(got["k_oval"]), bits_of(_hip(K, V, outliers_per_vector=k)["k_oval"]))
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
