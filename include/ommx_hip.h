@@ -73,6 +73,9 @@ void ommx_store_default_table(float* host_table);
  *                 k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32]; v_zp bf16[P,ps,H,D/32]
  *                 k_ms and k_mc both NULL: base-shared outliers, the FP4 code is taken of
  *                 (w - zp) / scale and no map planes exist (pack.py:502-506)
+ *   select_abs    0: outliers = the ceil(k/2) largest and floor(k/2) smallest values
+ *                 (`outlier_select="signed"`, pack.py:436-445); 1: the k largest magnitudes
+ *                 (`"abs"`, pack.py:446-448); ties go to the lower position either way
  *   err_flag      NULL or int32[1], OR-ed with OMMX_ERR_* (caller zeroes it)
  * k_outliers in 0..8; D a multiple of 32, at most 256; T a multiple of 32 and page_size;
  * 32 % page_size == 0.
@@ -82,7 +85,7 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
                     int64_t v_tok_stride, int64_t v_head_stride,
                     const int32_t* src_rows,
                     int T, int H, int D, int page_size, int k_outliers, int index_repr,
-                    const int32_t* dst_pages, const int32_t* dst_groups,
+                    int select_abs, const int32_t* dst_pages, const int32_t* dst_groups,
                     const float* table,
                     uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
                     uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index, uint8_t* k_oval,

@@ -63,7 +63,7 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"v_format={v_format!r}")
     if k > 0 and str(outlier_repr).lower() not in ("bitmap", "relidx7"):
         bad.append(f"outlier_repr={outlier_repr!r}")
-    if k > 0 and str(outlier_select).lower() != "signed":
+    if k > 0 and str(outlier_select).lower() not in ("signed", "abs"):
         bad.append(f"outlier_select={outlier_select!r}")
     if not use_pow2:
         bad.append("use_pow2=False")
@@ -77,9 +77,10 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"outliers_per_vector={k}")
     if bad:
         raise NotImplementedError(
-            "the HIP KV store implements the serving recipe only (i2f4, signed, bitmap, "
-            "use_pow2, dedicated FP4 map, int8 exponents, 32x32 groups, bf16 zero points, "
-            "0..8 outliers); unsupported: " + ", ".join(bad))
+            "the HIP KV store implements the serving recipe and its near variants only (i2f4, "
+            "signed or abs selection, bitmap or relidx7 index plane, use_pow2 with int8 exponents, "
+            "dedicated or base-shared FP4 outliers, 32x32 groups, bf16 zero points, 0..8 outliers); "
+            "unsupported: " + ", ".join(bad))
 
 
 class MultiSeqKVPool:
@@ -373,7 +374,7 @@ class MultiSeqKVPool:
         flat_k = self.k_hist.view(self.num_seqs * self.S_ring, self.H, self.D)
         flat_v = self.v_hist.view(self.num_seqs * self.S_ring, self.H, self.D)
         store_pack_into(flat_k, flat_v, self._planes_for_store(), outliers_per_vector=self.k,
-                        outlier_repr=self.outlier_repr,
+                        outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         page_size=self.ps, src_rows=idx[:n_s], dst_pages=idx[n_s:n_s + n_p],
                         dst_groups=idx[n_s + n_p:], err_flag=self.err_flag, num_tokens=n_s)
 
@@ -408,7 +409,7 @@ class MultiSeqKVPool:
         gp0 = r * self.G_per_seq + g0
         pp0 = r * self.P_per_seq + g0 * self.pages_per_group
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
-                        outlier_repr=self.outlier_repr,
+                        outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         page_size=self.ps,
                         dst_pages=self._req_to_token.view(-1)[pp0:pp0 + (g1 - g0) * self.pages_per_group],
                         dst_groups=self._req_to_group.view(-1)[gp0:gp0 + (g1 - g0)],

@@ -110,7 +110,7 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                     dst_groups: Optional[torch.Tensor] = None,
                     err_flag: Optional[torch.Tensor] = None,
                     num_tokens: Optional[int] = None,
-                    outlier_repr: str = "bitmap") -> None:
+                    outlier_repr: str = "bitmap", outlier_select: str = "signed") -> None:
     """Pack ``num_tokens`` (default: all rows) tokens of ``K``/``V`` into ``planes`` in place.
 
     ``src_rows`` int32[T] picks the source row of each packed token (a ring gather);
@@ -135,12 +135,15 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
             raise ValueError("index tables must be contiguous int32 device tensors of the right length")
     k = int(outliers_per_vector)
     index_repr, index_plane = _index_plane(planes, outlier_repr, k)
+    sel = str(outlier_select).lower()
+    if sel not in ("signed", "abs"):
+        raise ValueError(f"outlier_select must be signed|abs; got {outlier_select!r}")
     lib = _hip.load()
     with torch.cuda.device(K.device):
         rc = lib.ommx_store_pack(
             K.data_ptr(), V.data_ptr(), 1 if K.dtype == torch.float32 else 0,
             K.stride(0), K.stride(1), V.stride(0), V.stride(1),
-            _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr,
+            _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr, 1 if sel == "abs" else 0,
             _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
             planes["k_base"].data_ptr(), planes["k_scale"].data_ptr(), planes["k_zp"].data_ptr(),
             _hip.ptr(planes.get("k_fp4_mapscale")), _hip.ptr(planes.get("k_fp4_mapcenter")),
@@ -268,7 +271,7 @@ def ommx_pack_kv_canonical_block(
         unsupported.append("group_tokens/group_channels other than 32")
     if k > 0 and repr_l not in ("bitmap", "relidx7"):
         unsupported.append(f"outlier_repr={repr_l!r}")
-    if k > 0 and str(outlier_select).lower() != "signed":
+    if str(outlier_select).lower() not in ("signed", "abs"):
         unsupported.append(f"outlier_select={outlier_select!r}")
     if not use_pow2 or not kv_int8_scale:
         unsupported.append("non power-of-two / non int8-exponent scales")
@@ -305,7 +308,7 @@ def ommx_pack_kv_canonical_block(
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
         store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,
-                        outlier_repr=repr_l)
+                        outlier_repr=repr_l, outlier_select=outlier_select)
     raise_for_store_errors(int(err.item()))
 
     def _to(t):

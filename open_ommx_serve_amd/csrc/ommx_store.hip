@@ -37,6 +37,7 @@ struct StoreArgs {
     int H, D, ps, kout;
     int v_vec;              // V rows allow 16-byte loads
     int idx_repr;           // 0 flat bitmap (codec.py:330-372), 1 relidx7 (pack.py:128-164)
+    int select_abs;         // 0 signed top + bottom tails (pack.py:436-445), 1 largest |w| (pack.py:446-448)
 };
 
 template <bool F32>
@@ -119,6 +120,21 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         uint32_t top = 0, bot = 0;
         int key_hi[3] = {0, 0, 0}, key_lo[3] = {0, 0, 0};    // FAST6: sorted keys of the chosen lanes
         auto select_generic = [&]() {
+            if (a.select_abs) {
+                // the kout largest magnitudes, ties to the lower index (stable descending sort
+                // of |w|, pack.py:446-448)
+                top = bot = 0;
+                for (int r = 0; r < kout; ++r) {
+                    float best = 0.0f; int bi = -1;
+    #pragma unroll
+                    for (int i = 0; i < 32; ++i) {
+                        const bool free_lane = !((top >> i) & 1u);
+                        if (free_lane && (bi < 0 || fabsf(w[i]) > best)) { best = fabsf(w[i]); bi = i; }
+                    }
+                    if (bi >= 0) top |= 1u << bi;
+                }
+                return;
+            }
             // signed select (pack.py:436-445): kt largest, ties to the lower index ...
             top = 0;
             for (int r = 0; r < kt; ++r) {
@@ -394,7 +410,8 @@ extern "C" void ommx_store_default_table(float* t) {
 extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                                int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
                                const int32_t* src_rows, int T, int H, int D, int page_size,
-                               int k_outliers, int index_repr, const int32_t* dst_pages,
+                               int k_outliers, int index_repr, int select_abs,
+                               const int32_t* dst_pages,
                                const int32_t* dst_groups, const float* table,
                                uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
                                uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index,
@@ -425,13 +442,13 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                 k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval, v_main, v_scale, v_zp,
                 err_flag, H, D, page_size, k_outliers,
                 (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0,
-                index_repr};
+                index_repr, select_abs ? 1 : 0};
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (in_dtype == 1)
         hipLaunchKernelGGL((store_pack_kernel<true, false>), grid, block, shm, st, a);
-    else if (k_outliers == 6)
+    else if (k_outliers == 6 && !select_abs)
         hipLaunchKernelGGL((store_pack_kernel<false, true>), grid, block, shm, st, a);
     else
         hipLaunchKernelGGL((store_pack_kernel<false, false>), grid, block, shm, st, a);

@@ -21,6 +21,7 @@ Parity status of each function (what pins it, besides reading):
                                bitmap's for the same input     (tests/test_oracle_codec.py)
   pow2_exponent                rule 2^rint(log2(x)) incl. exact-tie vectors
   select_outliers_signed       brute-force rank counting on small vectors with ties
+  select_outliers_abs          the same, on magnitudes
   pack_kv                      golden planes written by the reference packer itself
                                (tests/golden/*.npz), plus all of the above
   dequant_kv                   golden dequant of the same planes; encode/decode identity
@@ -206,6 +207,16 @@ def select_outliers_signed(gw: torch.Tensor, k: int) -> torch.Tensor:
     return mask
 
 
+def select_outliers_abs(gw: torch.Tensor, k: int) -> torch.Tensor:
+    """Boolean outlier mask: the ``k`` largest magnitudes by stable descending sort of ``|w|``
+    (equal magnitudes keep ascending index order).  pack.py:446-448."""
+    mask = torch.zeros_like(gw, dtype=torch.bool)
+    if k == 0:
+        return mask
+    top = torch.sort(gw.abs(), dim=-1, descending=True, stable=True)[1][..., :k]
+    return mask.scatter_(-1, top, True)
+
+
 def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """min / max over lanes where ``keep``; sentinels +-1e9, an empty set gives 0.
     pack.py:455-458 and 486-489."""
@@ -219,7 +230,7 @@ def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor,
 
 def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
             outliers_per_vector: int = 6, outlier_repr: str = "bitmap",
-            kv_outlier_map: bool = True) -> Dict[str, object]:
+            kv_outlier_map: bool = True, outlier_select: str = "signed") -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
     i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
     exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
@@ -242,7 +253,10 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
 
     # ---- K, vector = (head, channel, group) over 32 tokens            pack.py:428-501
     gw = Kf.permute(1, 2, 0).contiguous().reshape(H, D, G, gt)
-    omask = select_outliers_signed(gw, k)
+    sel = str(outlier_select).lower()
+    if sel not in ("signed", "abs"):
+        raise ValueError("outlier_select must be signed or abs")
+    omask = select_outliers_signed(gw, k) if sel == "signed" else select_outliers_abs(gw, k)
     mn, mx = _masked_min_max(gw, ~omask)
     raw = (mx - mn).clamp_min(1e-8) / 3.0
     e = pow2_exponent(raw)
@@ -311,7 +325,7 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         req_to_token=torch.arange(pages, dtype=torch.int32).reshape(1, pages),
         req_to_group=torch.arange(G, dtype=torch.int32).reshape(1, G),
         head_dim=D, n_kv_heads=H, num_tokens=T, n_groups=G, page_size=int(page_size),
-        outliers_per_vector=k, outlier_repr=repr_l, outlier_select="signed",
+        outliers_per_vector=k, outlier_repr=repr_l, outlier_select=sel,
         group_tokens=gt, group_channels=gc, k_format="i2f4", v_format="i2",
         k_base_bits=2, oval_bits=4, use_pow2=True, kv_outlier_map=bool(kv_outlier_map) and k > 0,
         kv_int8_scale=True)

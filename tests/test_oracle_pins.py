@@ -280,6 +280,30 @@ def test_signed_selection_matches_brute_force_with_heavy_ties(k):
     assert bool((mask.sum(-1) == k).all())
 
 
+@pytest.mark.parametrize("k", [1, 3, 6, 8])
+def test_abs_selection_matches_brute_force_with_heavy_ties(k):
+    """Largest magnitudes, equal magnitudes (of either sign) to the lower index: lane i is chosen
+    iff fewer than k lanes beat it, where j beats i when |w_j| > |w_i| or (equal and j < i)."""
+    g = torch.Generator().manual_seed(21 + k)
+    lv = torch.tensor([-3.0, -1.0, 1.0, 0.0, -0.0, 0.5, -0.5, 2.0, -2.0, 3.0])
+    w = lv[torch.randint(0, 10, (200, 32), generator=g)]
+    w[0] = -1.25
+    w[1, ::2] = -2.0; w[1, 1::2] = 2.0
+    mask = O.select_outliers_abs(w, k)
+    for r in range(w.shape[0]):
+        a = [abs(x) for x in w[r].tolist()]
+        want = [i for i in range(32)
+                if sum(1 for j in range(32) if a[j] > a[i] or (a[j] == a[i] and j < i)) < k]
+        assert mask[r].nonzero().flatten().tolist() == want, r
+    # and through the packer: positions are those lanes, in ascending order
+    K = torch.zeros(32, 1, 32); K[:, 0, :] = w[:32].t()
+    pl = O.pack_kv(K, K.clone(), outliers_per_vector=k, outlier_select="abs")
+    assert pl["outlier_select"] == "abs"
+    pos = O.bitmap_unpack(pl["k_obmp"], k)[0, 0]
+    for c in range(32):
+        assert pos[c].tolist() == mask[c].nonzero().flatten().tolist()
+
+
 def test_base_range_excludes_outliers_and_map_closed_form():
     """One hand-built vector: the scale comes from the 26 inner lanes only, the FP4 map is
     centred on the 6 outliers, and every stored value follows the closed forms."""

@@ -78,6 +78,20 @@ def test_store_base_shared_outliers(k, T, H, D, rep):
     assert not np.array_equal(bits_of(got["k_oval"]), bits_of(_hip(K, V, outliers_per_vector=k)["k_oval"]))
 
 
+@pytest.mark.parametrize("k,T,H,D", [(6, 256, 8, 128), (3, 64, 2, 64), (1, 64, 1, 32), (8, 64, 2, 256)])
+def test_store_abs_selection(k, T, H, D):
+    """outlier_select="abs" (the reference packer's default argument): the k largest magnitudes.
+    Includes a block of heavy ties between values of both signs."""
+    K, V = synth_kv(T, H, D, 500 + k, outlier_channels=min(4, D // 8), sparse_frac=0.01)
+    g = torch.Generator().manual_seed(k)
+    lv = torch.tensor([-3.0, -1.0, 1.0, 0.0, -0.0, 0.5, -0.5, 2.0, -2.0, 3.0])
+    K[:32] = lv[torch.randint(0, 10, (32, H, D), generator=g)].to(torch.bfloat16)
+    want = O.pack_kv(K, V, outliers_per_vector=k, outlier_select="abs")
+    got = _hip(K, V, outliers_per_vector=k, outlier_select="abs")
+    assert got["outlier_select"] == "abs"
+    assert_planes_equal(got, want, what=f"abs k{k}", zero_sign_free=True)
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
