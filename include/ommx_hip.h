@@ -28,6 +28,11 @@ extern "C" {
 
 #define OMMX_ABI_VERSION 3   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments */
 
+/* step of the INT2 quantisers and the dtype of the k_scale / v_scale planes */
+#define OMMX_SCALE_POW2_INT8  0
+#define OMMX_SCALE_POW2_BF16  1
+#define OMMX_SCALE_BF16       2
+
 /* outlier index plane (pack.py:23-40, `outlier_repr`) */
 #define OMMX_INDEX_BITMAP   0   /* k_index u8[G,H,D,4]: bit p of the frame = position p (codec.py:330-372) */
 #define OMMX_INDEX_RELIDX7  1   /* k_index u8[G,H,D,ceil(7k/8)]: ascending positions, 7 bits each,
@@ -73,6 +78,12 @@ void ommx_store_default_table(float* host_table);
  *                 k_oval u8[G,H,D,ceil(k/2)]; v_scale i8[P,ps,H,D/32]; v_zp bf16[P,ps,H,D/32]
  *                 k_ms and k_mc both NULL: base-shared outliers, the FP4 code is taken of
  *                 (w - zp) / scale and no map planes exist (pack.py:502-506)
+ *   scale_mode    how the quantisation step of a vector is formed and stored in k_scale /
+ *                 v_scale (pack.py:459-463, 586-590, 612-623):
+ *                 OMMX_SCALE_POW2_INT8  2^rint(log2(range/3)), int8 exponent planes
+ *                                       (`use_pow2=True`, the serving recipe);
+ *                 OMMX_SCALE_POW2_BF16  the same step stored as bf16 (`kv_int8_scale=False`);
+ *                 OMMX_SCALE_BF16       bf16(range/3) as it comes (`use_pow2=False`), bf16 planes
  *   select_abs    0: outliers = the ceil(k/2) largest and floor(k/2) smallest values
  *                 (`outlier_select="signed"`, pack.py:436-445); 1: the k largest magnitudes
  *                 (`"abs"`, pack.py:446-448); ties go to the lower position either way
@@ -85,11 +96,12 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
                     int64_t v_tok_stride, int64_t v_head_stride,
                     const int32_t* src_rows,
                     int T, int H, int D, int page_size, int k_outliers, int index_repr,
-                    int select_abs, const int32_t* dst_pages, const int32_t* dst_groups,
+                    int select_abs, int scale_mode,
+                    const int32_t* dst_pages, const int32_t* dst_groups,
                     const float* table,
-                    uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
+                    uint8_t* k_base, void* k_scale, uint16_t* k_zp,
                     uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index, uint8_t* k_oval,
-                    uint8_t* v_main, int8_t* v_scale, uint16_t* v_zp,
+                    uint8_t* v_main, void* v_scale, uint16_t* v_zp,
                     int32_t* err_flag, void* stream);
 
 /*
@@ -106,21 +118,22 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 lse=-inf (paged_decode.py:2262-2284)
  * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
  * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64;
- * num_splits <= 256; planes 8-byte aligned.  head_dim 128 with r = 4 or 8 and 6 (or 0)
+ * num_splits <= 256; planes 8-byte aligned.  scale_bf16 = 1: k_scale / v_scale hold the steps
+ * themselves as bf16 instead of int8 exponents (plain kernel only).  head_dim 128 with r = 4 or 8 and 6 (or 0)
  * outliers runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-                        const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+                        const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
                         const uint16_t* k_ms, const uint16_t* k_mc,
                         const uint8_t* k_index, const uint8_t* k_oval,
-                        const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+                        const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
                         const void* req_to_token, int64_t rt_stride,
                         const void* req_to_group, int64_t rg_stride, int table_i64,
                         const int32_t* b_seq_len,
                         float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,
                         int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                        int index_repr, int num_splits, float sm_scale, float logit_cap,
+                        int index_repr, int scale_bf16, int num_splits, float sm_scale, float logit_cap,
                         int packed_start_offset, int seg_group_base, void* stream);
 
 /*
@@ -129,17 +142,17 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
  * kernels against each other and against the CPU oracle.
  */
 int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-                            const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+                            const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
                             const uint16_t* k_ms, const uint16_t* k_mc,
                             const uint8_t* k_index, const uint8_t* k_oval,
-                            const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+                            const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
                             const void* req_to_token, int64_t rt_stride,
                             const void* req_to_group, int64_t rg_stride, int table_i64,
                             const int32_t* b_seq_len,
                             float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                             int64_t al_stride_s,
                             int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                            int index_repr, int num_splits, float sm_scale, float logit_cap,
+                            int index_repr, int scale_bf16, int num_splits, float sm_scale, float logit_cap,
                             int packed_start_offset, int seg_group_base, void* stream);
 
 /*

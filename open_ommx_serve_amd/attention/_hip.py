@@ -18,6 +18,15 @@ _lib: Optional[C.CDLL] = None
 STORE_TABLE_FLOATS = 264
 ABI_VERSION = 3
 INDEX_BITMAP, INDEX_RELIDX7 = 0, 1
+SCALE_POW2_INT8, SCALE_POW2_BF16, SCALE_BF16 = 0, 1, 2
+
+
+def scale_mode(use_pow2: bool, kv_int8_scale: bool) -> int:
+    """C-ABI scale_mode of a recipe: the int8 exponent plane exists only for power-of-two
+    steps (reference pack.py:397 ``use_int8_scale = kv_int8_scale and use_pow2``)."""
+    if not use_pow2:
+        return SCALE_BF16
+    return SCALE_POW2_INT8 if kv_int8_scale else SCALE_POW2_BF16
 ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
@@ -29,7 +38,7 @@ _DECODE_ARGS = [
     _P, _L, _P, _L, _I,               # tables
     _P,                               # b_seq_len
     _P, _L, _L, _L,                   # attn_logits, strides
-    _I, _I, _I, _I, _I, _I, _I, _I,   # B Hq Hkv D ps kout index_repr S
+    _I, _I, _I, _I, _I, _I, _I, _I, _I,   # B Hq Hkv D ps kout index_repr scale_bf16 S
     _F, _F, _I, _I, _P,               # sm_scale cap off gbase stream
 ]
 
@@ -37,7 +46,7 @@ _SIGNATURES = {
     "ommx_abi_version": (_I, []),
     "ommx_last_error": (C.c_char_p, []),
     "ommx_store_default_table": (None, [_P]),
-    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P,
+    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P,
                              _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ommx_decode_splitkv": (_I, _DECODE_ARGS),
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),

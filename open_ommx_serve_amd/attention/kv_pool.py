@@ -65,10 +65,6 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"outlier_repr={outlier_repr!r}")
     if k > 0 and str(outlier_select).lower() not in ("signed", "abs"):
         bad.append(f"outlier_select={outlier_select!r}")
-    if not use_pow2:
-        bad.append("use_pow2=False")
-    if kv_int8_scale is False:
-        bad.append("kv_int8_scale=False")
     if group_tokens != 32 or group_channels != 32:
         bad.append(f"group_tokens={group_tokens}, group_channels={group_channels}")
     if scale_dtype != torch.bfloat16:
@@ -78,7 +74,7 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
     if bad:
         raise NotImplementedError(
             "the HIP KV store implements the serving recipe and its near variants only (i2f4, "
-            "signed or abs selection, bitmap or relidx7 index plane, use_pow2 with int8 exponents, "
+            "signed or abs selection, bitmap or relidx7 index plane, power-of-two or plain bf16 steps, "
             "dedicated or base-shared FP4 outliers, 32x32 groups, bf16 zero points, 0..8 outliers); "
             "unsupported: " + ", ".join(bad))
 
@@ -128,9 +124,9 @@ class MultiSeqKVPool:
         self.k = int(outliers_per_vector)
         self.outlier_select = str(outlier_select).lower()
         self.outlier_repr = str(outlier_repr).lower()
-        self.use_pow2 = True
+        self.use_pow2 = bool(use_pow2)
         self.kv_outlier_map = bool(kv_outlier_map)
-        self.kv_int8_scale = True
+        self.kv_int8_scale = bool(kv_int8_scale) and bool(use_pow2)      # pack.py:397
         self.scale_dtype = scale_dtype
         self.device = torch.device(device)
         _hip.require_gpu(self.device)
@@ -151,9 +147,10 @@ class MultiSeqKVPool:
         z = torch.zeros
         self.k_base = z(self.P_cap, self.ps, self.H, self.k_base_w, dtype=torch.uint8, device=dev)
         self.v_main = z(self.P_cap, self.ps, self.H, self.D // 4, dtype=torch.uint8, device=dev)
-        self.k_scale = z(self.G_cap, self.H, self.D, dtype=torch.int8, device=dev)
+        sdt = torch.int8 if self.kv_int8_scale else bf      # exponents, or the steps themselves
+        self.k_scale = z(self.G_cap, self.H, self.D, dtype=sdt, device=dev)
         self.k_zp = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-        self.v_scale = z(self.P_cap, self.ps, self.H, self.NGV, dtype=torch.int8, device=dev)
+        self.v_scale = z(self.P_cap, self.ps, self.H, self.NGV, dtype=sdt, device=dev)
         self.v_zp = z(self.P_cap, self.ps, self.H, self.NGV, dtype=bf, device=dev)
         self.k_oidx = None
         self.k_crank = None
@@ -375,6 +372,7 @@ class MultiSeqKVPool:
         flat_v = self.v_hist.view(self.num_seqs * self.S_ring, self.H, self.D)
         store_pack_into(flat_k, flat_v, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
+                        use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
                         page_size=self.ps, src_rows=idx[:n_s], dst_pages=idx[n_s:n_s + n_p],
                         dst_groups=idx[n_s + n_p:], err_flag=self.err_flag, num_tokens=n_s)
 
@@ -410,6 +408,7 @@ class MultiSeqKVPool:
         pp0 = r * self.P_per_seq + g0 * self.pages_per_group
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
+                        use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
                         page_size=self.ps,
                         dst_pages=self._req_to_token.view(-1)[pp0:pp0 + (g1 - g0) * self.pages_per_group],
                         dst_groups=self._req_to_group.view(-1)[gp0:gp0 + (g1 - g0)],
@@ -437,7 +436,7 @@ class MultiSeqKVPool:
             "group_tokens": self.gt, "group_channels": self.gc,
             "k_base_bits": self.k_base_bits, "oval_bits": self.oval_bits,
             "kv_outlier_map": bool(self.kv_outlier_map and self.k > 0),
-            "kv_int8_scale": True,
+            "kv_int8_scale": self.kv_int8_scale,
         }
 
     def request_planes(self, req: int) -> dict:
@@ -464,7 +463,7 @@ class MultiSeqKVPool:
             "outlier_repr": self.outlier_repr, "outlier_select": self.outlier_select,
             "group_tokens": self.gt, "group_channels": self.gc, "k_format": self.k_format,
             "k_base_bits": self.k_base_bits, "oval_bits": self.oval_bits,
-            "kv_outlier_map": bool(self.kv_outlier_map and self.k > 0), "kv_int8_scale": True,
+            "kv_outlier_map": bool(self.kv_outlier_map and self.k > 0), "kv_int8_scale": self.kv_int8_scale,
         }
 
     def _gather(self, kt, vt, *, seq=None, tail_idx=None, slots=None, b_tail=None, b_seq=None):

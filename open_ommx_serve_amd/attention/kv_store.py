@@ -71,7 +71,8 @@ class CanonicalKVStore:
         self.k = int(outliers_per_vector)
         self.outlier_select = str(outlier_select).lower()
         self.outlier_repr = str(outlier_repr).lower()
-        self.use_pow2, self.kv_int8_scale = True, True
+        self.use_pow2 = bool(use_pow2)
+        self.kv_int8_scale = bool(kv_int8_scale) and bool(use_pow2)      # pack.py:397
         self.kv_outlier_map = bool(kv_outlier_map)
         self.scale_dtype = scale_dtype
         self.device = torch.device(device)
@@ -89,9 +90,10 @@ class CanonicalKVStore:
         dev, bf, z = self.device, torch.bfloat16, torch.zeros
         self.k_base = z(self.P_cap, self.ps, self.H, self.k_base_w, dtype=torch.uint8, device=dev)
         self.v_main = z(self.P_cap, self.ps, self.H, self.D // 4, dtype=torch.uint8, device=dev)
-        self.k_scale = z(self.G_cap, self.H, self.D, dtype=torch.int8, device=dev)
+        sdt = torch.int8 if self.kv_int8_scale else bf      # exponents, or the steps themselves
+        self.k_scale = z(self.G_cap, self.H, self.D, dtype=sdt, device=dev)
         self.k_zp = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
-        self.v_scale = z(self.P_cap, self.ps, self.H, self.NGV, dtype=torch.int8, device=dev)
+        self.v_scale = z(self.P_cap, self.ps, self.H, self.NGV, dtype=sdt, device=dev)
         self.v_zp = z(self.P_cap, self.ps, self.H, self.NGV, dtype=bf, device=dev)
         self.k_oidx = None
         self.k_crank = None
@@ -274,6 +276,7 @@ class CanonicalKVStore:
         ppg = self.pages_per_group
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
+                        use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
                         page_size=self.ps, src_rows=src_rows,
                         dst_pages=self._req_to_token_full.view(-1)[g0 * ppg:g1 * ppg],
                         dst_groups=self._req_to_group_full.view(-1)[g0:g1],
@@ -287,7 +290,7 @@ class CanonicalKVStore:
                 "outlier_select": self.outlier_select, "group_tokens": self.gt,
                 "group_channels": self.gc, "k_format": self.k_format, "v_format": self.v_format,
                 "k_base_bits": self.k_base_bits, "oval_bits": self.oval_bits,
-                "kv_outlier_map": bool(self.kv_outlier_map and self.k > 0), "kv_int8_scale": True}
+                "kv_outlier_map": bool(self.kv_outlier_map and self.k > 0), "kv_int8_scale": self.kv_int8_scale}
 
     def decode_planes(self) -> dict:
         """Plane dict over the filled slots (kv_store.py:614-649)."""

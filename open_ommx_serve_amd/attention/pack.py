@@ -110,7 +110,8 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                     dst_groups: Optional[torch.Tensor] = None,
                     err_flag: Optional[torch.Tensor] = None,
                     num_tokens: Optional[int] = None,
-                    outlier_repr: str = "bitmap", outlier_select: str = "signed") -> None:
+                    outlier_repr: str = "bitmap", outlier_select: str = "signed",
+                    use_pow2: bool = True, kv_int8_scale: bool = True) -> None:
     """Pack ``num_tokens`` (default: all rows) tokens of ``K``/``V`` into ``planes`` in place.
 
     ``src_rows`` int32[T] picks the source row of each packed token (a ring gather);
@@ -138,12 +139,16 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
     sel = str(outlier_select).lower()
     if sel not in ("signed", "abs"):
         raise ValueError(f"outlier_select must be signed|abs; got {outlier_select!r}")
+    mode = _hip.scale_mode(bool(use_pow2), bool(kv_int8_scale))
+    want_dt = torch.int8 if mode == _hip.SCALE_POW2_INT8 else torch.bfloat16
+    if planes["k_scale"].dtype != want_dt or planes["v_scale"].dtype != want_dt:
+        raise ValueError(f"k_scale / v_scale planes must be {want_dt} for this recipe")
     lib = _hip.load()
     with torch.cuda.device(K.device):
         rc = lib.ommx_store_pack(
             K.data_ptr(), V.data_ptr(), 1 if K.dtype == torch.float32 else 0,
             K.stride(0), K.stride(1), V.stride(0), V.stride(1),
-            _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr, 1 if sel == "abs" else 0,
+            _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr, 1 if sel == "abs" else 0, mode,
             _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
             planes["k_base"].data_ptr(), planes["k_scale"].data_ptr(), planes["k_zp"].data_ptr(),
             _hip.ptr(planes.get("k_fp4_mapscale")), _hip.ptr(planes.get("k_fp4_mapcenter")),
@@ -169,11 +174,12 @@ def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int):
 def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim: int, *,
                  page_size: int = 16, outliers_per_vector: int = 6,
                  device: Any = "cuda", outlier_repr: str = "bitmap",
-                 kv_outlier_map: bool = True) -> Dict[str, Any]:
+                 kv_outlier_map: bool = True, int8_scale: bool = True) -> Dict[str, Any]:
     """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``."""
     P, G, H, D, ps, k = num_pages, num_group_slots, n_kv_heads, head_dim, page_size, outliers_per_vector
     dev = torch.device(device)
-    u8, i8, bf = torch.uint8, torch.int8, torch.bfloat16
+    u8, bf = torch.uint8, torch.bfloat16
+    i8 = torch.int8 if int8_scale else torch.bfloat16       # dtype of the two step planes (pack.py:586-590)
     out: Dict[str, Any] = {
         "k_base": torch.empty(P, ps, H, D // 4, dtype=u8, device=dev),
         "k_scale": torch.empty(G, H, D, dtype=i8, device=dev),
@@ -273,8 +279,6 @@ def ommx_pack_kv_canonical_block(
         unsupported.append(f"outlier_repr={repr_l!r}")
     if str(outlier_select).lower() not in ("signed", "abs"):
         unsupported.append(f"outlier_select={outlier_select!r}")
-    if not use_pow2 or not kv_int8_scale:
-        unsupported.append("non power-of-two / non int8-exponent scales")
     if k > 8:
         unsupported.append("more than 8 outliers per vector")
     if vfmt != "i2":
@@ -304,11 +308,13 @@ def ommx_pack_kv_canonical_block(
         Vd = Vd.contiguous()
     G, pages = T // gt, T // int(page_size)
     planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev,
-                          outlier_repr=repr_l, kv_outlier_map=bool(kv_outlier_map))
+                          outlier_repr=repr_l, kv_outlier_map=bool(kv_outlier_map),
+                          int8_scale=bool(use_pow2) and bool(kv_int8_scale))
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
         store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,
-                        outlier_repr=repr_l, outlier_select=outlier_select)
+                        outlier_repr=repr_l, outlier_select=outlier_select,
+                        use_pow2=bool(use_pow2), kv_int8_scale=bool(kv_int8_scale))
     raise_for_store_errors(int(err.item()))
 
     def _to(t):
@@ -326,7 +332,8 @@ def ommx_pack_kv_canonical_block(
         outliers_per_vector=k, outlier_repr=repr_l, outlier_select=str(outlier_select).lower(),
         group_tokens=gt, group_channels=gc, k_format=kfmt, v_format=vfmt,
         k_base_bits=2, oval_bits=4, use_pow2=bool(use_pow2),
-        kv_outlier_map=bool(kv_outlier_map and k > 0), kv_int8_scale=True)
+        kv_outlier_map=bool(kv_outlier_map and k > 0),
+        kv_int8_scale=bool(use_pow2) and bool(kv_int8_scale))
     return out
 
 

@@ -161,8 +161,11 @@ def ommx_paged_decode_attention_canonical(
         unsupported.append("combinadic outlier index plane")
     if k > 8:
         unsupported.append("more than 8 outliers per vector")
-    if k_scale.dtype != torch.int8 or v_scale.dtype != torch.int8:
-        unsupported.append("bf16 scale planes (int8 exponents only)")
+    # int8 exponent planes (kv_int8_scale) or the steps themselves as bf16 (paged_decode.py:1846-1855)
+    scale_bf16 = k_scale.dtype == torch.bfloat16
+    if k_scale.dtype != v_scale.dtype or k_scale.dtype not in (torch.int8, torch.bfloat16) \
+            or scale_bf16 == bool(kv_int8_scale):
+        unsupported.append(f"k_scale {k_scale.dtype} / v_scale {v_scale.dtype} with kv_int8_scale={bool(kv_int8_scale)}")
     if D != Dv or D not in (64, 128) or (Hq // Hkv) not in (1, 2, 4, 8):
         unsupported.append(f"head_dim {D}/{Dv} or GQA ratio {Hq // Hkv}")
     if 32 % ps != 0:
@@ -229,7 +232,8 @@ def ommx_paged_decode_attention_canonical(
             1 if req_to_token.dtype == torch.int64 else 0,
             b_seq_len.data_ptr(),
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            B, Hq, Hkv, D, ps, k, index_repr, S, float(sm_scale), float(logit_cap), off, gbase, stream)
+            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, S, float(sm_scale), float(logit_cap),
+            off, gbase, stream)
         _hip.check(rc, "ommx_decode_splitkv")
         rc = lib.ommx_decode_combine(
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),

@@ -21,13 +21,13 @@ extern "C" const char* ommx_last_error(void) { return ommx::g_error.c_str(); }
 
 extern "C" int ommx_decode_splitkv(
     const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-    const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
     const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
-    const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
     const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int num_splits,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
@@ -68,11 +68,11 @@ extern "C" int ommx_decode_splitkv(
         set_error("ommx_decode_splitkv: outlier planes missing");
         return -1;
     }
-    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval,
-                 v_main, v_scale, v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
+    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, static_cast<const int8_t*>(k_scale), k_zp, k_ms, k_mc,
+                 k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr};
+                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc = launch_decode_fast(a, D, R, st);
     if (rc == 1) rc = launch_decode_ref(a, D, R, st);
@@ -84,13 +84,13 @@ extern "C" int ommx_decode_splitkv(
 // Same operator through the plain fp32 kernel only (cross-check entry used by tests).
 extern "C" int ommx_decode_splitkv_ref(
     const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-    const uint8_t* k_base, const int8_t* k_scale, const uint16_t* k_zp,
+    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
     const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
-    const uint8_t* v_main, const int8_t* v_scale, const uint16_t* v_zp,
+    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
     const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int num_splits,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
@@ -99,11 +99,11 @@ extern "C" int ommx_decode_splitkv_ref(
         set_error("ommx_decode_splitkv_ref: bad arguments");
         return -1;
     }
-    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval,
-                 v_main, v_scale, v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
+    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, static_cast<const int8_t*>(k_scale), k_zp, k_ms, k_mc,
+                 k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr};
+                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0};
     if (launch_decode_ref(a, D, Hq / Hkv, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_splitkv_ref: unsupported shape");
         return -1;

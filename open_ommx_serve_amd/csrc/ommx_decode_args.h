@@ -18,6 +18,7 @@ struct DecodeArgs {
     float sm_scale, cap;
     int off, gbase;
     int idx_repr;                    // 0 flat bitmap, 1 relidx7
+    int scale_bf16;                  // k_scale / v_scale hold bf16 steps instead of int8 exponents
 };
 
 // 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)

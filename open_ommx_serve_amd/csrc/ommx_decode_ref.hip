@@ -47,7 +47,9 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
         const int64_t gslot = table_at(a.rg, b * a.rg_s + a.gbase + n0 / 32, a.i64);
         const int64_t gidx0 = (gslot * a.Hkv + kvh) * D;
         if (tid < D) {
-            s_sc[tid] = __uint_as_float(static_cast<uint32_t>(a.k_scale[gidx0 + tid] + 127) << 23);
+            s_sc[tid] = a.scale_bf16
+                ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.k_scale)[gidx0 + tid])
+                : __uint_as_float(static_cast<uint32_t>(a.k_scale[gidx0 + tid] + 127) << 23);
             s_zp[tid] = bf16_to_f32(a.k_zp[gidx0 + tid]);
         }
         if (tid < 32) {
@@ -158,7 +160,9 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
                     const int64_t rowh = s_row[t] * a.Hkv + kvh;
                     const uint32_t byte = a.v_main[rowh * (D / 4) + bc];
                     const int64_t vg = rowh * (D / 32) + (bc >> 3);
-                    const float vs = __uint_as_float(static_cast<uint32_t>(a.v_scale[vg] + 127) << 23);
+                    const float vs = a.scale_bf16
+                        ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.v_scale)[vg])
+                        : __uint_as_float(static_cast<uint32_t>(a.v_scale[vg] + 127) << 23);
                     const float vz = bf16_to_f32(a.v_zp[vg]);
                     float v[4];
 #pragma unroll

@@ -38,7 +38,10 @@ struct StoreArgs {
     int v_vec;              // V rows allow 16-byte loads
     int idx_repr;           // 0 flat bitmap (codec.py:330-372), 1 relidx7 (pack.py:128-164)
     int select_abs;         // 0 signed top + bottom tails (pack.py:436-445), 1 largest |w| (pack.py:446-448)
+    int scale_mode;         // 0 power of two, int8 exponent plane; 1 power of two, bf16 plane;
+                            // 2 bf16((max - min) / 3) as it comes, bf16 plane (pack.py:459-463, 586-590)
 };
+
 
 template <bool F32>
 __device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
@@ -67,6 +70,32 @@ __device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict_
 
 // x / 2^e is computed as x * 2^-e: 2^-e is exact for e in [-126,126], the product and the
 // quotient are then the same real number, so they round alike, denormal results included.
+// The quantisation step of one vector from raw = max(range, 1e-8) / 3 (pack.py:459-463).
+struct Step {
+    float scale;            // the step as the packer uses it (after its bf16 round trip)
+    float inv;              // exact inverse when inv_ok
+    bool inv_ok;
+    int e;                  // exponent (power-of-two modes)
+    uint16_t bits;          // the step as bf16
+    bool in_range;
+};
+__device__ __forceinline__ Step make_step(float raw, int mode, const float* tab) {
+    Step s;
+    if (mode == 2) {
+        s.bits = f32_to_bf16_rne(raw);
+        s.scale = bf16_to_f32(s.bits);
+        s.inv = 0.0f; s.inv_ok = false; s.e = 0; s.in_range = true;
+        return s;
+    }
+    s.e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
+    s.in_range = s.e >= -126 && s.e <= 127;
+    s.scale = exp2_int(s.e);
+    s.inv_ok = s.e >= -126 && s.e <= 126;
+    s.inv = exp2_int(s.inv_ok ? -s.e : 0);
+    s.bits = static_cast<uint16_t>((s.e + 127) << 7);
+    return s;
+}
+
 // INT2 code clamp(rint(x / 2^e), 0, 3) of a finite x.  v_cvt_pk_u8_f32 rounds to nearest even
 // and saturates below at 0; the upper clamp commutes with the rounding.
 __device__ __forceinline__ uint32_t int2_code(float x, float scale, float inv_scale, bool inv_ok) {
@@ -213,9 +242,9 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (omn > 1e8f) omn = 0.0f;
         if (omx < -1e8f) omx = 0.0f;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
-        const int e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
-        if (e < -126 || e > 127) err |= OMMX_ERR_EXP_RANGE;
-        const float scale = exp2_int(e);
+        const Step st = make_step(raw, a.scale_mode, tab);
+        if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
 
@@ -231,8 +260,8 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             ms = bf16_to_f32(ms_b);
         }
 
-        const bool inv_ok = e >= -126 && e <= 126;
-        const float inv_scale = exp2_int(inv_ok ? -e : 0);
+        const bool inv_ok = st.inv_ok;
+        const float inv_scale = st.inv;
         // the value whose FP4 code is stored: (w - centre) * map_scale, or (w - zp) / scale
         // (a division by a power of two: the same rounding as the exact inverse multiply)
         auto fp4_input = [&](float wv) {
@@ -275,7 +304,8 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (!mfin) err |= OMMX_ERR_NONFINITE_K;
 
         const int64_t gidx = (gs * a.H + h) * D + d;
-        a.k_scale[gidx] = static_cast<int8_t>(e);
+        if (a.scale_mode == 0) a.k_scale[gidx] = static_cast<int8_t>(st.e);
+        else reinterpret_cast<uint16_t*>(a.k_scale)[gidx] = st.bits;
         a.k_zp[gidx] = zp_b;
         if (kout > 0) {
             if (own_map) {
@@ -365,13 +395,13 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         }
         if (!fin) err |= OMMX_ERR_NONFINITE_V;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
-        const int e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
-        if (e < -126 || e > 127) err |= OMMX_ERR_EXP_RANGE;
-        const float scale = exp2_int(e);
+        const Step st = make_step(raw, a.scale_mode, tab);
+        if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
-        const bool inv_ok = e >= -126 && e <= 126;
-        const float inv_scale = exp2_int(inv_ok ? -e : 0);
+        const bool inv_ok = st.inv_ok;
+        const float inv_scale = st.inv;
         uint64_t vb8 = 0;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
@@ -379,7 +409,8 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         }
         const int64_t vidx = (prow * a.H + h) * NGV + j;
         reinterpret_cast<uint64_t*>(a.v_main)[vidx] = vb8;
-        a.v_scale[vidx] = static_cast<int8_t>(e);
+        if (a.scale_mode == 0) a.v_scale[vidx] = static_cast<int8_t>(st.e);
+        else reinterpret_cast<uint16_t*>(a.v_scale)[vidx] = st.bits;
         a.v_zp[vidx] = zp_b;
     }
     if (err && a.err) atomicOr(a.err, err);
@@ -410,12 +441,12 @@ extern "C" void ommx_store_default_table(float* t) {
 extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                                int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
                                const int32_t* src_rows, int T, int H, int D, int page_size,
-                               int k_outliers, int index_repr, int select_abs,
+                               int k_outliers, int index_repr, int select_abs, int scale_mode,
                                const int32_t* dst_pages,
                                const int32_t* dst_groups, const float* table,
-                               uint8_t* k_base, int8_t* k_scale, uint16_t* k_zp,
+                               uint8_t* k_base, void* k_scale, uint16_t* k_zp,
                                uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index,
-                               uint8_t* k_oval, uint8_t* v_main, int8_t* v_scale,
+                               uint8_t* k_oval, uint8_t* v_main, void* v_scale,
                                uint16_t* v_zp, int32_t* err_flag, void* stream) {
     using namespace ommx;
     if (T < 0 || T % 32 || page_size <= 0 || 32 % page_size || T % page_size) {
@@ -431,6 +462,7 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
         return -1;
     }
     if (index_repr != 0 && index_repr != 1) { set_error("ommx_store_pack: index_repr"); return -1; }
+    if (scale_mode < 0 || scale_mode > 2) { set_error("ommx_store_pack: scale_mode"); return -1; }
     if (in_dtype != 0 && in_dtype != 1) { set_error("ommx_store_pack: in_dtype"); return -1; }
     if (!K || !V || !table || !k_base || !k_scale || !k_zp || !v_main || !v_scale || !v_zp ||
         (k_outliers > 0 && (!k_index || !k_oval)) || (!k_ms != !k_mc)) {
@@ -439,10 +471,11 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
     }
     if (T == 0) return 0;
     StoreArgs a{K, V, k_ts, k_hs, v_ts, v_hs, src_rows, dst_pages, dst_groups, table,
-                k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval, v_main, v_scale, v_zp,
+                k_base, static_cast<int8_t*>(k_scale), k_zp, k_ms, k_mc, k_index, k_oval, v_main,
+                static_cast<int8_t*>(v_scale), v_zp,
                 err_flag, H, D, page_size, k_outliers,
                 (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0,
-                index_repr, select_abs ? 1 : 0};
+                index_repr, select_abs ? 1 : 0, scale_mode};
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -78,7 +78,7 @@ class DecodeCase:
                     k_obmp=p["k_obmp"],
                     k_fp4_mapscale=p["k_fp4_mapscale"], k_fp4_mapcenter=p["k_fp4_mapcenter"],
                     kv_outlier_map=self.outliers_per_vector > 0 and p["k_fp4_mapscale"] is not None,
-                    kv_int8_scale=True,
+                    kv_int8_scale=p["k_scale"].dtype == torch.int8,
                     max_seq_len=max(1, int(max(self.packed_lens))),
                     max_tail_len=int(self.k_tail.shape[1]))
 
@@ -113,7 +113,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       outliers_per_vector: int = 6, window: Optional[WindowSpec] = None,
                       device: Any = "cuda", keep_source: bool = False,
                       table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
-                      outlier_repr: str = "bitmap", kv_outlier_map: bool = True) -> DecodeCase:
+                      outlier_repr: str = "bitmap", kv_outlier_map: bool = True,
+                      use_pow2: bool = True, kv_int8_scale: bool = True) -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -134,7 +135,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     group_ids = g.permutation(tot_groups) if permute_tables else np.arange(tot_groups)
     planes = alloc_planes(tot_pages, tot_groups, H, D, page_size=ps,
                           outliers_per_vector=outliers_per_vector, device=dev,
-                          outlier_repr=outlier_repr, kv_outlier_map=kv_outlier_map)
+                          outlier_repr=outlier_repr, kv_outlier_map=kv_outlier_map,
+                          int8_scale=bool(use_pow2) and bool(kv_int8_scale))
     planes["outlier_repr"] = str(outlier_repr).lower()
     for t in planes.values():
         if torch.is_tensor(t):
@@ -166,7 +168,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
             store_pack_into(Kd, Vd, planes, outliers_per_vector=outliers_per_vector, page_size=ps,
                             dst_pages=torch.from_numpy(rt[b, :n_pages[b]].astype(np.int32)).to(dev),
                             dst_groups=torch.from_numpy(rg[b, :n_groups[b]].astype(np.int32)).to(dev),
-                            err_flag=err, outlier_repr=outlier_repr)
+                            err_flag=err, outlier_repr=outlier_repr, use_pow2=use_pow2,
+                            kv_int8_scale=kv_int8_scale)
         po += n_pages[b]
         go += n_groups[b]
         if keep_source:

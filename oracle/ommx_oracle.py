@@ -230,12 +230,15 @@ def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor,
 
 def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
             outliers_per_vector: int = 6, outlier_repr: str = "bitmap",
-            kv_outlier_map: bool = True, outlier_select: str = "signed") -> Dict[str, object]:
+            kv_outlier_map: bool = True, outlier_select: str = "signed",
+            use_pow2: bool = True, kv_int8_scale: bool = True) -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
     i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
     exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
     ``kv_outlier_map=False`` is the base-shared outlier variant (pack.py:502-506): the FP4 code
-    is taken of ``(w - zp) / scale`` and there are no map planes.
+    is taken of ``(w - zp) / scale`` and there are no map planes.  ``use_pow2=False`` keeps the
+    step ``bf16((max - min) / 3)`` as it comes; the step planes are then bf16, as they are with
+    ``kv_int8_scale=False`` (pack.py:397, 459-463, 586-590).
 
     ``K``/``V`` are ``[T, H, D]`` bf16 or fp32 with T a multiple of 32 and of
     ``page_size``.  Returns the ten planes, identity tables and the metadata keys.
@@ -258,9 +261,9 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         raise ValueError("outlier_select must be signed or abs")
     omask = select_outliers_signed(gw, k) if sel == "signed" else select_outliers_abs(gw, k)
     mn, mx = _masked_min_max(gw, ~omask)
+    int8_scale = bool(kv_int8_scale) and bool(use_pow2)                  # pack.py:397
     raw = (mx - mn).clamp_min(1e-8) / 3.0
-    e = pow2_exponent(raw)
-    scale = _bf16_rt(torch.pow(2.0, e))
+    scale = _bf16_rt(torch.pow(2.0, pow2_exponent(raw)) if use_pow2 else raw)
     zp = _bf16_rt(mn)
     code = torch.round((gw - zp) / scale).clamp(0, 3).to(torch.int64)
 
@@ -303,7 +306,8 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     codes_tok = code.reshape(H, D, T).permute(2, 0, 1)                    # [T,H,D]
     planes["k_base"] = pack_int2(codes_tok).reshape(pages, page_size, H, D // 4).contiguous()
     scale_ghd = scale.squeeze(-1).permute(2, 0, 1).contiguous()
-    planes["k_scale"] = pow2_exponent(scale_ghd).to(torch.int8)           # pack.py:586
+    planes["k_scale"] = pow2_exponent(scale_ghd).to(torch.int8) if int8_scale \
+        else scale_ghd.to(torch.bfloat16)                                 # pack.py:586-590
     planes["k_zp"] = zp.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
 
     # ---- V, vector = (token, head, 32 channels)                         pack.py:604-623
@@ -313,11 +317,12 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     vmn = gv.min(-1, keepdim=True)[0]
     vmx = gv.max(-1, keepdim=True)[0]
     vraw = (vmx - vmn).clamp_min(1e-8) / 3.0
-    vscale = _bf16_rt(torch.pow(2.0, pow2_exponent(vraw)))
+    vscale = _bf16_rt(torch.pow(2.0, pow2_exponent(vraw)) if use_pow2 else vraw)
     vzp = _bf16_rt(vmn)
     vcode = torch.round((gv - vzp) / vscale).clamp(0, 3).to(torch.int64)
     planes["v_main"] = pack_int2(vcode.reshape(T, H, D)).reshape(pages, page_size, H, D // 4).contiguous()
-    planes["v_scale"] = pow2_exponent(vscale.squeeze(-1)).to(torch.int8).reshape(pages, page_size, H, NGV).contiguous()
+    vs_flat = vscale.squeeze(-1).reshape(pages, page_size, H, NGV).contiguous()
+    planes["v_scale"] = pow2_exponent(vs_flat).to(torch.int8) if int8_scale else vs_flat.to(torch.bfloat16)
     planes["v_zp"] = vzp.squeeze(-1).to(torch.bfloat16).reshape(pages, page_size, H, NGV).contiguous()
 
     planes.update(
@@ -327,14 +332,22 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         head_dim=D, n_kv_heads=H, num_tokens=T, n_groups=G, page_size=int(page_size),
         outliers_per_vector=k, outlier_repr=repr_l, outlier_select=sel,
         group_tokens=gt, group_channels=gc, k_format="i2f4", v_format="i2",
-        k_base_bits=2, oval_bits=4, use_pow2=True, kv_outlier_map=bool(kv_outlier_map) and k > 0,
-        kv_int8_scale=True)
+        k_base_bits=2, oval_bits=4, use_pow2=bool(use_pow2),
+        kv_outlier_map=bool(kv_outlier_map) and k > 0, kv_int8_scale=int8_scale)
     return planes
 
 
 # ---------------------------------------------------------------------------------------
 # dequant                                                             pack.py:701-781
 # ---------------------------------------------------------------------------------------
+
+def _steps(plane: torch.Tensor) -> torch.Tensor:
+    """fp32 quantisation steps from a step plane: 2^e for an int8 exponent plane, the stored
+    values for a bf16 plane.  pack.py:719-726, 770-776."""
+    if plane.dtype == torch.int8:
+        return torch.exp2(plane.to(torch.float32))
+    return plane.to(torch.float32)
+
 
 def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
     """Planes (slot-linear, tables ignored) -> fp32 ``(K, V)`` each ``[T, H, D]``.
@@ -349,7 +362,7 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
     G = T // gt
     k = int(planes["outliers_per_vector"])
     code = unpack_int2(k_base.reshape(T, H, D4)).to(torch.float32)
-    scale = torch.exp2(planes["k_scale"].to(torch.float32))[:G]
+    scale = _steps(planes["k_scale"])[:G]
     zp = planes["k_zp"].to(torch.float32)[:G]
     Kd = code * scale.repeat_interleave(gt, 0) + zp.repeat_interleave(gt, 0)
     if k > 0:
@@ -366,7 +379,7 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
         Kd = Kg.permute(0, 3, 1, 2).reshape(T, H, D)
     vcode = unpack_int2(planes["v_main"].reshape(T, H, D4)).to(torch.float32)
     NGV = D // gc
-    vs = torch.exp2(planes["v_scale"].to(torch.float32)).reshape(T, H, NGV, 1)
+    vs = _steps(planes["v_scale"]).reshape(T, H, NGV, 1)
     vz = planes["v_zp"].to(torch.float32).reshape(T, H, NGV, 1)
     Vd = (vcode.reshape(T, H, NGV, gc) * vs + vz).reshape(T, H, D)
     return Kd, Vd
@@ -465,7 +478,7 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
     n_g = (L + gt - 1) // gt
     gs = req_to_group.to(torch.int64)[:n_g]
     code = unpack_int2(k_base.reshape(P * ps, H, D4)[rows]).to(torch.float32)
-    scale = torch.exp2(planes["k_scale"].to(torch.float32))[gslot]
+    scale = _steps(planes["k_scale"])[gslot]
     zp = planes["k_zp"].to(torch.float32)[gslot]
     Kd = code * scale + zp
     k = int(planes["outliers_per_vector"])
@@ -478,7 +491,7 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
             mc = planes["k_fp4_mapcenter"].to(torch.float32)[gs].unsqueeze(-1)
             dq = lvl / ms + mc
         else:
-            gsc = torch.exp2(planes["k_scale"].to(torch.float32))[gs].unsqueeze(-1)
+            gsc = _steps(planes["k_scale"])[gs].unsqueeze(-1)
             dq = lvl * gsc + planes["k_zp"].to(torch.float32)[gs].unsqueeze(-1)
         Kp = torch.zeros(Lp, H, D, dtype=torch.float32)
         Kp[:L] = Kd
@@ -487,7 +500,7 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
         Kd = Kg.permute(0, 3, 1, 2).reshape(Lp, H, D)[:L]
     vcode = unpack_int2(planes["v_main"].reshape(P * ps, H, D4)[rows]).to(torch.float32)
     NGV = D // gc
-    vs = torch.exp2(planes["v_scale"].reshape(P * ps, H, NGV)[rows].to(torch.float32)).unsqueeze(-1)
+    vs = _steps(planes["v_scale"].reshape(P * ps, H, NGV)[rows]).unsqueeze(-1)
     vz = planes["v_zp"].reshape(P * ps, H, NGV)[rows].to(torch.float32).unsqueeze(-1)
     Vd = (vcode.reshape(L, H, NGV, gc) * vs + vz).reshape(L, H, D)
     return Kd, Vd

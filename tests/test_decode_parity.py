@@ -192,6 +192,25 @@ def test_base_shared_outliers(hq, hkv, rep, ref_kernel):
         _check(_run(case, num_kv_splits=S, ref_kernel=ref_kernel), want, f"base-shared S{S}")
 
 
+@pytest.mark.parametrize("kw", [dict(use_pow2=False), dict(kv_int8_scale=False),
+                                dict(use_pow2=False, outlier_repr="relidx7", kv_outlier_map=False)])
+@pytest.mark.parametrize("hq,hkv,D", [(32, 8, 128), (4, 2, 64)])
+def test_bf16_step_planes(hq, hkv, D, kw):
+    """Planes whose k_scale / v_scale hold the steps as bf16 (use_pow2=False: not powers of two;
+    kv_int8_scale=False: powers of two stored as bf16) decode through the plain kernel."""
+    case = build_decode_case([1300, 90], q_heads=hq, kv_heads=hkv, head_dim=D, seed=51,
+                             permute_tables=True, sparse_frac=0.005, **kw)
+    assert case.planes["k_scale"].dtype == torch.bfloat16 and case.decode_kwargs()["kv_int8_scale"] is False
+    want = _oracle(case)
+    for S in (None, 3):
+        _check(_run(case, num_kv_splits=S), want, f"bf16 steps {kw} S{S}")
+    if "use_pow2" not in kw:         # same numbers as the int8-exponent twin of the same cache
+        twin = build_decode_case([1300, 90], q_heads=hq, kv_heads=hkv, head_dim=D, seed=51,
+                                 permute_tables=True, sparse_frac=0.005)
+        a, b = _run(case, ref_kernel=True), _run(twin, ref_kernel=True)
+        assert torch.equal(a[0], b[0])
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)

@@ -110,7 +110,7 @@ def test_pack_argument_errors_match_the_reference():
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "outlier_repr": "combinadic"})
     with pytest.raises(NotImplementedError):
-        P(K, K, **{**good, "use_pow2": False})
+        P(K, K, **{**good, "v_format": "bf16"})
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "group_tokens": 64})
     if not torch.cuda.is_available():
@@ -213,8 +213,8 @@ def test_store_classes_refuse_other_recipes_and_the_cpu():
         MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "outlier_repr": "combinadic"})
     check_serving_recipe(**{**good, "outlier_repr": "relidx7"}, kv_outlier_map=True, kv_int8_scale=True,
                          group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError, match="use_pow2"):
-        CanonicalKVStore(128, 8, 256, device="cpu", **{**good, "use_pow2": False})
+    with pytest.raises(NotImplementedError, match="v_format"):
+        CanonicalKVStore(128, 8, 256, device="cpu", v_format="bf16", **good)
     with pytest.raises(ValueError, match="k_format"):
         MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "k_format": "i3"})
     with pytest.raises(ValueError, match="multiple of 32"):

@@ -195,6 +195,43 @@ def test_base_shared_outliers_hand_built_vector():
     assert O.pack_kv(K, K.clone())["k_fp4_mapscale"] is not None
 
 
+def test_plain_bf16_steps_hand_built_vectors():
+    """use_pow2=False (pack.py:459-465): the step is bf16((max - min) / 3), not a power of two,
+    and the bf16 rounding of the step happens BEFORE the codes are formed.  No outliers, so the
+    whole vector is the base.
+    Channel 0: values in [0, 4.5] -> step 1.5 (exact in bf16); 1.4 / 1.5 = 0.93 -> 1,
+               2.3 / 1.5 = 1.53 -> 2, 0.75 / 1.5 = 0.5 -> ties to even -> 0, 2.25 / 1.5 = 1.5 -> 2.
+    Channel 1: values in [0, 1] -> 1/3 = 0.33333 rounds to bf16 0.333984375 (0x3EAB);
+               0.5 / 0.333984375 = 1.497 -> 1 (with the unrounded third it would be a tie -> 2).
+    Power-of-two twin of channel 0: 2^rint(log2(1.5)) = 2^1 -> codes rint(w / 2)."""
+    w0 = [0.0, 4.5, 1.4, 2.3, 0.75, 2.25] + [3.0] * 26
+    w1 = [0.0, 1.0, 0.5] + [0.25] * 29
+    K = torch.zeros(32, 1, 32)
+    K[:, 0, 0] = torch.tensor(w0)
+    K[:, 0, 1] = torch.tensor(w1)
+    pl = O.pack_kv(K, K.clone(), outliers_per_vector=0, use_pow2=False)
+    assert pl["k_scale"].dtype == torch.bfloat16 and pl["v_scale"].dtype == torch.bfloat16
+    assert pl["use_pow2"] is False and pl["kv_int8_scale"] is False
+    assert float(pl["k_scale"][0, 0, 0]) == 1.5 and float(pl["k_scale"][0, 0, 1]) == 0.333984375
+    codes = O.unpack_int2(pl["k_base"].reshape(32, 1, 8))
+    assert codes[:6, 0, 0].tolist() == [0, 3, 1, 2, 0, 2] and codes[6, 0, 0].item() == 2
+    assert codes[:4, 0, 1].tolist() == [0, 3, 1, 1]
+    Kd, _ = O.dequant_kv(pl)
+    assert Kd[:6, 0, 0].tolist() == [0.0, 4.5, 1.5, 3.0, 0.0, 3.0]
+    assert Kd[2, 0, 1].item() == 0.333984375
+    # the power-of-two recipe on the same data, stored either way, is another quantiser
+    p2 = O.pack_kv(K, K.clone(), outliers_per_vector=0)
+    assert int(p2["k_scale"][0, 0, 0]) == 1
+    assert O.unpack_int2(p2["k_base"].reshape(32, 1, 8))[:6, 0, 0].tolist() == [0, 2, 1, 1, 0, 1]
+    p3 = O.pack_kv(K, K.clone(), outliers_per_vector=0, kv_int8_scale=False)
+    assert p3["k_scale"].dtype == torch.bfloat16 and float(p3["k_scale"][0, 0, 0]) == 2.0
+    assert torch.equal(p3["k_base"], p2["k_base"]) and torch.equal(p3["v_main"], p2["v_main"])
+    assert torch.equal(O.dequant_kv(p3)[0], O.dequant_kv(p2)[0])
+    # V vector (token 1, channels 0..31): values 4.5, 1.0, zeros -> step 1.5, codes 3, 1 (0.67 -> 1), 0
+    vc = O.unpack_int2(pl["v_main"].reshape(32, 1, 8))[1, 0]
+    assert float(pl["v_scale"].reshape(32, 1, 1)[1, 0, 0]) == 1.5 and vc[:3].tolist() == [3, 1, 0]
+
+
 def test_nibble_stream_even_slot_low():
     v = torch.tensor([[1, 2, 3, 4, 5, 6]])
     assert O.nibbles_pack(v).tolist() == [[0x21, 0x43, 0x65]]

@@ -92,6 +92,44 @@ def test_store_abs_selection(k, T, H, D):
     assert_planes_equal(got, want, what=f"abs k{k}", zero_sign_free=True)
 
 
+@pytest.mark.parametrize("kw", [dict(use_pow2=False), dict(use_pow2=True, kv_int8_scale=False),
+                                dict(use_pow2=False, kv_outlier_map=False, outlier_repr="relidx7"),
+                                dict(use_pow2=False, outlier_select="abs", outliers_per_vector=3)])
+@pytest.mark.parametrize("T,H,D", [(256, 8, 128), (64, 2, 64)])
+def test_store_bf16_step_planes(kw, T, H, D):
+    """use_pow2=False (the step bf16((max - min) / 3) as it comes: true division for the codes)
+    and kv_int8_scale=False (power-of-two steps stored as bf16): bit-exact against the oracle.
+    The last two rows are the reference packer's default arguments but for the outlier count
+    / selection: relidx7, abs, no power-of-two rounding."""
+    K, V = synth_kv(T, H, D, 600 + T, outlier_channels=min(4, D // 8), sparse_frac=0.01)
+    args = dict(outliers_per_vector=6, outlier_repr="bitmap", outlier_select="signed")
+    args.update(kw)
+    want = O.pack_kv(K, V, **args)
+    got = _hip(K, V, **args)
+    assert got["k_scale"].dtype == torch.bfloat16 and got["v_scale"].dtype == torch.bfloat16
+    assert got["kv_int8_scale"] is False and got["use_pow2"] is bool(args.get("use_pow2", True))
+    names = ["k_base", "k_scale", "k_zp", "k_oval", "v_main", "v_scale", "v_zp",
+             "k_oidx" if args["outlier_repr"] == "relidx7" else "k_obmp"]
+    if args.get("kv_outlier_map", True):
+        names += ["k_fp4_mapscale", "k_fp4_mapcenter"]
+    for n in names:
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+
+
+def test_store_reference_default_arguments():
+    """ommx_pack_kv_canonical_block(K, V) with nothing else: 3 outliers by magnitude, relidx7,
+    plain bf16 steps, dedicated map (pack.py:293-309)."""
+    K, V = synth_kv(128, 4, 128, 77, sparse_frac=0.01)
+    got = ommx_pack_kv_canonical_block(K.cuda(), V.cuda())
+    want = O.pack_kv(K, V, outliers_per_vector=3, outlier_repr="relidx7", outlier_select="abs",
+                     use_pow2=False)
+    assert (got["outliers_per_vector"], got["outlier_repr"], got["outlier_select"], got["use_pow2"]) == \
+        (3, "relidx7", "abs", False)
+    for n in ("k_base", "k_scale", "k_zp", "k_oidx", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter",
+              "v_main", "v_scale", "v_zp"):
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
