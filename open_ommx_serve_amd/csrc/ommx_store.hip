@@ -119,19 +119,24 @@ __device__ __forceinline__ int med3_i32(int a, int b, int c) {
     return max(min(a, b), min(max(a, b), c));          // v_med3_i32
 }
 
-template <bool F32, bool FAST6>
+// IDXT: index plane known at compile time (0 bitmap, 1 relidx7) or read from the arguments (2)
+template <bool F32, bool FAST6, int IDXT>
 __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int D = a.D;
     uint8_t* s_codes = smem;                       // [32][D] one code per byte
-    uint8_t* s_oval = smem + 32 * D;               // [D][4] nibble bytes (3 used at k=6)
-    uint8_t* s_oidx = smem + 36 * D;               // [D][8] position stream bytes (relidx7 only)
+    uint8_t* s_oval = smem + 32 * D;               // [D][nval] nibble bytes, packed as in memory
+    uint8_t* s_oidx = smem + 36 * D;               // [D][nidx] position stream bytes (relidx7 only)
     const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int NGV = D >> 5;
     const int kout = a.kout, kt = (kout + 1) >> 1, kb = kout - kt;
     const int nval = (kout + 1) >> 1;              // nibble bytes per frame
     const int64_t gs = a.dst_groups ? a.dst_groups[g] : g;
     const float* __restrict__ tab = a.table;
+    // the tuned instantiation serves the serving recipe only: its variants are compile-time there
+    const int scale_mode = FAST6 ? 0 : a.scale_mode;
+    const bool select_abs = FAST6 ? false : a.select_abs != 0;
+    const int idx_repr = IDXT == 2 ? a.idx_repr : IDXT;
     int err = 0;
 
     // ------------------------------------------------------------------ K vector
@@ -149,7 +154,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         uint32_t top = 0, bot = 0;
         int key_hi[3] = {0, 0, 0}, key_lo[3] = {0, 0, 0};    // FAST6: sorted keys of the chosen lanes
         auto select_generic = [&]() {
-            if (a.select_abs) {
+            if (select_abs) {
                 // the kout largest magnitudes, ties to the lower index (stable descending sort
                 // of |w|, pack.py:446-448)
                 top = bot = 0;
@@ -242,7 +247,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (omn > 1e8f) omn = 0.0f;
         if (omx < -1e8f) omx = 0.0f;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
-        const Step st = make_step(raw, a.scale_mode, tab);
+        const Step st = make_step(raw, scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
         const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
@@ -250,7 +255,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
 
         // dedicated FP4 map over the outlier lanes (pack.py:486-498); without map planes the
         // outliers share the base scale and zero point instead (pack.py:502-506)
-        const bool own_map = a.k_ms != nullptr;
+        const bool own_map = FAST6 ? true : a.k_ms != nullptr;
         uint16_t mc_b = 0, ms_b = 0;
         float mc = 0.0f, ms = 0.0f;
         if (kout > 0 && own_map) {
@@ -304,7 +309,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         if (!mfin) err |= OMMX_ERR_NONFINITE_K;
 
         const int64_t gidx = (gs * a.H + h) * D + d;
-        if (a.scale_mode == 0) a.k_scale[gidx] = static_cast<int8_t>(st.e);
+        if (scale_mode == 0) a.k_scale[gidx] = static_cast<int8_t>(st.e);
         else reinterpret_cast<uint16_t*>(a.k_scale)[gidx] = st.bits;
         a.k_zp[gidx] = zp_b;
         if (kout > 0) {
@@ -312,7 +317,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                 a.k_ms[gidx] = ms_b;
                 a.k_mc[gidx] = mc_b;
             }
-            if (a.idx_repr == 0) {
+            if (idx_repr == 0) {
                 reinterpret_cast<uint32_t*>(a.k_obmp)[gidx] = om;  // byte p>>3, bit p&7
             } else {               // ascending positions, 7 bits each, least significant first
                 uint64_t stream = 0;
@@ -321,9 +326,11 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                     stream |= static_cast<uint64_t>(__ffs(m) - 1) << (7 * s);
                     m &= m - 1;
                 }
-                reinterpret_cast<uint64_t*>(s_oidx)[d] = stream;
+                const int nidx = (7 * kout + 7) / 8;
+                for (int b = 0; b < nidx; ++b)
+                    s_oidx[d * nidx + b] = static_cast<uint8_t>(stream >> (8 * b));
             }
-            reinterpret_cast<uint32_t*>(s_oval)[d] = nib;
+            for (int b = 0; b < nval; ++b) s_oval[d * nval + b] = static_cast<uint8_t>(nib >> (8 * b));
         }
     }
     __syncthreads();
@@ -331,13 +338,14 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
     // nibble plane: D frames of nval bytes, contiguous in memory
     if (kout > 0) {
         const int64_t obase = (gs * a.H + h) * (int64_t)D * nval;
-        for (int b = tid; b < D * nval; b += D)
-            a.k_oval[obase + b] = s_oval[(b / nval) * 4 + (b % nval)];
-        if (a.idx_repr != 0) {     // D frames of nidx bytes, contiguous in memory
+        // (D is a multiple of 32 and the plane is 8-byte aligned: whole dwords)
+        for (int w = tid; w < D * nval / 4; w += D)
+            reinterpret_cast<uint32_t*>(a.k_oval + obase)[w] = reinterpret_cast<const uint32_t*>(s_oval)[w];
+        if (idx_repr != 0) {     // D frames of nidx bytes, contiguous in memory
             const int nidx = (7 * kout + 7) / 8;
             const int64_t ibase = (gs * a.H + h) * (int64_t)D * nidx;
-            for (int b = tid; b < D * nidx; b += D)
-                a.k_obmp[ibase + b] = s_oidx[(b / nidx) * 8 + (b % nidx)];
+            for (int w = tid; w < D * nidx / 4; w += D)
+                reinterpret_cast<uint32_t*>(a.k_obmp + ibase)[w] = reinterpret_cast<const uint32_t*>(s_oidx)[w];
         }
     }
 
@@ -395,7 +403,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         }
         if (!fin) err |= OMMX_ERR_NONFINITE_V;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
-        const Step st = make_step(raw, a.scale_mode, tab);
+        const Step st = make_step(raw, scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
         const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
@@ -409,7 +417,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         }
         const int64_t vidx = (prow * a.H + h) * NGV + j;
         reinterpret_cast<uint64_t*>(a.v_main)[vidx] = vb8;
-        if (a.scale_mode == 0) a.v_scale[vidx] = static_cast<int8_t>(st.e);
+        if (scale_mode == 0) a.v_scale[vidx] = static_cast<int8_t>(st.e);
         else reinterpret_cast<uint16_t*>(a.v_scale)[vidx] = st.bits;
         a.v_zp[vidx] = zp_b;
     }
@@ -479,12 +487,15 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool tuned = k_outliers == 6 && !select_abs && scale_mode == 0 && k_ms;   // the serving recipe
     if (in_dtype == 1)
-        hipLaunchKernelGGL((store_pack_kernel<true, false>), grid, block, shm, st, a);
-    else if (k_outliers == 6 && !select_abs)
-        hipLaunchKernelGGL((store_pack_kernel<false, true>), grid, block, shm, st, a);
+        hipLaunchKernelGGL((store_pack_kernel<true, false, 2>), grid, block, shm, st, a);
+    else if (tuned && index_repr == 0)
+        hipLaunchKernelGGL((store_pack_kernel<false, true, 0>), grid, block, shm, st, a);
+    else if (tuned)
+        hipLaunchKernelGGL((store_pack_kernel<false, true, 1>), grid, block, shm, st, a);
     else
-        hipLaunchKernelGGL((store_pack_kernel<false, false>), grid, block, shm, st, a);
+        hipLaunchKernelGGL((store_pack_kernel<false, false, 2>), grid, block, shm, st, a);
     if (hipGetLastError() != hipSuccess) { set_error("ommx_store_pack: launch failed"); return -2; }
     return 0;
 }
