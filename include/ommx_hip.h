@@ -70,7 +70,7 @@ void ommx_store_default_table(float* host_table);
  *                 row r of head h starts at r*tok_stride + h*head_stride, D contiguous
  *   src_rows      NULL, or int32[T]: source row of packed token t (ring gather)
  *   dst_pages     NULL (identity), or int32[T/page_size]: physical page of logical page
- *   dst_groups    NULL (identity), or int32[T/32]: group slot of logical group
+ *   dst_groups    NULL (identity), or int32[T/group_tokens]: group slot of logical group
  *   table         float[OMMX_STORE_TABLE_FLOATS] on the device
  *   planes        as written by pack.py:576-623:
  *                 k_base,v_main u8[P,ps,H,D/4]; k_scale i8[G,H,D]; k_zp,k_ms,k_mc bf16[G,H,D];
@@ -88,15 +88,19 @@ void ommx_store_default_table(float* host_table);
  *                 (`outlier_select="signed"`, pack.py:436-445); 1: the k largest magnitudes
  *                 (`"abs"`, pack.py:446-448); ties go to the lower position either way
  *   err_flag      NULL or int32[1], OR-ed with OMMX_ERR_* (caller zeroes it)
- * k_outliers in 0..8; D a multiple of 32, at most 256; T a multiple of 32 and page_size;
- * 32 % page_size == 0.
+ *   group_tokens, group_channels   tokens per K vector / channels per V vector, each 16, 32,
+ *                 64 or 128 (pack.py:403-408); 32 and 32 is the serving recipe and runs the
+ *                 tuned kernel, everything else a general one
+ * k_outliers in 0..min(16, group_tokens); D a multiple of 32 and of group_channels, at most 256;
+ * T a multiple of group_tokens and page_size; G = T / group_tokens, the bitmap plane has
+ * group_tokens / 8 bytes per frame.
  */
 int ommx_store_pack(const void* K, const void* V, int in_dtype,
                     int64_t k_tok_stride, int64_t k_head_stride,
                     int64_t v_tok_stride, int64_t v_head_stride,
                     const int32_t* src_rows,
                     int T, int H, int D, int page_size, int k_outliers, int index_repr,
-                    int select_abs, int scale_mode,
+                    int select_abs, int scale_mode, int group_tokens, int group_channels,
                     const int32_t* dst_pages, const int32_t* dst_groups,
                     const float* table,
                     uint8_t* k_base, void* k_scale, uint16_t* k_zp,

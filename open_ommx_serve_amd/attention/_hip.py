@@ -46,7 +46,7 @@ _SIGNATURES = {
     "ommx_abi_version": (_I, []),
     "ommx_last_error": (C.c_char_p, []),
     "ommx_store_default_table": (None, [_P]),
-    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P,
+    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P] + [_I] * 10 + [_P, _P, _P,
                              _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ommx_decode_splitkv": (_I, _DECODE_ARGS),
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),

@@ -111,7 +111,8 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                     err_flag: Optional[torch.Tensor] = None,
                     num_tokens: Optional[int] = None,
                     outlier_repr: str = "bitmap", outlier_select: str = "signed",
-                    use_pow2: bool = True, kv_int8_scale: bool = True) -> None:
+                    use_pow2: bool = True, kv_int8_scale: bool = True,
+                    group_tokens: int = 32, group_channels: int = 32) -> None:
     """Pack ``num_tokens`` (default: all rows) tokens of ``K``/``V`` into ``planes`` in place.
 
     ``src_rows`` int32[T] picks the source row of each packed token (a ring gather);
@@ -130,12 +131,13 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
     H, D = int(K.shape[1]), int(K.shape[2])
     T = int(num_tokens) if num_tokens is not None else (
         int(src_rows.numel()) if src_rows is not None else int(K.shape[0]))
-    for t, n in ((src_rows, T), (dst_pages, T // max(1, page_size)), (dst_groups, T // 32)):
+    gt, gc = int(group_tokens), int(group_channels)
+    for t, n in ((src_rows, T), (dst_pages, T // max(1, page_size)), (dst_groups, T // max(1, gt))):
         if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()
                               or int(t.numel()) < n or t.device != K.device):
             raise ValueError("index tables must be contiguous int32 device tensors of the right length")
     k = int(outliers_per_vector)
-    index_repr, index_plane = _index_plane(planes, outlier_repr, k)
+    index_repr, index_plane = _index_plane(planes, outlier_repr, k, gt)
     sel = str(outlier_select).lower()
     if sel not in ("signed", "abs"):
         raise ValueError(f"outlier_select must be signed|abs; got {outlier_select!r}")
@@ -149,7 +151,7 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
             K.data_ptr(), V.data_ptr(), 1 if K.dtype == torch.float32 else 0,
             K.stride(0), K.stride(1), V.stride(0), V.stride(1),
             _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr, 1 if sel == "abs" else 0, mode,
-            _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
+            gt, gc, _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
             planes["k_base"].data_ptr(), planes["k_scale"].data_ptr(), planes["k_zp"].data_ptr(),
             _hip.ptr(planes.get("k_fp4_mapscale")), _hip.ptr(planes.get("k_fp4_mapcenter")),
             _hip.ptr(index_plane), _hip.ptr(planes.get("k_oval")),
@@ -158,11 +160,14 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
     _hip.check(rc, "ommx_store_pack")
 
 
-def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int):
+def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int, gt: int = 32):
     """(index_repr code of the C ABI, index plane tensor) for an ``outlier_repr`` name."""
     repr_l = str(outlier_repr).lower()
     if repr_l == "bitmap":
-        return _hip.INDEX_BITMAP, planes.get("k_obmp")
+        t = planes.get("k_obmp")
+        if k > 0 and (t is None or int(t.shape[-1]) != (gt + 7) // 8):
+            raise ValueError("bitmap needs a k_obmp plane of group_tokens/8 bytes per frame")
+        return _hip.INDEX_BITMAP, t
     if repr_l == "relidx7":
         t = planes.get("k_oidx")
         if k > 0 and (t is None or int(t.shape[-1]) != (7 * k + 7) // 8):
@@ -174,8 +179,10 @@ def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int):
 def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim: int, *,
                  page_size: int = 16, outliers_per_vector: int = 6,
                  device: Any = "cuda", outlier_repr: str = "bitmap",
-                 kv_outlier_map: bool = True, int8_scale: bool = True) -> Dict[str, Any]:
-    """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``."""
+                 kv_outlier_map: bool = True, int8_scale: bool = True,
+                 group_tokens: int = 32, group_channels: int = 32) -> Dict[str, Any]:
+    """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``;
+    ``num_group_slots`` counts K groups of ``group_tokens`` tokens."""
     P, G, H, D, ps, k = num_pages, num_group_slots, n_kv_heads, head_dim, page_size, outliers_per_vector
     dev = torch.device(device)
     u8, bf = torch.uint8, torch.bfloat16
@@ -185,8 +192,8 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
         "k_scale": torch.empty(G, H, D, dtype=i8, device=dev),
         "k_zp": torch.empty(G, H, D, dtype=bf, device=dev),
         "v_main": torch.empty(P, ps, H, D // 4, dtype=u8, device=dev),
-        "v_scale": torch.empty(P, ps, H, D // 32, dtype=i8, device=dev),
-        "v_zp": torch.empty(P, ps, H, D // 32, dtype=bf, device=dev),
+        "v_scale": torch.empty(P, ps, H, D // int(group_channels), dtype=i8, device=dev),
+        "v_zp": torch.empty(P, ps, H, D // int(group_channels), dtype=bf, device=dev),
         "k_oidx": None, "k_crank": None,
         "k_obmp": None, "k_oval": None, "k_fp4_mapscale": None, "k_fp4_mapcenter": None,
     }
@@ -194,7 +201,7 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
         if str(outlier_repr).lower() == "relidx7":      # pack.py:128-164: ceil(7k/8) bytes per frame
             out["k_oidx"] = torch.empty(G, H, D, (7 * k + 7) // 8, dtype=u8, device=dev)
         else:
-            out["k_obmp"] = torch.empty(G, H, D, 4, dtype=u8, device=dev)
+            out["k_obmp"] = torch.empty(G, H, D, (int(group_tokens) + 7) // 8, dtype=u8, device=dev)
         out["k_oval"] = torch.empty(G, H, D, (k + 1) // 2, dtype=u8, device=dev)
         if kv_outlier_map:       # base-shared outliers carry no map planes (pack.py:502-506)
             out["k_fp4_mapscale"] = torch.empty(G, H, D, dtype=bf, device=dev)
@@ -273,20 +280,18 @@ def ommx_pack_kv_canonical_block(
         raise ValueError(f"v_format must be i2|bf16; got {v_format!r}")
 
     unsupported = []
-    if gt != 32 or gc != 32:
-        unsupported.append("group_tokens/group_channels other than 32")
     if k > 0 and repr_l not in ("bitmap", "relidx7"):
         unsupported.append(f"outlier_repr={repr_l!r}")
     if str(outlier_select).lower() not in ("signed", "abs"):
         unsupported.append(f"outlier_select={outlier_select!r}")
-    if k > 8:
-        unsupported.append("more than 8 outliers per vector")
+    if k > 16:
+        unsupported.append("more than 16 outliers per vector")
     if vfmt != "i2":
         unsupported.append("v_format='bf16'")
     if scale_dtype != torch.bfloat16:
         unsupported.append(f"scale_dtype={scale_dtype}")
-    if 32 % int(page_size) != 0 or D > 256:
-        unsupported.append("page_size not dividing 32 / head_dim above 256")
+    if D > 256 or D % 32 != 0:
+        unsupported.append("head_dim above 256 or not a multiple of 32")
     if unsupported:
         raise NotImplementedError(
             "the HIP store kernel implements the serving recipe only; not: " + ", ".join(unsupported))
@@ -309,12 +314,14 @@ def ommx_pack_kv_canonical_block(
     G, pages = T // gt, T // int(page_size)
     planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev,
                           outlier_repr=repr_l, kv_outlier_map=bool(kv_outlier_map),
-                          int8_scale=bool(use_pow2) and bool(kv_int8_scale))
+                          int8_scale=bool(use_pow2) and bool(kv_int8_scale),
+                          group_tokens=gt, group_channels=gc)
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
         store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,
                         outlier_repr=repr_l, outlier_select=outlier_select,
-                        use_pow2=bool(use_pow2), kv_int8_scale=bool(kv_int8_scale))
+                        use_pow2=bool(use_pow2), kv_int8_scale=bool(kv_int8_scale),
+                        group_tokens=gt, group_channels=gc)
     raise_for_store_errors(int(err.item()))
 
     def _to(t):

@@ -19,6 +19,7 @@ LIB = os.path.join(HERE, "libommx_hip.so")
 ARCH = "gfx950"
 SOURCES = {
     "ommx_store.hip": ["-ffp-contract=off"],
+    "ommx_store_generic.hip": ["-ffp-contract=off"],
     "ommx_decode_ref.hip": [],
     "ommx_decode.hip": [],
     "ommx_combine.hip": [],

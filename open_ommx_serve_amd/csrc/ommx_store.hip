@@ -11,98 +11,9 @@
 // through LDS and written as 8-byte pieces of the token-major rows.
 #include <limits.h>
 
-#include "ommx_common.h"
+#include "ommx_store_common.h"
 
 namespace ommx {
-
-struct StoreArgs {
-    const void* K;
-    const void* V;
-    int64_t k_ts, k_hs, v_ts, v_hs;
-    const int32_t* src_rows;
-    const int32_t* dst_pages;
-    const int32_t* dst_groups;
-    const float* table;
-    uint8_t* k_base;
-    int8_t* k_scale;
-    uint16_t* k_zp;
-    uint16_t* k_ms;
-    uint16_t* k_mc;
-    uint8_t* k_obmp;        // index plane: bitmaps [G,H,D,4], or 7-bit streams [G,H,D,ceil(7k/8)]
-    uint8_t* k_oval;
-    uint8_t* v_main;
-    int8_t* v_scale;
-    uint16_t* v_zp;
-    int32_t* err;
-    int H, D, ps, kout;
-    int v_vec;              // V rows allow 16-byte loads
-    int idx_repr;           // 0 flat bitmap (codec.py:330-372), 1 relidx7 (pack.py:128-164)
-    int select_abs;         // 0 signed top + bottom tails (pack.py:436-445), 1 largest |w| (pack.py:446-448)
-    int scale_mode;         // 0 power of two, int8 exponent plane; 1 power of two, bf16 plane;
-                            // 2 bf16((max - min) / 3) as it comes, bf16 plane (pack.py:459-463, 586-590)
-};
-
-
-template <bool F32>
-__device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
-    if (F32) return static_cast<const float*>(base)[idx];
-    return bf16_to_f32(static_cast<const uint16_t*>(base)[idx]);
-}
-
-// rint(log2(x)) for x >= 1e-12 through the threshold table: the exponent of x's binade,
-// plus one when x has reached that binade's rounding point.
-__device__ __forceinline__ int pow2_round_exp(float x, const float* __restrict__ table) {
-    const uint32_t kb = (__float_as_uint(x) >> 23) & 0xFFu;
-    return static_cast<int>(kb) - 127 + (x >= table[kb] ? 1 : 0);
-}
-
-__device__ __forceinline__ float exp2_int(int e) {   // exact 2^e, e in [-126,127]
-    return __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-}
-
-__device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict__ fthr) {
-    const float a = fabsf(m);
-    uint32_t idx = 0;
-#pragma unroll
-    for (int j = 1; j <= 7; ++j) idx += (a >= fthr[j]) ? 1u : 0u;
-    return ((m < 0.0f) ? 8u : 0u) | idx;
-}
-
-// x / 2^e is computed as x * 2^-e: 2^-e is exact for e in [-126,126], the product and the
-// quotient are then the same real number, so they round alike, denormal results included.
-// The quantisation step of one vector from raw = max(range, 1e-8) / 3 (pack.py:459-463).
-struct Step {
-    float scale;            // the step as the packer uses it (after its bf16 round trip)
-    float inv;              // exact inverse when inv_ok
-    bool inv_ok;
-    int e;                  // exponent (power-of-two modes)
-    uint16_t bits;          // the step as bf16
-    bool in_range;
-};
-__device__ __forceinline__ Step make_step(float raw, int mode, const float* tab) {
-    Step s;
-    if (mode == 2) {
-        s.bits = f32_to_bf16_rne(raw);
-        s.scale = bf16_to_f32(s.bits);
-        s.inv = 0.0f; s.inv_ok = false; s.e = 0; s.in_range = true;
-        return s;
-    }
-    s.e = pow2_round_exp(fmaxf(raw, 1e-12f), tab);
-    s.in_range = s.e >= -126 && s.e <= 127;
-    s.scale = exp2_int(s.e);
-    s.inv_ok = s.e >= -126 && s.e <= 126;
-    s.inv = exp2_int(s.inv_ok ? -s.e : 0);
-    s.bits = static_cast<uint16_t>((s.e + 127) << 7);
-    return s;
-}
-
-// INT2 code clamp(rint(x / 2^e), 0, 3) of a finite x.  v_cvt_pk_u8_f32 rounds to nearest even
-// and saturates below at 0; the upper clamp commutes with the rounding.
-__device__ __forceinline__ uint32_t int2_code(float x, float scale, float inv_scale, bool inv_ok) {
-    if (inv_ok) return __builtin_amdgcn_cvt_pk_u8_f32(fminf(x * inv_scale, 3.0f), 0u, 0u);
-    const float c = fminf(fmaxf(rintf(__fdiv_rn(x, scale)), 0.0f), 3.0f);
-    return static_cast<uint32_t>(static_cast<int>(c));
-}
 
 // Order-preserving integer image of a bf16 value held as fp32 bits, low 16 bits cleared.
 // -0 must have been turned into +0 before (they tie in the reference's sorts).
@@ -450,23 +361,28 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                                int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
                                const int32_t* src_rows, int T, int H, int D, int page_size,
                                int k_outliers, int index_repr, int select_abs, int scale_mode,
-                               const int32_t* dst_pages,
+                               int group_tokens, int group_channels, const int32_t* dst_pages,
                                const int32_t* dst_groups, const float* table,
                                uint8_t* k_base, void* k_scale, uint16_t* k_zp,
                                uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index,
                                uint8_t* k_oval, uint8_t* v_main, void* v_scale,
                                uint16_t* v_zp, int32_t* err_flag, void* stream) {
     using namespace ommx;
-    if (T < 0 || T % 32 || page_size <= 0 || 32 % page_size || T % page_size) {
-        set_error("ommx_store_pack: T must be a multiple of 32 and page_size must divide 32");
+    const int gt = group_tokens, gc = group_channels;
+    if (!(gt == 16 || gt == 32 || gt == 64 || gt == 128) || !(gc == 16 || gc == 32 || gc == 64 || gc == 128)) {
+        set_error("ommx_store_pack: group_tokens and group_channels must be 16, 32, 64 or 128");
         return -1;
     }
-    if (D < 32 || D > 256 || D % 32 || H <= 0) {
-        set_error("ommx_store_pack: head_dim must be a multiple of 32 in [32,256]");
+    if (T < 0 || T % gt || page_size <= 0 || T % page_size) {
+        set_error("ommx_store_pack: T must be a multiple of group_tokens and of page_size");
         return -1;
     }
-    if (k_outliers < 0 || k_outliers > 8) {
-        set_error("ommx_store_pack: outliers_per_vector must be in [0,8]");
+    if (D < 32 || D > 256 || D % 32 || D % gc || H <= 0) {
+        set_error("ommx_store_pack: head_dim must be a multiple of 32 and of group_channels in [32,256]");
+        return -1;
+    }
+    if (k_outliers < 0 || k_outliers > 16 || k_outliers > gt) {
+        set_error("ommx_store_pack: outliers_per_vector must be in [0, min(16, group_tokens)]");
         return -1;
     }
     if (index_repr != 0 && index_repr != 1) { set_error("ommx_store_pack: index_repr"); return -1; }
@@ -483,10 +399,18 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                 static_cast<int8_t*>(v_scale), v_zp,
                 err_flag, H, D, page_size, k_outliers,
                 (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0,
-                index_repr, select_abs ? 1 : 0, scale_mode};
+                index_repr, select_abs ? 1 : 0, scale_mode, gt, gc};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (gt != 32 || gc != 32 || k_outliers > 8 || 32 % page_size) {     // everything but the 32x32 recipe
+        if (launch_store_generic(a, T, in_dtype, st) != 0) {
+            set_error("ommx_store_pack: no kernel for this recipe");
+            return -1;
+        }
+        if (hipGetLastError() != hipSuccess) { set_error("ommx_store_pack: launch failed"); return -2; }
+        return 0;
+    }
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const bool tuned = k_outliers == 6 && !select_abs && scale_mode == 0 && k_ms;   // the serving recipe
     if (in_dtype == 1)
         hipLaunchKernelGGL((store_pack_kernel<true, false, 2>), grid, block, shm, st, a);

@@ -231,7 +231,8 @@ def _masked_min_max(gw: torch.Tensor, keep: torch.Tensor) -> Tuple[torch.Tensor,
 def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
             outliers_per_vector: int = 6, outlier_repr: str = "bitmap",
             kv_outlier_map: bool = True, outlier_select: str = "signed",
-            use_pow2: bool = True, kv_int8_scale: bool = True) -> Dict[str, object]:
+            use_pow2: bool = True, kv_int8_scale: bool = True,
+            group_tokens: int = GROUP_TOKENS, group_channels: int = GROUP_CHANNELS) -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
     i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
     exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
@@ -244,7 +245,9 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     ``page_size``.  Returns the ten planes, identity tables and the metadata keys.
     """
     T, H, D = (int(s) for s in K.shape)
-    gt, gc, k = GROUP_TOKENS, GROUP_CHANNELS, int(outliers_per_vector)
+    gt, gc, k = int(group_tokens), int(group_channels), int(outliers_per_vector)
+    if gt not in (16, 32, 64, 128) or gc not in (16, 32, 64, 128):          # pack.py:405-408
+        raise ValueError("group sizes must be in {16, 32, 64, 128}")
     if tuple(V.shape) != (T, H, D):
         raise ValueError("K/V shape mismatch")
     if T % gt or T % page_size or D % gc:
@@ -358,7 +361,8 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
     k_base = planes["k_base"]
     P, ps, H, D4 = (int(s) for s in k_base.shape)
     T, D = P * ps, D4 * 4
-    gt, gc = GROUP_TOKENS, GROUP_CHANNELS
+    gt = int(planes.get("group_tokens", GROUP_TOKENS))
+    gc = int(planes.get("group_channels", GROUP_CHANNELS))
     G = T // gt
     k = int(planes["outliers_per_vector"])
     code = unpack_int2(k_base.reshape(T, H, D4)).to(torch.float32)
@@ -462,8 +466,9 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
     """Dequantised packed rows ``[seq_len, H, D]`` of ONE request read through its page and
     group-slot tables the way the decode kernel addresses them: packed token p lives in
     physical row ``req_to_token[(p+off)//ps]*ps + (p+off)%ps`` and uses group slot
-    ``req_to_group[p//32]``.  paged_decode.py:1668-1677."""
-    gt, gc = GROUP_TOKENS, GROUP_CHANNELS
+    ``req_to_group[p//gt]``.  paged_decode.py:1668-1677."""
+    gt = int(planes.get("group_tokens", GROUP_TOKENS))
+    gc = int(planes.get("group_channels", GROUP_CHANNELS))
     k_base = planes["k_base"]
     P, ps, H, D4 = (int(s) for s in k_base.shape)
     assert ps == page_size

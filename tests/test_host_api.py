@@ -112,7 +112,7 @@ def test_pack_argument_errors_match_the_reference():
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "v_format": "bf16"})
     with pytest.raises(NotImplementedError):
-        P(K, K, **{**good, "group_tokens": 64})
+        P(K, K, **{**good, "outliers_per_vector": 17, "outlier_repr": "relidx7"})
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             P(K, K, **good)

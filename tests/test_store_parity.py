@@ -130,6 +130,44 @@ def test_store_reference_default_arguments():
         assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
 
 
+GROUP_RECIPES = [
+    # the two other named recipes of the reference: "low-bit lever" and "paper-kv"
+    dict(group_tokens=64, group_channels=64, outliers_per_vector=6, outlier_repr="relidx7", kv_outlier_map=False),
+    dict(group_tokens=128, group_channels=128, outliers_per_vector=10, outlier_repr="relidx7"),
+    dict(group_tokens=128, group_channels=32, outliers_per_vector=8, outlier_repr="bitmap"),
+    dict(group_tokens=16, group_channels=16, outliers_per_vector=3, outlier_repr="bitmap"),
+    dict(group_tokens=64, group_channels=128, outliers_per_vector=16, outlier_repr="bitmap", outlier_select="abs"),
+    dict(group_tokens=16, group_channels=64, outliers_per_vector=2, outlier_repr="relidx7", use_pow2=False),
+    dict(group_tokens=32, group_channels=32, outliers_per_vector=12, outlier_repr="relidx7"),
+    dict(group_tokens=64, group_channels=64, outliers_per_vector=0),
+]
+
+
+@pytest.mark.parametrize("recipe", GROUP_RECIPES)
+@pytest.mark.parametrize("T,H,D,fp32", [(256, 8, 128, False), (128, 2, 256, True)])
+def test_store_other_group_sizes(recipe, T, H, D, fp32):
+    """K vectors of 16 / 64 / 128 tokens, V vectors of 16 / 64 / 128 channels, up to 16 outliers,
+    multi-word bitmaps and position streams: bit-exact against the oracle on every plane."""
+    K, V = synth_kv(T, H, D, 700 + T, outlier_channels=4, sparse_frac=0.01)
+    if fp32:
+        K, V = K.float() * 1.0009765625, V.float() * 0.99951171875       # leave the bf16 grid
+    args = dict(outlier_repr="bitmap", outlier_select="signed")
+    args.update(recipe)
+    want = O.pack_kv(K, V, **args)
+    got = _hip(K, V, **args)
+    gt, gc, k = args["group_tokens"], args["group_channels"], args["outliers_per_vector"]
+    assert (got["group_tokens"], got["group_channels"], got["n_groups"]) == (gt, gc, T // gt)
+    names = ["k_base", "k_scale", "k_zp", "v_main", "v_scale", "v_zp"]
+    if k > 0:
+        names += ["k_oval", "k_oidx" if args["outlier_repr"] == "relidx7" else "k_obmp"]
+        if args.get("kv_outlier_map", True):
+            names += ["k_fp4_mapscale", "k_fp4_mapcenter"]
+    for n in names:
+        assert got[n].shape == want[n].shape, n
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+    assert got["k_field_bytes"] == want["k_field_bytes"]
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
