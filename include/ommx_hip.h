@@ -123,7 +123,10 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
  * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64;
  * num_splits <= 256; planes 8-byte aligned.  scale_bf16 = 1: k_scale / v_scale hold the steps
- * themselves as bf16 instead of int8 exponents (plain kernel only).  head_dim 128 with r = 4 or 8 and 6 (or 0)
+ * themselves as bf16 instead of int8 exponents (plain kernel only).  group_tokens /
+ * group_channels: tokens per K group and channels per V vector, 16, 32, 64 or 128; the split
+ * length is rounded to group_tokens, and ommx_decode_combine must be given the same value.
+ * 32 and 32 with 6 (or 0) outliers is the matrix-core shape; k_outliers up to 16 otherwise.  head_dim 128 with r = 4 or 8 and 6 (or 0)
  * outliers runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
@@ -137,7 +140,8 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
                         float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,
                         int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                        int index_repr, int scale_bf16, int num_splits, float sm_scale, float logit_cap,
+                        int index_repr, int scale_bf16, int group_tokens, int group_channels,
+                        int num_splits, float sm_scale, float logit_cap,
                         int packed_start_offset, int seg_group_base, void* stream);
 
 /*
@@ -156,7 +160,8 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
                             float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                             int64_t al_stride_s,
                             int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
-                            int index_repr, int scale_bf16, int num_splits, float sm_scale, float logit_cap,
+                            int index_repr, int scale_bf16, int group_tokens, int group_channels,
+                        int num_splits, float sm_scale, float logit_cap,
                             int packed_start_offset, int seg_group_base, void* stream);
 
 /*
@@ -180,7 +185,7 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
                         const int32_t* b_tail_len, const int32_t* b_seq_len,
                         float* o, int64_t o_stride_b, int64_t o_stride_h,
                         float* lse, int64_t lse_stride_b,
-                        int B, int Hq, int Hkv, int D, int num_splits,
+                        int B, int Hq, int Hkv, int D, int num_splits, int group_tokens,
                         float sm_scale, float logit_cap, void* stream);
 
 /*

@@ -38,7 +38,8 @@ _DECODE_ARGS = [
     _P, _L, _P, _L, _I,               # tables
     _P,                               # b_seq_len
     _P, _L, _L, _L,                   # attn_logits, strides
-    _I, _I, _I, _I, _I, _I, _I, _I, _I,   # B Hq Hkv D ps kout index_repr scale_bf16 S
+    _I, _I, _I, _I, _I, _I, _I, _I,       # B Hq Hkv D ps kout index_repr scale_bf16
+    _I, _I, _I,                           # group_tokens group_channels S
     _F, _F, _I, _I, _P,               # sm_scale cap off gbase stream
 ]
 
@@ -51,7 +52,7 @@ _SIGNATURES = {
     "ommx_decode_splitkv": (_I, _DECODE_ARGS),
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),
     "ommx_decode_combine": (_I, [_P, _L, _L, _L, _P, _L, _L, _P, _P, _L, _L, _L, _L, _L, _L,
-                                 _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _F, _F, _P]),
+                                 _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _I, _F, _F, _P]),
     "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
                              _I, _I, _I, _I, _I, _P, _P]),
     "ommx_merge_states": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P]),

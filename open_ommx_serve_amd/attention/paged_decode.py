@@ -155,12 +155,10 @@ def ommx_paged_decode_attention_canonical(
         raise ValueError("kv_outlier_map=True requires k_fp4_mapscale + k_fp4_mapcenter planes.")
 
     unsupported = []
-    if group_tokens != 32 or group_channels != 32:
-        unsupported.append("group sizes other than 32")
     if k > 0 and combinadic_read:
         unsupported.append("combinadic outlier index plane")
-    if k > 8:
-        unsupported.append("more than 8 outliers per vector")
+    if k > 16:
+        unsupported.append("more than 16 outliers per vector")
     # int8 exponent planes (kv_int8_scale) or the steps themselves as bf16 (paged_decode.py:1846-1855)
     scale_bf16 = k_scale.dtype == torch.bfloat16
     if k_scale.dtype != v_scale.dtype or k_scale.dtype not in (torch.int8, torch.bfloat16) \
@@ -168,8 +166,8 @@ def ommx_paged_decode_attention_canonical(
         unsupported.append(f"k_scale {k_scale.dtype} / v_scale {v_scale.dtype} with kv_int8_scale={bool(kv_int8_scale)}")
     if D != Dv or D not in (64, 128) or (Hq // Hkv) not in (1, 2, 4, 8):
         unsupported.append(f"head_dim {D}/{Dv} or GQA ratio {Hq // Hkv}")
-    if 32 % ps != 0:
-        unsupported.append("page_size not dividing 32")
+    if group_tokens % ps != 0:
+        unsupported.append("page_size not dividing the K group")
     if q.dtype != torch.bfloat16 or q.stride(-1) != 1:
         unsupported.append("q that is not bf16 with unit inner stride")
     if unsupported:
@@ -178,8 +176,9 @@ def ommx_paged_decode_attention_canonical(
     # which index plane the kernels read (paged_decode.py:945-968 bitmap, :843-913 relidx7)
     k_index, index_repr = (k_obmp, _hip.INDEX_BITMAP) if bitmap_read else (k_oidx, _hip.INDEX_RELIDX7)
     if k > 0 and (k_index.dtype != torch.uint8 or tuple(k_index.shape[:3]) != tuple(k_scale.shape)
-                  or int(k_index.shape[-1]) != (4 if bitmap_read else (7 * k + 7) // 8)):
-        raise ValueError("outlier index plane must be u8 [group_slots, Hkv, D, 4 (bitmap) or ceil(7k/8) (relidx7)]")
+                  or int(k_index.shape[-1]) != ((group_tokens + 7) // 8 if bitmap_read else (7 * k + 7) // 8)):
+        raise ValueError("outlier index plane must be u8 [group_slots, Hkv, D, group_tokens/8 (bitmap) "
+                         "or ceil(7k/8) (relidx7)]")
     for name, t in (("k_scale", k_scale), ("k_zp", k_zp), ("k_oval", k_oval), ("k_index", k_index),
                     ("k_fp4_mapscale", k_fp4_mapscale), ("k_fp4_mapcenter", k_fp4_mapcenter)):
         if t is not None and not t.is_contiguous():
@@ -232,8 +231,8 @@ def ommx_paged_decode_attention_canonical(
             1 if req_to_token.dtype == torch.int64 else 0,
             b_seq_len.data_ptr(),
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, S, float(sm_scale), float(logit_cap),
-            off, gbase, stream)
+            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, group_tokens, group_channels, S,
+            float(sm_scale), float(logit_cap), off, gbase, stream)
         _hip.check(rc, "ommx_decode_splitkv")
         rc = lib.ommx_decode_combine(
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
@@ -243,7 +242,7 @@ def ommx_paged_decode_attention_canonical(
                 v_tail.stride(0), v_tail.stride(1), v_tail.stride(2)) if has_tail else (0,) * 6),
             b_tail_len.data_ptr() if has_tail else None, b_seq_len.data_ptr(),
             o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(0),
-            B, Hq, Hkv, D, S, float(sm_scale), float(logit_cap), stream)
+            B, Hq, Hkv, D, S, group_tokens, float(sm_scale), float(logit_cap), stream)
         _hip.check(rc, "ommx_decode_combine")
 
 

@@ -27,7 +27,8 @@ extern "C" int ommx_decode_splitkv(
     const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16, int num_splits,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
+    int group_tokens, int group_channels, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
@@ -40,17 +41,23 @@ extern "C" int ommx_decode_splitkv(
         set_error("ommx_decode_splitkv: supported shapes are head_dim 64|128 and 1|2|4|8 q heads per kv head");
         return -1;
     }
-    if (page_size <= 0 || 32 % page_size) {
-        set_error("ommx_decode_splitkv: page_size must divide the 32-token group");
+    if (!(group_tokens == 16 || group_tokens == 32 || group_tokens == 64 || group_tokens == 128) ||
+        !(group_channels == 16 || group_channels == 32 || group_channels == 64 || group_channels == 128) ||
+        D % group_channels) {
+        set_error("ommx_decode_splitkv: group_tokens / group_channels must be 16, 32, 64 or 128");
+        return -1;
+    }
+    if (page_size <= 0 || group_tokens % page_size) {
+        set_error("ommx_decode_splitkv: page_size must divide the K group");
         return -1;
     }
     if (packed_start_offset < 0 || packed_start_offset >= page_size || seg_group_base < 0) {
         set_error("ommx_decode_splitkv: packed_start_offset must be in [0,page_size), seg_group_base >= 0");
         return -1;
     }
-    if (k_outliers < 0 || k_outliers > 8 || num_splits < 1 || num_splits > 256 ||
+    if (k_outliers < 0 || k_outliers > 16 || k_outliers > group_tokens || num_splits < 1 || num_splits > 256 ||
         (index_repr != 0 && index_repr != 1)) {
-        set_error("ommx_decode_splitkv: k_outliers in [0,8], num_splits in [1,256], index_repr 0|1");
+        set_error("ommx_decode_splitkv: k_outliers in [0,min(16,group_tokens)], num_splits in [1,256], index_repr 0|1");
         return -1;
     }
     if ((reinterpret_cast<uintptr_t>(k_base) | reinterpret_cast<uintptr_t>(v_main) |
@@ -72,7 +79,8 @@ extern "C" int ommx_decode_splitkv(
                  k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0};
+                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
+                 group_tokens, group_channels};
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc = launch_decode_fast(a, D, R, st);
     if (rc == 1) rc = launch_decode_ref(a, D, R, st);
@@ -90,12 +98,16 @@ extern "C" int ommx_decode_splitkv_ref(
     const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16, int num_splits,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
+    int group_tokens, int group_channels, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
-    if (B <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 || 32 % page_size || num_splits < 1 ||
-        k_outliers < 0 || k_outliers > 8 || (index_repr != 0 && index_repr != 1)) {
+    if (B <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 || num_splits < 1 || k_outliers < 0 ||
+        k_outliers > 16 || (index_repr != 0 && index_repr != 1) ||
+        !(group_tokens == 16 || group_tokens == 32 || group_tokens == 64 || group_tokens == 128) ||
+        !(group_channels == 16 || group_channels == 32 || group_channels == 64 || group_channels == 128) ||
+        group_tokens % page_size || k_outliers > group_tokens || D % group_channels) {
         set_error("ommx_decode_splitkv_ref: bad arguments");
         return -1;
     }
@@ -103,7 +115,8 @@ extern "C" int ommx_decode_splitkv_ref(
                  k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0};
+                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
+                 group_tokens, group_channels};
     if (launch_decode_ref(a, D, Hq / Hkv, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_splitkv_ref: unsupported shape");
         return -1;
@@ -120,10 +133,11 @@ extern "C" int ommx_decode_combine(
     int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
     const int32_t* b_tail_len, const int32_t* b_seq_len,
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
-    int B, int Hq, int Hkv, int D, int num_splits, float sm_scale, float logit_cap,
+    int B, int Hq, int Hkv, int D, int num_splits, int group_tokens, float sm_scale, float logit_cap,
     void* stream) {
     using namespace ommx;
-    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || num_splits < 1 || !(D == 64 || D == 128)) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || num_splits < 1 || !(D == 64 || D == 128) ||
+        group_tokens < 16 || group_tokens > 128 || (group_tokens & (group_tokens - 1))) {
         set_error("ommx_decode_combine: bad shape");
         return -1;
     }
@@ -145,7 +159,7 @@ extern "C" int ommx_decode_combine(
                   k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h,
                   vt_stride_b, vt_stride_t, vt_stride_h, b_tail_len, b_seq_len,
                   o, o_stride_b, o_stride_h, lse, lse_stride_b, B, Hq, Hkv, num_splits,
-                  sm_scale, logit_cap};
+                  sm_scale, logit_cap, group_tokens};
     if (launch_combine(a, D, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_combine: unsupported head_dim");
         return -1;

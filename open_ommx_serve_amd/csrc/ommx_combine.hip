@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
         }
     }
     const uint32_t q_raw = a.q ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + d] : 0u;
-    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
+    const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:2407
     float my_lse = -INFINITY;
     if (tid < MAXS) {
         const bool valid = tid < a.S && min(per * tid + per, L) > per * tid;

@@ -19,6 +19,7 @@ struct DecodeArgs {
     int off, gbase;
     int idx_repr;                    // 0 flat bitmap, 1 relidx7
     int scale_bf16;                  // k_scale / v_scale hold bf16 steps instead of int8 exponents
+    int gt, gc;                      // tokens per K group, channels per V vector (16, 32, 64 or 128)
 };
 
 // 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)
@@ -45,6 +46,7 @@ struct CombineArgs {
     float* lse; int64_t lse_b;
     int B, Hq, Hkv, S;
     float sm_scale, cap;
+    int gt;                          // tokens per K group: the splits are rounded to it
 };
 
 int launch_decode_ref(const DecodeArgs& a, int D, int R, hipStream_t st);

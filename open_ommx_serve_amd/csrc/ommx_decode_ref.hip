@@ -19,15 +19,15 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
     extern __shared__ float sm[];
     float* s_K = sm;                      // [32][KS]   (reused for the final reduction)
     float* s_q = s_K + (32 * KS > TS * R * D ? 32 * KS : TS * R * D);   // [R][D]
-    float* s_sc = s_q + R * D;            // [D]
-    float* s_zp = s_sc + D;               // [D]
+    float* s_sc = s_q + R * D;            // [2][D]  (two K groups per tile when groups are 16 tokens)
+    float* s_zp = s_sc + 2 * D;           // [2][D]
     float* s_p = s_zp + D;                // [R][32]
     float* s_al = s_p + R * 32;           // [R]
     int64_t* s_row = reinterpret_cast<int64_t*>(s_al + 8);   // [32]
 
     const int b = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z, tid = threadIdx.x;
     const int L = a.seq[b];
-    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
+    const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:1429-1430
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
 
@@ -43,20 +43,31 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
         for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;       // live in threads tid < 32*R
 
+    const int gt = a.gt;                          // tokens per K group: 16, 32, 64 or 128
+    const int ngv = D / a.gc;                     // V vectors per token
     for (int n0 = n_begin; n0 < n_end; n0 += 32) {
-        const int64_t gslot = table_at(a.rg, b * a.rg_s + a.gbase + n0 / 32, a.i64);
-        const int64_t gidx0 = (gslot * a.Hkv + kvh) * D;
-        if (tid < D) {
-            s_sc[tid] = a.scale_bf16
-                ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.k_scale)[gidx0 + tid])
-                : __uint_as_float(static_cast<uint32_t>(a.k_scale[gidx0 + tid] + 127) << 23);
-            s_zp[tid] = bf16_to_f32(a.k_zp[gidx0 + tid]);
+        // A tile is 32 tokens.  With 16-token groups it spans two K groups (sub-group u = t / 16),
+        // otherwise it lies inside one (n0 is a multiple of 32 and so is the group size).
+        const int nsub = gt == 16 ? 2 : 1;
+        const int g_first = n0 / gt;
+        int64_t gidx_u[2] = {0, 0};
+        for (int u = 0; u < nsub; ++u) {
+            const int gi = min(g_first + u, (n_end - 1) / gt);
+            const int64_t gslot = table_at(a.rg, b * a.rg_s + a.gbase + gi, a.i64);
+            gidx_u[u] = (gslot * a.Hkv + kvh) * D;
+        }
+        for (int i = tid; i < nsub * D; i += 256) {
+            const int u = i / D, d = i % D;
+            s_sc[i] = a.scale_bf16
+                ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.k_scale)[gidx_u[u] + d])
+                : __uint_as_float(static_cast<uint32_t>(a.k_scale[gidx_u[u] + d] + 127) << 23);
+            s_zp[i] = bf16_to_f32(a.k_zp[gidx_u[u] + d]);
         }
         if (tid < 32) {
             const int n = n0 + tid;
             int64_t prow = 0;
             if (n < n_end) {
-                const int64_t p = (int64_t)n + (int64_t)a.gbase * 32 + a.off;
+                const int64_t p = (int64_t)n + (int64_t)a.gbase * gt + a.off;
                 prow = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
             }
             s_row[tid] = prow;
@@ -65,6 +76,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
 
         {   // base dequant: thread (token t, slice c of D/8 channels)
             const int t = tid >> 3, c = tid & 7;
+            const int u = gt == 16 ? (t >> 4) : 0;
             constexpr int NB = D / 32;            // bytes per thread
             const uint8_t* src = a.k_base + (s_row[t] * a.Hkv + kvh) * (D / 4) + c * NB;
             uint32_t bits = 0;
@@ -74,37 +86,48 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
             for (int j = 0; j < 4 * NB; ++j) {
                 const int d = c * 4 * NB + j;
                 const float code = static_cast<float>((bits >> (2 * j)) & 3u);
-                s_K[t * KS + d] = code * s_sc[d] + s_zp[d];
+                s_K[t * KS + d] = code * s_sc[u * D + d] + s_zp[u * D + d];
             }
         }
         __syncthreads();
 
         if (a.kout > 0 && tid < D) {   // outlier splice: thread = channel
             const int nval = (a.kout + 1) >> 1;
-            uint32_t bm = 0;
-            if (a.idx_repr == 0) {
-                bm = reinterpret_cast<const uint32_t*>(a.k_obmp)[gidx0 + tid];
-            } else {               // 7-bit position stream -> the same occupancy mask
-                const int nidx = relidx7_bytes(a.kout);
-                const uint8_t* ip = a.k_obmp + (gidx0 + tid) * nidx;
-                uint64_t stream = 0;
-                for (int j = 0; j < nidx; ++j) stream |= static_cast<uint64_t>(ip[j]) << (8 * j);
-                for (int s = 0; s < a.kout; ++s) bm |= 1u << ((stream >> (7 * s)) & 31u);
-            }
-            const uint8_t* ov = a.k_oval + (gidx0 + tid) * nval;
-            uint32_t nib = 0;
-            for (int j = 0; j < nval; ++j) nib |= static_cast<uint32_t>(ov[j]) << (8 * j);
-            // dedicated map: level / map_scale + centre; else the base scale and zero point
+            const int nidx = a.idx_repr == 0 ? (gt + 7) / 8 : relidx7_bytes(a.kout);
             const bool own_map = a.k_ms != nullptr;
-            const float ms = own_map ? bf16_to_f32(a.k_ms[gidx0 + tid]) : 0.0f;
-            const float mc = own_map ? bf16_to_f32(a.k_mc[gidx0 + tid]) : 0.0f;
-            while (bm) {
-                const int pos = __ffs(bm) - 1;
-                bm &= bm - 1;
-                float lvl = fp4_level(nib & 7u);
-                if (nib & 8u) lvl = -lvl;
-                nib >>= 4;
-                s_K[pos * KS + tid] = own_map ? __fdiv_rn(lvl, ms) + mc : lvl * s_sc[tid] + s_zp[tid];
+            for (int u = 0; u < nsub; ++u) {
+                if ((g_first + u) * gt >= n_end) break;
+                const int64_t fr = gidx_u[u] + tid;
+                // tile-local index of group position 0 (negative when the group began before the tile)
+                const int base = (g_first + u) * gt - n0;
+                const uint8_t* ip = a.k_obmp + fr * nidx;
+                const uint8_t* ov = a.k_oval + fr * nval;
+                // dedicated map: level / map_scale + centre; else the base scale and zero point
+                const float ms = own_map ? bf16_to_f32(a.k_ms[fr]) : 0.0f;
+                const float mc = own_map ? bf16_to_f32(a.k_mc[fr]) : 0.0f;
+                int byte_i = 0, bit0 = 0;           // bitmap walk state: next byte, bit offset of the current one
+                uint32_t cur = 0;
+                for (int sl = 0; sl < a.kout; ++sl) {
+                    int pos;
+                    if (a.idx_repr == 0) {          // next set bit, ascending
+                        while (cur == 0 && byte_i < nidx) { cur = ip[byte_i]; bit0 = 8 * byte_i; ++byte_i; }
+                        if (cur == 0) break;
+                        pos = bit0 + __ffs(cur) - 1;
+                        cur &= cur - 1;
+                    } else {                        // 7-bit field sl of the stream
+                        const int bit = 7 * sl;
+                        const uint32_t two = static_cast<uint32_t>(ip[bit >> 3]) |
+                            ((bit >> 3) + 1 < nidx ? static_cast<uint32_t>(ip[(bit >> 3) + 1]) << 8 : 0u);
+                        pos = (two >> (bit & 7)) & 127;
+                    }
+                    const uint32_t code = (ov[sl >> 1] >> (4 * (sl & 1))) & 0xFu;
+                    const int tl = base + pos;
+                    if (tl < 0 || tl >= 32) continue;
+                    float lvl = fp4_level(code & 7u);
+                    if (code & 8u) lvl = -lvl;
+                    s_K[tl * KS + tid] = own_map ? __fdiv_rn(lvl, ms) + mc
+                                                 : lvl * s_sc[u * D + tid] + s_zp[u * D + tid];
+                }
             }
         }
         __syncthreads();
@@ -159,7 +182,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
                 if (n0 + t < n_end) {
                     const int64_t rowh = s_row[t] * a.Hkv + kvh;
                     const uint32_t byte = a.v_main[rowh * (D / 4) + bc];
-                    const int64_t vg = rowh * (D / 32) + (bc >> 3);
+                    const int64_t vg = rowh * ngv + (bc * 4) / a.gc;
                     const float vs = a.scale_bf16
                         ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.v_scale)[vg])
                         : __uint_as_float(static_cast<uint32_t>(a.v_scale[vg] + 127) << 23);
@@ -207,7 +230,7 @@ static void launch_ref(const DecodeArgs& a, hipStream_t st) {
     constexpr int KS = D + 4;
     constexpr int TS = 256 / (D / 4);
     constexpr int big = 32 * KS > TS * R * D ? 32 * KS : TS * R * D;
-    const size_t shm = sizeof(float) * (big + R * D + 2 * D + R * 32 + 8) + sizeof(int64_t) * 32;
+    const size_t shm = sizeof(float) * (big + R * D + 4 * D + R * 32 + 8) + sizeof(int64_t) * 32;
     hipLaunchKernelGGL((decode_splitkv_ref_kernel<D, R>), dim3(a.B, a.Hkv, a.S), dim3(256), shm, st, a);
 }
 

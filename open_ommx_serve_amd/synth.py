@@ -114,21 +114,24 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       device: Any = "cuda", keep_source: bool = False,
                       table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
                       outlier_repr: str = "bitmap", kv_outlier_map: bool = True,
-                      use_pow2: bool = True, kv_int8_scale: bool = True) -> DecodeCase:
+                      use_pow2: bool = True, kv_int8_scale: bool = True,
+                      group_tokens: int = 32, group_channels: int = 32) -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
     ``permute_tables`` the ids of all requests are shuffled together, so consecutive
     logical pages of a request land anywhere in the pool.
     """
-    win = window or WindowSpec(page_size=page_size)
+    gt, gc = int(group_tokens), int(group_channels)
+    win = window or WindowSpec(page_size=page_size, group_tokens=gt)
+    assert win.group_tokens == gt
     dev = torch.device(device)
     B, H, D, ps = len(seq_lens), kv_heads, head_dim, page_size
     packed = [win.packed_len(int(n)) for n in seq_lens]
     n_pages = [p // ps for p in packed]
-    n_groups = [p // 32 for p in packed]
-    # at least one whole group (32 // ps pages), so the planes keep the 32-token geometry
-    tot_pages, tot_groups = max(32 // ps, sum(n_pages)), max(1, sum(n_groups))
+    n_groups = [p // gt for p in packed]
+    # at least one whole group (gt // ps pages), so the planes keep the group geometry
+    tot_pages, tot_groups = max(max(1, gt // ps), sum(n_pages)), max(1, sum(n_groups))
     g = _rng(seed, 424242)
     page_ids = g.permutation(tot_pages) if permute_tables else np.arange(tot_pages)
     # group slots follow their pages only through the tables, so shuffle them separately
@@ -136,8 +139,10 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     planes = alloc_planes(tot_pages, tot_groups, H, D, page_size=ps,
                           outliers_per_vector=outliers_per_vector, device=dev,
                           outlier_repr=outlier_repr, kv_outlier_map=kv_outlier_map,
-                          int8_scale=bool(use_pow2) and bool(kv_int8_scale))
+                          int8_scale=bool(use_pow2) and bool(kv_int8_scale),
+                          group_tokens=gt, group_channels=gc)
     planes["outlier_repr"] = str(outlier_repr).lower()
+    planes["group_tokens"], planes["group_channels"] = gt, gc
     for t in planes.values():
         if torch.is_tensor(t):
             t.zero_()
@@ -169,7 +174,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                             dst_pages=torch.from_numpy(rt[b, :n_pages[b]].astype(np.int32)).to(dev),
                             dst_groups=torch.from_numpy(rg[b, :n_groups[b]].astype(np.int32)).to(dev),
                             err_flag=err, outlier_repr=outlier_repr, use_pow2=use_pow2,
-                            kv_int8_scale=kv_int8_scale)
+                            kv_int8_scale=kv_int8_scale, group_tokens=gt, group_channels=gc)
         po += n_pages[b]
         go += n_groups[b]
         if keep_source:

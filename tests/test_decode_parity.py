@@ -211,6 +211,32 @@ def test_bf16_step_planes(hq, hkv, D, kw):
         assert torch.equal(a[0], b[0])
 
 
+@pytest.mark.parametrize("recipe", [
+    dict(group_tokens=64, group_channels=64, outliers_per_vector=6, outlier_repr="relidx7", kv_outlier_map=False),
+    dict(group_tokens=128, group_channels=128, outliers_per_vector=10, outlier_repr="relidx7"),
+    dict(group_tokens=128, group_channels=32, outliers_per_vector=8, outlier_repr="bitmap"),
+    dict(group_tokens=16, group_channels=16, outliers_per_vector=3, outlier_repr="bitmap"),
+    dict(group_tokens=16, group_channels=64, outliers_per_vector=2, outlier_repr="relidx7", use_pow2=False),
+    dict(group_tokens=64, group_channels=128, outliers_per_vector=16, outlier_repr="relidx7"),
+    dict(group_tokens=32, group_channels=32, outliers_per_vector=12, outlier_repr="relidx7"),
+    dict(group_tokens=64, group_channels=64, outliers_per_vector=0),
+])
+@pytest.mark.parametrize("hq,hkv,D", [(32, 8, 128), (4, 2, 64)])
+def test_other_group_sizes(hq, hkv, D, recipe):
+    """K groups of 16 / 64 / 128 tokens, V vectors of 16 / 64 / 128 channels, up to 16 outliers:
+    the window boundary, the split rounding and both tables follow the group size.  The first
+    two rows are the reference's "low-bit lever" and "paper-kv" recipes."""
+    if D % recipe["group_channels"]:
+        recipe = {**recipe, "group_channels": D}          # a V vector cannot be wider than the head
+    case = build_decode_case([1500, 300, 40], q_heads=hq, kv_heads=hkv, head_dim=D, seed=61,
+                             permute_tables=True, sparse_frac=0.005, **recipe)
+    gt = recipe["group_tokens"]
+    assert all(n % gt == 0 for n in case.packed_lens) and case.packed_lens[0] > 0
+    want = _oracle(case)
+    for S in (None, 1, 7):
+        _check(_run(case, num_kv_splits=S), want, f"{recipe} S{S}")
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)
