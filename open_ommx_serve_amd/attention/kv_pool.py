@@ -65,17 +65,15 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
         bad.append(f"outlier_repr={outlier_repr!r}")
     if k > 0 and str(outlier_select).lower() not in ("signed", "abs"):
         bad.append(f"outlier_select={outlier_select!r}")
-    if group_tokens != 32 or group_channels != 32:
-        bad.append(f"group_tokens={group_tokens}, group_channels={group_channels}")
     if scale_dtype != torch.bfloat16:
         bad.append(f"scale_dtype={scale_dtype}")
-    if not 0 <= k <= 8:
+    if not 0 <= k <= min(16, int(group_tokens)):
         bad.append(f"outliers_per_vector={k}")
     if bad:
         raise NotImplementedError(
             "the HIP KV store implements the serving recipe and its near variants only (i2f4, "
             "signed or abs selection, bitmap or relidx7 index plane, power-of-two or plain bf16 steps, "
-            "dedicated or base-shared FP4 outliers, 32x32 groups, bf16 zero points, 0..8 outliers); "
+            "dedicated or base-shared FP4 outliers, bf16 zero points, 0..16 outliers); "
             "unsupported: " + ", ".join(bad))
 
 
@@ -373,6 +371,7 @@ class MultiSeqKVPool:
         store_pack_into(flat_k, flat_v, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
+                        group_tokens=self.gt, group_channels=self.gc,
                         page_size=self.ps, src_rows=idx[:n_s], dst_pages=idx[n_s:n_s + n_p],
                         dst_groups=idx[n_s + n_p:], err_flag=self.err_flag, num_tokens=n_s)
 
@@ -409,6 +408,7 @@ class MultiSeqKVPool:
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
+                        group_tokens=self.gt, group_channels=self.gc,
                         page_size=self.ps,
                         dst_pages=self._req_to_token.view(-1)[pp0:pp0 + (g1 - g0) * self.pages_per_group],
                         dst_groups=self._req_to_group.view(-1)[gp0:gp0 + (g1 - g0)],

@@ -277,6 +277,7 @@ class CanonicalKVStore:
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
+                        group_tokens=self.gt, group_channels=self.gc,
                         page_size=self.ps, src_rows=src_rows,
                         dst_pages=self._req_to_token_full.view(-1)[g0 * ppg:g1 * ppg],
                         dst_groups=self._req_to_group_full.view(-1)[g0:g1],

@@ -275,6 +275,97 @@ def test_pool_with_the_relidx7_index_plane(ring):
                                 "store", "relidx7")
 
 
+@pytest.mark.parametrize("ring", [False, True])
+@pytest.mark.parametrize("recipe", [
+    # the reference's "low-bit lever" and "paper-kv" recipes (pack.py:334-362, recipes.py:183-200)
+    dict(group_tokens=64, group_channels=64, outliers_per_vector=6, outlier_repr="relidx7", kv_outlier_map=False),
+    dict(group_tokens=128, group_channels=128, outliers_per_vector=10, outlier_repr="relidx7"),
+    dict(group_tokens=16, group_channels=32, outliers_per_vector=2, outlier_repr="bitmap", use_pow2=False),
+])
+def test_pool_other_group_sizes(recipe, ring):
+    """Pool and single-sequence store with K groups of 16 / 64 / 128 tokens: the window, the ring
+    span, the page / group-slot tables and the incremental packs follow the group size.  Planes
+    against the oracle packer after every pack, decode against the oracle at the end."""
+    H, D, B, q_heads = 4, 128, 2, 16
+    gt, gc, k = recipe["group_tokens"], recipe["group_channels"], recipe["outliers_per_vector"]
+    win = WindowSpec(group_tokens=gt)
+    prefill, steps = [300, 45], 2 * gt + 5
+    sm_scale = 1.0 / math.sqrt(D)
+    okw = dict(outliers_per_vector=k, outlier_repr=recipe["outlier_repr"], group_tokens=gt, group_channels=gc,
+               kv_outlier_map=recipe.get("kv_outlier_map", True), use_pow2=recipe.get("use_pow2", True))
+    kw = {**RECIPE, **recipe}
+    kw.pop("group_tokens")
+    Ks, Vs = zip(*[synth_kv(n + steps, H, D, seed=800 + i, sparse_frac=0.005) for i, n in enumerate(prefill)])
+    pool = MultiSeqKVPool(D, H, num_seqs=2, max_seq_len=1024, window=win, device=DEV, kv_ring=ring, **kw)
+
+    def planes_equal(got, n_tok, r, what):
+        edge = win.boundary(n_tok)
+        assert got["num_tokens"] == max(0, edge - win.sink_tokens), what
+        if edge <= win.sink_tokens:
+            return
+        want = O.pack_kv(Ks[r][win.sink_tokens:edge], Vs[r][win.sink_tokens:edge], page_size=win.page_size, **okw)
+        for name in ("k_base", "k_scale", "k_zp", "k_obmp", "k_oidx", "k_oval", "k_fp4_mapscale",
+                     "k_fp4_mapcenter", "v_main", "v_scale", "v_zp"):
+            if want[name] is None:
+                assert got[name] is None, (what, name)
+                continue
+            a, b = got[name].cpu(), want[name]
+            assert a.shape == b.shape and a.dtype == b.dtype, (what, name, a.shape, b.shape)
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{what}: plane {name} differs"
+
+    for r in range(B):
+        pool.append_block(r, Ks[r][:prefill[r]].to(DEV), Vs[r][:prefill[r]].to(DEV))
+        planes_equal(pool.request_planes(r), prefill[r], r, f"prefill req {r}")
+    q_all = synth_q(steps, B * q_heads, D, seed=7).reshape(steps, B, q_heads, D)
+    n_packs = 0
+    for s in range(steps):
+        newK = torch.stack([Ks[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        newV = torch.stack([Vs[i][prefill[i] + s] for i in range(B)]).to(DEV)
+        packed = pool.append_decode_batched(range(B), newK, newV)
+        cur = [prefill[i] + s + 1 for i in range(B)]
+        if packed:
+            n_packs += 1
+            for r in range(B):
+                planes_equal(pool.request_planes(r), cur[r], r, f"step {s} req {r}")
+        if s % 16 == 15 or s == steps - 1:
+            bundle = pool.decode_inputs_batched(range(B))
+            assert bundle["b_seq_len"].tolist() == [win.packed_len(n) for n in cur]
+            pl = bundle["planes"]
+            q = q_all[s].to(DEV)
+            o = torch.full((B, q_heads, D), float("nan"), dtype=torch.float32, device=DEV)
+            lse = torch.full((B, q_heads), float("nan"), dtype=torch.float32, device=DEV)
+            ommx_paged_decode_attention_canonical(
+                q, pl["k_base"], pl["k_scale"], pl["k_zp"], pl.get("k_oidx"), pl["k_oval"],
+                pl["v_main"], pl["v_scale"], pl["v_zp"], bundle["k_tail"], bundle["v_tail"],
+                bundle["b_tail_len"], o, lse, bundle["req_to_token"], bundle["req_to_group"], bundle["b_seq_len"],
+                sm_scale=sm_scale, page_size=pl["page_size"], k_outliers_per_vector=k,
+                bitmap_read=pl["outlier_repr"] == "bitmap", k_obmp=pl["k_obmp"],
+                k_fp4_mapscale=pl["k_fp4_mapscale"], k_fp4_mapcenter=pl["k_fp4_mapcenter"],
+                kv_outlier_map=pl["kv_outlier_map"], kv_int8_scale=pl["kv_int8_scale"],
+                max_seq_len=bundle["max_seq_len"], max_tail_len=bundle["max_tail_len"],
+                packed_start_offset=bundle["packed_start_offset"])
+            torch.cuda.synchronize()
+            outs, lses = [], []
+            for b in range(B):
+                n = cur[b]
+                edge = win.boundary(n)
+                ti = win.tail_indices(n)
+                Kd = torch.stack([Ks[b][i].float() for i in ti])
+                Vd = torch.stack([Vs[b][i].float() for i in ti])
+                if edge > win.sink_tokens:
+                    Kp, Vp = O.dequant_kv(O.pack_kv(Ks[b][win.sink_tokens:edge], Vs[b][win.sink_tokens:edge],
+                                                    page_size=win.page_size, **okw))
+                    Kd, Vd = torch.cat([Kp, Kd]), torch.cat([Vp, Vd])
+                ob, lb = O.attend(q[b].cpu(), Kd, Vd, sm_scale, dtype=torch.float64)
+                outs.append(ob); lses.append(lb)
+            _check_out((o.cpu(), lse.cpu()), (torch.stack(outs), torch.stack(lses)), f"{recipe} ring={ring} step {s}")
+    assert n_packs >= 2
+    pool.check_errors()
+    store = CanonicalKVStore(D, H, max_seq_len=1024, window=win, device=DEV, kv_ring=ring, **kw)
+    store.append_block(Ks[0][:prefill[0]].to(DEV), Vs[0][:prefill[0]].to(DEV))
+    planes_equal(store.decode_planes(), prefill[0], 0, "store")
+
+
 def test_pool_device_counter_path_equals_the_host_path():
     """append_decode_device / decode_inputs_device (device sequence counter) against
     append_decode_batched / decode_inputs_batched on a second pool fed the same rows."""
