@@ -109,7 +109,7 @@ def _make_runner(case, splits=None):
             case.req_to_group.data_ptr(), case.req_to_group.stride(0),
             1 if case.req_to_token.dtype == torch.int64 else 0, case.b_seq_len.data_ptr(),
             ws.data_ptr(), ws.stride(0), ws.stride(1), ws.stride(2),
-            B, Hq, case.kv_heads, D, case.page_size, case.outliers_per_vector, _hip.INDEX_BITMAP, 0, 32, 32, S,
+            B, Hq, case.kv_heads, D, case.page_size, case.outliers_per_vector, _hip.INDEX_BITMAP, 0, 32, 32, 0, S,
             float(case.sm_scale), 0.0, 0, 0, torch.cuda.current_stream(dev).cuda_stream)
         _hip.check(rc, "ommx_decode_splitkv")
 

@@ -91,6 +91,9 @@ void ommx_store_default_table(float* host_table);
  *   group_tokens, group_channels   tokens per K vector / channels per V vector, each 16, 32,
  *                 64 or 128 (pack.py:403-408); 32 and 32 is the serving recipe and runs the
  *                 tuned kernel, everything else a general one
+ *   v_bf16        1: V is not quantised; v_main is bf16 [P,ps,H,D] (the rows rounded to bf16),
+ *                 v_scale is filled with ones and v_zp with zeros (`v_format="bf16"`,
+ *                 pack.py:596-602)
  * k_outliers in 0..min(16, group_tokens); D a multiple of 32 and of group_channels, at most 256;
  * T a multiple of group_tokens and page_size; G = T / group_tokens, the bitmap plane has
  * group_tokens / 8 bytes per frame.
@@ -101,7 +104,7 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
                     const int32_t* src_rows,
                     int T, int H, int D, int page_size, int k_outliers, int index_repr,
                     int select_abs, int scale_mode, int group_tokens, int group_channels,
-                    const int32_t* dst_pages, const int32_t* dst_groups,
+                    int v_bf16, const int32_t* dst_pages, const int32_t* dst_groups,
                     const float* table,
                     uint8_t* k_base, void* k_scale, uint16_t* k_zp,
                     uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index, uint8_t* k_oval,
@@ -126,7 +129,8 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  * themselves as bf16 instead of int8 exponents (plain kernel only).  group_tokens /
  * group_channels: tokens per K group and channels per V vector, 16, 32, 64 or 128; the split
  * length is rounded to group_tokens, and ommx_decode_combine must be given the same value.
- * 32 and 32 with 6 (or 0) outliers is the matrix-core shape; k_outliers up to 16 otherwise.  head_dim 128 with r = 4 or 8 and 6 (or 0)
+ * 32 and 32 with 6 (or 0) outliers is the matrix-core shape; k_outliers up to 16 otherwise.
+ * v_bf16 = 1: v_main is bf16 [P,ps,H,D] and v_scale / v_zp are ignored (plain kernel only).  head_dim 128 with r = 4 or 8 and 6 (or 0)
  * outliers runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
@@ -141,7 +145,7 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
                         int64_t al_stride_s,
                         int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
                         int index_repr, int scale_bf16, int group_tokens, int group_channels,
-                        int num_splits, float sm_scale, float logit_cap,
+                        int v_bf16, int num_splits, float sm_scale, float logit_cap,
                         int packed_start_offset, int seg_group_base, void* stream);
 
 /*
@@ -161,7 +165,7 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
                             int64_t al_stride_s,
                             int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
                             int index_repr, int scale_bf16, int group_tokens, int group_channels,
-                        int num_splits, float sm_scale, float logit_cap,
+                        int v_bf16, int num_splits, float sm_scale, float logit_cap,
                             int packed_start_offset, int seg_group_base, void* stream);
 
 /*

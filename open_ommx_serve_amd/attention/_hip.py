@@ -39,7 +39,7 @@ _DECODE_ARGS = [
     _P,                               # b_seq_len
     _P, _L, _L, _L,                   # attn_logits, strides
     _I, _I, _I, _I, _I, _I, _I, _I,       # B Hq Hkv D ps kout index_repr scale_bf16
-    _I, _I, _I,                           # group_tokens group_channels S
+    _I, _I, _I, _I,                       # group_tokens group_channels v_bf16 S
     _F, _F, _I, _I, _P,               # sm_scale cap off gbase stream
 ]
 
@@ -47,7 +47,7 @@ _SIGNATURES = {
     "ommx_abi_version": (_I, []),
     "ommx_last_error": (C.c_char_p, []),
     "ommx_store_default_table": (None, [_P]),
-    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P] + [_I] * 10 + [_P, _P, _P,
+    "ommx_store_pack": (_I, [_P, _P, _I, _L, _L, _L, _L, _P] + [_I] * 11 + [_P, _P, _P,
                              _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ommx_decode_splitkv": (_I, _DECODE_ARGS),
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),

@@ -57,8 +57,6 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
     if group_tokens not in (16, 32, 64, 128):
         raise ValueError(f"group_tokens must be in {{16,32,64,128}}; got {group_tokens}")
     bad = []
-    if str(k_format).lower() != "i2f4":
-        bad.append(f"k_format={k_format!r}")
     if str(v_format).lower() != "i2":
         bad.append(f"v_format={v_format!r}")
     if k > 0 and str(outlier_repr).lower() not in ("bitmap", "relidx7"):
@@ -118,7 +116,7 @@ class MultiSeqKVPool:
                              scale_dtype=scale_dtype, outliers_per_vector=outliers_per_vector)
         self.D, self.H = int(head_dim), int(n_kv_heads)
         self.num_seqs, self.max_seq_len = int(num_seqs), int(max_seq_len)
-        self.k_format = "i2f4"
+        self.k_format = str(k_format).lower()          # "i2f4" and "itf4" name the same planes
         self.k = int(outliers_per_vector)
         self.outlier_select = str(outlier_select).lower()
         self.outlier_repr = str(outlier_repr).lower()

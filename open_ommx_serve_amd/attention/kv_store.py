@@ -67,7 +67,7 @@ class CanonicalKVStore:
                              scale_dtype=scale_dtype, outliers_per_vector=outliers_per_vector,
                              v_format=v_format)
         self.D, self.H, self.max_seq_len = int(head_dim), int(n_kv_heads), int(max_seq_len)
-        self.k_format, self.v_format = "i2f4", "i2"
+        self.k_format, self.v_format = str(k_format).lower(), "i2"     # "itf4" is the same format
         self.k = int(outliers_per_vector)
         self.outlier_select = str(outlier_select).lower()
         self.outlier_repr = str(outlier_repr).lower()

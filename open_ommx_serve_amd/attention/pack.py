@@ -112,7 +112,7 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                     num_tokens: Optional[int] = None,
                     outlier_repr: str = "bitmap", outlier_select: str = "signed",
                     use_pow2: bool = True, kv_int8_scale: bool = True,
-                    group_tokens: int = 32, group_channels: int = 32) -> None:
+                    group_tokens: int = 32, group_channels: int = 32, v_format: str = "i2") -> None:
     """Pack ``num_tokens`` (default: all rows) tokens of ``K``/``V`` into ``planes`` in place.
 
     ``src_rows`` int32[T] picks the source row of each packed token (a ring gather);
@@ -141,6 +141,9 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
     sel = str(outlier_select).lower()
     if sel not in ("signed", "abs"):
         raise ValueError(f"outlier_select must be signed|abs; got {outlier_select!r}")
+    v_bf16 = str(v_format).lower() == "bf16"
+    if (planes["v_main"].dtype == torch.bfloat16) != v_bf16:
+        raise ValueError("v_main must be bf16 [pages, page_size, H, D] for v_format='bf16', else uint8 codes")
     mode = _hip.scale_mode(bool(use_pow2), bool(kv_int8_scale))
     want_dt = torch.int8 if mode == _hip.SCALE_POW2_INT8 else torch.bfloat16
     if planes["k_scale"].dtype != want_dt or planes["v_scale"].dtype != want_dt:
@@ -151,7 +154,7 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
             K.data_ptr(), V.data_ptr(), 1 if K.dtype == torch.float32 else 0,
             K.stride(0), K.stride(1), V.stride(0), V.stride(1),
             _hip.ptr(src_rows), T, H, D, int(page_size), k, index_repr, 1 if sel == "abs" else 0, mode,
-            gt, gc, _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
+            gt, gc, 1 if v_bf16 else 0, _hip.ptr(dst_pages), _hip.ptr(dst_groups), store_table(K.device).data_ptr(),
             planes["k_base"].data_ptr(), planes["k_scale"].data_ptr(), planes["k_zp"].data_ptr(),
             _hip.ptr(planes.get("k_fp4_mapscale")), _hip.ptr(planes.get("k_fp4_mapcenter")),
             _hip.ptr(index_plane), _hip.ptr(planes.get("k_oval")),
@@ -180,7 +183,7 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
                  page_size: int = 16, outliers_per_vector: int = 6,
                  device: Any = "cuda", outlier_repr: str = "bitmap",
                  kv_outlier_map: bool = True, int8_scale: bool = True,
-                 group_tokens: int = 32, group_channels: int = 32) -> Dict[str, Any]:
+                 group_tokens: int = 32, group_channels: int = 32, v_format: str = "i2") -> Dict[str, Any]:
     """Empty planes with the shapes and dtypes of reference ``pack.py:576-623``;
     ``num_group_slots`` counts K groups of ``group_tokens`` tokens."""
     P, G, H, D, ps, k = num_pages, num_group_slots, n_kv_heads, head_dim, page_size, outliers_per_vector
@@ -191,7 +194,8 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
         "k_base": torch.empty(P, ps, H, D // 4, dtype=u8, device=dev),
         "k_scale": torch.empty(G, H, D, dtype=i8, device=dev),
         "k_zp": torch.empty(G, H, D, dtype=bf, device=dev),
-        "v_main": torch.empty(P, ps, H, D // 4, dtype=u8, device=dev),
+        "v_main": (torch.empty(P, ps, H, D, dtype=bf, device=dev) if str(v_format).lower() == "bf16"
+                   else torch.empty(P, ps, H, D // 4, dtype=u8, device=dev)),     # pack.py:596-598
         "v_scale": torch.empty(P, ps, H, D // int(group_channels), dtype=i8, device=dev),
         "v_zp": torch.empty(P, ps, H, D // int(group_channels), dtype=bf, device=dev),
         "k_oidx": None, "k_crank": None,
@@ -286,8 +290,6 @@ def ommx_pack_kv_canonical_block(
         unsupported.append(f"outlier_select={outlier_select!r}")
     if k > 16:
         unsupported.append("more than 16 outliers per vector")
-    if vfmt != "i2":
-        unsupported.append("v_format='bf16'")
     if scale_dtype != torch.bfloat16:
         unsupported.append(f"scale_dtype={scale_dtype}")
     if D > 256 or D % 32 != 0:
@@ -315,13 +317,13 @@ def ommx_pack_kv_canonical_block(
     planes = alloc_planes(pages, G, H, D, page_size=int(page_size), outliers_per_vector=k, device=dev,
                           outlier_repr=repr_l, kv_outlier_map=bool(kv_outlier_map),
                           int8_scale=bool(use_pow2) and bool(kv_int8_scale),
-                          group_tokens=gt, group_channels=gc)
+                          group_tokens=gt, group_channels=gc, v_format=vfmt)
     err = torch.zeros(1, dtype=torch.int32, device=dev)
     if T > 0:
         store_pack_into(Kd, Vd, planes, outliers_per_vector=k, page_size=int(page_size), err_flag=err,
                         outlier_repr=repr_l, outlier_select=outlier_select,
                         use_pow2=bool(use_pow2), kv_int8_scale=bool(kv_int8_scale),
-                        group_tokens=gt, group_channels=gc)
+                        group_tokens=gt, group_channels=gc, v_format=vfmt)
     raise_for_store_errors(int(err.item()))
 
     def _to(t):

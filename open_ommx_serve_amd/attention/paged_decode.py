@@ -108,7 +108,9 @@ def ommx_paged_decode_attention_canonical(
                 f"derived GROUP_TOKENS={group_tokens} (pages={pages} page_size={ps} "
                 f"n_group_slots={ngroups}) must be in {{16,32,64,128}}")
     vsc = int(v_scale.shape[-1])
-    group_channels = 32 if vsc == 0 else (int(v_main.shape[-1]) * 4) // vsc
+    v_bf16 = v_main.dtype == torch.bfloat16            # rows kept unquantised (pack.py:596-602)
+    v_width = int(v_main.shape[-1]) if v_bf16 else int(v_main.shape[-1]) * 4
+    group_channels = 32 if vsc == 0 else v_width // vsc
     if group_channels not in (16, 32, 64, 128):
         raise ValueError(f"derived GROUP_CHANNELS={group_channels} must be in {{16,32,64,128}}")
     kfmt = str(k_format).lower()
@@ -118,7 +120,7 @@ def ommx_paged_decode_attention_canonical(
         raise ValueError("combinadic_read and bitmap_read are mutually exclusive outlier-index sources")
     B, Hq = int(q.shape[0]), int(q.shape[1])
     D = int(k_base.shape[-1]) * 4
-    Dv = int(v_main.shape[-1]) * 4
+    Dv = v_width
     Hkv = int(k_base.shape[-2])
     if Dv % group_channels != 0:
         raise ValueError(f"canonical KV requires head_dim % {group_channels} == 0; got Lv={Dv}.")
@@ -231,7 +233,8 @@ def ommx_paged_decode_attention_canonical(
             1 if req_to_token.dtype == torch.int64 else 0,
             b_seq_len.data_ptr(),
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, group_tokens, group_channels, S,
+            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, group_tokens, group_channels,
+            1 if v_bf16 else 0, S,
             float(sm_scale), float(logit_cap), off, gbase, stream)
         _hip.check(rc, "ommx_decode_splitkv")
         rc = lib.ommx_decode_combine(

@@ -28,7 +28,7 @@ extern "C" int ommx_decode_splitkv(
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int num_splits,
+    int group_tokens, int group_channels, int v_bf16, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
@@ -80,7 +80,7 @@ extern "C" int ommx_decode_splitkv(
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
                  packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
-                 group_tokens, group_channels};
+                 group_tokens, group_channels, v_bf16 ? 1 : 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc = launch_decode_fast(a, D, R, st);
     if (rc == 1) rc = launch_decode_ref(a, D, R, st);
@@ -99,7 +99,7 @@ extern "C" int ommx_decode_splitkv_ref(
     int table_i64, const int32_t* b_seq_len,
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int num_splits,
+    int group_tokens, int group_channels, int v_bf16, int num_splits,
     float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
     void* stream) {
     using namespace ommx;
@@ -116,7 +116,7 @@ extern "C" int ommx_decode_splitkv_ref(
                  table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
                  B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
                  packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
-                 group_tokens, group_channels};
+                 group_tokens, group_channels, v_bf16 ? 1 : 0};
     if (launch_decode_ref(a, D, Hq / Hkv, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_splitkv_ref: unsupported shape");
         return -1;

@@ -19,6 +19,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
     return static_cast<uint16_t>(u >> 16);
 }
 
+// fp32 -> bf16 as torch's `.to(torch.bfloat16)` does for any input: round to nearest even,
+// infinities kept, NaN made quiet.
+__device__ __forceinline__ uint16_t f32_to_bf16_any(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    return f32_to_bf16_rne(x);
+}
+
 __device__ __forceinline__ bool is_finite_f32(float x) {
     return (__float_as_uint(x) & 0x7F800000u) != 0x7F800000u;
 }

@@ -858,7 +858,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     if (Dh != 128 || !(R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
     if (a.scale_bf16) return 1;      // operands are exact only for power-of-two steps
-    if (a.gt != 32 || a.gc != 32) return 1;
+    if (a.gt != 32 || a.gc != 32 || a.v_bf16) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);    // one wave per kv head

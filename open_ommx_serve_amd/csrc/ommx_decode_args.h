@@ -20,6 +20,7 @@ struct DecodeArgs {
     int idx_repr;                    // 0 flat bitmap, 1 relidx7
     int scale_bf16;                  // k_scale / v_scale hold bf16 steps instead of int8 exponents
     int gt, gc;                      // tokens per K group, channels per V vector (16, 32, 64 or 128)
+    int v_bf16;                      // v_main holds bf16 rows [P,ps,H,D] instead of INT2 codes
 };
 
 // 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)

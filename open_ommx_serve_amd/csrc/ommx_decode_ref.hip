@@ -181,6 +181,16 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
                 const int t = ts * TPS + i;
                 if (n0 + t < n_end) {
                     const int64_t rowh = s_row[t] * a.Hkv + kvh;
+                    if (a.v_bf16) {                 // the rows as they are
+                        const uint16_t* vr = reinterpret_cast<const uint16_t*>(a.v_main) + rowh * D + bc * 4;
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const float p = s_p[r * 32 + t];
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(p, bf16_to_f32(vr[c]), acc[r][c]);
+                        }
+                        continue;
+                    }
                     const uint32_t byte = a.v_main[rowh * (D / 4) + bc];
                     const int64_t vg = rowh * ngv + (bc * 4) / a.gc;
                     const float vs = a.scale_bf16

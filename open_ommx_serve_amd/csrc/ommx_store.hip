@@ -361,7 +361,8 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                                int64_t k_ts, int64_t k_hs, int64_t v_ts, int64_t v_hs,
                                const int32_t* src_rows, int T, int H, int D, int page_size,
                                int k_outliers, int index_repr, int select_abs, int scale_mode,
-                               int group_tokens, int group_channels, const int32_t* dst_pages,
+                               int group_tokens, int group_channels, int v_bf16,
+                               const int32_t* dst_pages,
                                const int32_t* dst_groups, const float* table,
                                uint8_t* k_base, void* k_scale, uint16_t* k_zp,
                                uint16_t* k_ms, uint16_t* k_mc, uint8_t* k_index,
@@ -399,9 +400,9 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
                 static_cast<int8_t*>(v_scale), v_zp,
                 err_flag, H, D, page_size, k_outliers,
                 (reinterpret_cast<uintptr_t>(V) % 16 == 0 && v_ts % 8 == 0 && v_hs % 8 == 0) ? 1 : 0,
-                index_repr, select_abs ? 1 : 0, scale_mode, gt, gc};
+                index_repr, select_abs ? 1 : 0, scale_mode, gt, gc, v_bf16 ? 1 : 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (gt != 32 || gc != 32 || k_outliers > 8 || 32 % page_size) {     // everything but the 32x32 recipe
+    if (gt != 32 || gc != 32 || k_outliers > 8 || 32 % page_size || v_bf16) {   // everything but the 32x32 recipe
         if (launch_store_generic(a, T, in_dtype, st) != 0) {
             set_error("ommx_store_pack: no kernel for this recipe");
             return -1;

@@ -32,6 +32,7 @@ struct StoreArgs {
     int scale_mode;         // 0 power of two, int8 exponent plane; 1 power of two, bf16 plane;
                             // 2 bf16((max - min) / 3) as it comes, bf16 plane (pack.py:459-463, 586-590)
     int gt, gc;             // tokens per K vector, channels per V vector (32 and 32 in the tuned kernel)
+    int v_bf16;             // V is kept as bf16 rows [pages, ps, H, D]; v_scale = 1, v_zp = 0 (pack.py:596-602)
 };
 
 

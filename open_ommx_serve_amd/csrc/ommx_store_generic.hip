@@ -195,6 +195,19 @@ __global__ void __launch_bounds__(256) store_generic_kernel(StoreArgs a) {
         const int64_t prow = phys_row(tok);
         const int64_t row = a.src_rows ? a.src_rows[tok] : tok;
         const int64_t vbase = row * a.v_ts + (int64_t)h * a.v_hs + GC * j;
+        if (a.v_bf16) {     // the row itself, rounded to bf16; the step planes are placeholders
+            uint16_t* dst16 = reinterpret_cast<uint16_t*>(a.v_main) + (prow * H + h) * (int64_t)D + GC * j;
+#pragma unroll
+            for (int c = 0; c < GC; ++c) {
+                if (F32) dst16[c] = f32_to_bf16_any(static_cast<const float*>(a.V)[vbase + c]);
+                else dst16[c] = static_cast<const uint16_t*>(a.V)[vbase + c];
+            }
+            const int64_t vidx = (prow * H + h) * ngv + j;
+            if (a.scale_mode == 0) a.v_scale[vidx] = 1;
+            else reinterpret_cast<uint16_t*>(a.v_scale)[vidx] = 0x3F80;     // bf16 1.0
+            a.v_zp[vidx] = 0;
+            continue;
+        }
         float v[GC];
         bool fin = true;
         float mn = 0.0f, mx = 0.0f;

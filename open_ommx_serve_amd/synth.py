@@ -115,7 +115,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
                       outlier_repr: str = "bitmap", kv_outlier_map: bool = True,
                       use_pow2: bool = True, kv_int8_scale: bool = True,
-                      group_tokens: int = 32, group_channels: int = 32) -> DecodeCase:
+                      group_tokens: int = 32, group_channels: int = 32, v_format: str = "i2") -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -140,7 +140,7 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                           outliers_per_vector=outliers_per_vector, device=dev,
                           outlier_repr=outlier_repr, kv_outlier_map=kv_outlier_map,
                           int8_scale=bool(use_pow2) and bool(kv_int8_scale),
-                          group_tokens=gt, group_channels=gc)
+                          group_tokens=gt, group_channels=gc, v_format=v_format)
     planes["outlier_repr"] = str(outlier_repr).lower()
     planes["group_tokens"], planes["group_channels"] = gt, gc
     for t in planes.values():
@@ -174,7 +174,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                             dst_pages=torch.from_numpy(rt[b, :n_pages[b]].astype(np.int32)).to(dev),
                             dst_groups=torch.from_numpy(rg[b, :n_groups[b]].astype(np.int32)).to(dev),
                             err_flag=err, outlier_repr=outlier_repr, use_pow2=use_pow2,
-                            kv_int8_scale=kv_int8_scale, group_tokens=gt, group_channels=gc)
+                            kv_int8_scale=kv_int8_scale, group_tokens=gt, group_channels=gc,
+                            v_format=v_format)
         po += n_pages[b]
         go += n_groups[b]
         if keep_source:

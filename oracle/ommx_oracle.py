@@ -232,7 +232,8 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
             outliers_per_vector: int = 6, outlier_repr: str = "bitmap",
             kv_outlier_map: bool = True, outlier_select: str = "signed",
             use_pow2: bool = True, kv_int8_scale: bool = True,
-            group_tokens: int = GROUP_TOKENS, group_channels: int = GROUP_CHANNELS) -> Dict[str, object]:
+            group_tokens: int = GROUP_TOKENS, group_channels: int = GROUP_CHANNELS,
+            v_format: str = "i2") -> Dict[str, object]:
     """The pinned serving recipe of ``ommx_pack_kv_canonical_block`` (pack.py:293-655):
     i2f4, signed select, bitmap (or relidx7) index plane, pow2 scales stored as int8
     exponents, dedicated FP4 map, 32-token K vectors, 32-channel V vectors, bf16 side planes.
@@ -314,6 +315,14 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     planes["k_zp"] = zp.squeeze(-1).permute(2, 0, 1).contiguous().to(torch.bfloat16)
 
     # ---- V, vector = (token, head, 32 channels)                         pack.py:604-623
+    vfmt = str(v_format).lower()
+    if vfmt not in ("i2", "bf16"):
+        raise ValueError("v_format must be i2 or bf16")
+    if vfmt == "bf16":                                                    # pack.py:596-602
+        planes["v_main"] = V.to(torch.bfloat16).reshape(pages, page_size, H, D).contiguous()
+        planes["v_scale"] = torch.ones(pages, page_size, H, NGV, dtype=torch.int8 if int8_scale else torch.bfloat16)
+        planes["v_zp"] = torch.zeros(pages, page_size, H, NGV, dtype=torch.bfloat16)
+        return _finish_planes(planes, locals())
     gv = Vf.reshape(T, H, NGV, gc)
     if not bool(torch.isfinite(gv).all()):
         raise ValueError("V pack: non-finite input")
@@ -327,16 +336,21 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     vs_flat = vscale.squeeze(-1).reshape(pages, page_size, H, NGV).contiguous()
     planes["v_scale"] = pow2_exponent(vs_flat).to(torch.int8) if int8_scale else vs_flat.to(torch.bfloat16)
     planes["v_zp"] = vzp.squeeze(-1).to(torch.bfloat16).reshape(pages, page_size, H, NGV).contiguous()
+    return _finish_planes(planes, locals())
 
+
+def _finish_planes(planes: Dict[str, object], v: Dict[str, object]) -> Dict[str, object]:
+    """Identity tables and the metadata keys of pack.py:628-654."""
+    gt, k = v["gt"], v["k"]
     planes.update(
-        k_crank=None, k_field_bytes=(gt + 7) // 8 if (k > 0 and repr_l == "bitmap") else 0,
-        req_to_token=torch.arange(pages, dtype=torch.int32).reshape(1, pages),
-        req_to_group=torch.arange(G, dtype=torch.int32).reshape(1, G),
-        head_dim=D, n_kv_heads=H, num_tokens=T, n_groups=G, page_size=int(page_size),
-        outliers_per_vector=k, outlier_repr=repr_l, outlier_select=sel,
-        group_tokens=gt, group_channels=gc, k_format="i2f4", v_format="i2",
-        k_base_bits=2, oval_bits=4, use_pow2=bool(use_pow2),
-        kv_outlier_map=bool(kv_outlier_map) and k > 0, kv_int8_scale=int8_scale)
+        k_crank=None, k_field_bytes=(gt + 7) // 8 if (k > 0 and v["repr_l"] == "bitmap") else 0,
+        req_to_token=torch.arange(v["pages"], dtype=torch.int32).reshape(1, v["pages"]),
+        req_to_group=torch.arange(v["G"], dtype=torch.int32).reshape(1, v["G"]),
+        head_dim=v["D"], n_kv_heads=v["H"], num_tokens=v["T"], n_groups=v["G"], page_size=int(v["page_size"]),
+        outliers_per_vector=k, outlier_repr=v["repr_l"], outlier_select=v["sel"],
+        group_tokens=gt, group_channels=v["gc"], k_format="i2f4", v_format=v["vfmt"],
+        k_base_bits=2, oval_bits=4, use_pow2=bool(v["use_pow2"]),
+        kv_outlier_map=bool(v["kv_outlier_map"]) and k > 0, kv_int8_scale=v["int8_scale"])
     return planes
 
 
@@ -381,6 +395,8 @@ def dequant_kv(planes: Dict[str, object]) -> Tuple[torch.Tensor, torch.Tensor]:
         Kg = Kd.reshape(G, gt, H, D).permute(0, 2, 3, 1).contiguous()        # [G,H,D,gt]
         Kg.scatter_(-1, pos, dq)
         Kd = Kg.permute(0, 3, 1, 2).reshape(T, H, D)
+    if planes["v_main"].dtype == torch.bfloat16:                             # pack.py:766-769
+        return Kd, planes["v_main"].to(torch.float32).reshape(T, H, D)
     vcode = unpack_int2(planes["v_main"].reshape(T, H, D4)).to(torch.float32)
     NGV = D // gc
     vs = _steps(planes["v_scale"]).reshape(T, H, NGV, 1)
@@ -503,6 +519,8 @@ def gather_request(planes: Dict[str, object], req_to_token: torch.Tensor,
         Kg = Kp.reshape(n_g, gt, H, D).permute(0, 2, 3, 1).contiguous()
         Kg.scatter_(-1, pos, dq)
         Kd = Kg.permute(0, 3, 1, 2).reshape(Lp, H, D)[:L]
+    if planes["v_main"].dtype == torch.bfloat16:
+        return Kd, planes["v_main"].reshape(P * ps, H, D)[rows].to(torch.float32)
     vcode = unpack_int2(planes["v_main"].reshape(P * ps, H, D4)[rows]).to(torch.float32)
     NGV = D // gc
     vs = _steps(planes["v_scale"].reshape(P * ps, H, NGV)[rows]).unsqueeze(-1)

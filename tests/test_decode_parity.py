@@ -237,6 +237,17 @@ def test_other_group_sizes(hq, hkv, D, recipe):
         _check(_run(case, num_kv_splits=S), want, f"{recipe} S{S}")
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(group_tokens=64, group_channels=64, outlier_repr="relidx7")])
+def test_bf16_v_rows(kw):
+    """v_format="bf16": P.V from unquantised bf16 rows (pack.py:596-602, dequant :766-769)."""
+    case = build_decode_case([900, 50], q_heads=32, kv_heads=8, seed=71, permute_tables=True,
+                             sparse_frac=0.005, v_format="bf16", **kw)
+    assert case.planes["v_main"].dtype == torch.bfloat16
+    want = _oracle(case)
+    for S in (None, 2):
+        _check(_run(case, num_kv_splits=S), want, f"bf16 V {kw} S{S}")
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)

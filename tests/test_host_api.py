@@ -110,7 +110,7 @@ def test_pack_argument_errors_match_the_reference():
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "outlier_repr": "combinadic"})
     with pytest.raises(NotImplementedError):
-        P(K, K, **{**good, "v_format": "bf16"})
+        P(K, K, **{**good, "scale_dtype": torch.float16})
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "outliers_per_vector": 17, "outlier_repr": "relidx7"})
     if not torch.cuda.is_available():

@@ -168,6 +168,27 @@ def test_store_other_group_sizes(recipe, T, H, D, fp32):
     assert got["k_field_bytes"] == want["k_field_bytes"]
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(group_tokens=64, group_channels=64, outlier_repr="relidx7"),
+                                dict(use_pow2=False)])
+@pytest.mark.parametrize("fp32", [False, True])
+def test_store_bf16_v_rows(kw, fp32):
+    """v_format="bf16" (pack.py:596-602): V is kept as bf16 rows [pages, ps, H, D], the step planes
+    are ones and zeros; K is packed as usual."""
+    K, V = synth_kv(128, 4, 128, 900, sparse_frac=0.01)
+    if fp32:
+        K, V = K.float() * 1.0009765625, V.float() * 0.99951171875
+    args = dict(outliers_per_vector=6, outlier_repr="bitmap", outlier_select="signed", v_format="bf16")
+    args.update(kw)
+    want = O.pack_kv(K, V, **args)
+    got = _hip(K, V, **args)
+    assert got["v_format"] == "bf16" and got["v_main"].dtype == torch.bfloat16
+    assert tuple(got["v_main"].shape) == (8, 16, 4, 128)
+    for n in ("v_main", "v_scale", "v_zp", "k_base", "k_scale", "k_zp", "k_oval",
+              "k_oidx" if args["outlier_repr"] == "relidx7" else "k_obmp", "k_fp4_mapscale", "k_fp4_mapcenter"):
+        assert got[n].dtype == want[n].dtype and got[n].shape == want[n].shape, n
+        assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
