@@ -1,5 +1,5 @@
-// Tuned split-KV decode kernel for gfx950: head_dim 128, 4 or 8 q heads per kv head, 6 (or 0)
-// outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
+// Tuned split-KV decode kernel for gfx950: head_dim 128, 1, 2, 4 or 8 q heads per kv head, 6 (or
+// 0) outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
 //
 // Work decomposition.  A wavefront owns one kv head (and all 4 or 8 of its q heads) of one
 // split and walks it 64 tokens (two 32-token K groups) at a time; waves never synchronise with
@@ -273,7 +273,9 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 // bitmaps, 1 = from 7-bit position streams (6 bytes per channel and group at 6 outliers).
 // OWN_MAP: outliers decode through their own (map_scale, centre) pair; false = through the
 // base scale and zero point (level * 2^e + zp), and there are no map planes.
-template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP>
+// PARTIAL (HR = 4 only): the kv head serves 1 or 2 q heads; the spare head slots repeat the
+// last head and are not written out.
+template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -290,7 +292,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int Hkv = a.Hkv;
     const int waves = blockDim.x >> 6;
     const int kvh = blockIdx.y * waves + wave;
-    const int qh0 = kvh * HR;             // first of this wave's q heads
+    const int heads = PARTIAL ? a.Hq / Hkv : HR;      // q heads this kv head really serves
+    const int qh0 = kvh * heads;          // first of this wave's q heads
     const int b = blockIdx.z, sp = blockIdx.x;
     const int L = a.seq[b];
     const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
@@ -410,7 +413,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     {
         // this lane's 32 channels of q: 16 dwords, channel 2i in the low half of dword i
         const uint32_t* qh = reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + (j & (HR - 1))) * a.q_sh + 32 * kq);
+            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & (HR - 1), heads - 1)) * a.q_sh + 32 * kq);
         uint32_t qw[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) qw[i] = qh[i];
@@ -444,7 +447,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 #pragma unroll
         for (int r = 0; r < HR; ++r)
             qraw[r] = *reinterpret_cast<const uint32_t*>(
-                a.q + b * a.q_sb + (int64_t)(qh0 + r) * a.q_sh + 2 * lane);
+                a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
         if constexpr (HR == 4) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -811,6 +814,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             const int ch0 = 16 * (j & 7) + 8 * (j >> 3);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
+                if (r >= heads) break;
                 float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
                 const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
 #pragma unroll
@@ -844,7 +848,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             }
         }
     }
-    if (j < 4 && kq < HR / 4) {                    // lane 16*hg + r holds head 4*hg + r
+    if (j < 4 && kq < HR / 4 && 4 * kq + j < heads) {     // lane 16*hg + r holds head 4*hg + r
         float* dst = a.al + b * a.al_b + (int64_t)(qh0 + 4 * kq + j) * a.al_h + (int64_t)sp * a.al_s;
         const float lt = j == 0 ? l_tot[0] : (j == 1 ? l_tot[1] : (j == 2 ? l_tot[2] : l_tot[3]));
         const float mt = j == 0 ? m_run[0] : (j == 1 ? m_run[1] : (j == 2 ? m_run[2] : m_run[3]));
@@ -856,19 +860,28 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 
 // Returns 0 when launched, 1 when the shape is not covered by the tuned kernel.
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
-    if (Dh != 128 || !(R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
+    if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
     if (a.scale_bf16) return 1;      // operands are exact only for power-of-two steps
     if (a.gt != 32 || a.gc != 32 || a.v_bf16) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);    // one wave per kv head
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * (R == 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
+    const size_t shm = (size_t)waves * (R <= 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
                                                : (a.kout == 6 ? LdsMap<8>::END : LdsMap<8>::DT));
     const bool own_map = a.k_ms != nullptr;
 #define OMMX_LAUNCH(HR, IDX, MAP) \
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a)
-    if (a.kout == 6) {
+#define OMMX_LAUNCH_PARTIAL(IDX, MAP) \
+    hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, IDX, MAP, true>), grid, block, shm, st, a)
+    if (a.kout == 6 && R < 4) {
+        switch ((a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
+            case 0: OMMX_LAUNCH_PARTIAL(0, false); break;
+            case 1: OMMX_LAUNCH_PARTIAL(0, true); break;
+            case 2: OMMX_LAUNCH_PARTIAL(1, false); break;
+            default: OMMX_LAUNCH_PARTIAL(1, true); break;
+        }
+    } else if (a.kout == 6) {
         const int variant = (R == 8 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0);
         switch (variant) {
             case 0: OMMX_LAUNCH(4, 0, false); break;
@@ -880,12 +893,15 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
             case 6: OMMX_LAUNCH(8, 1, false); break;
             default: OMMX_LAUNCH(8, 1, true); break;
         }
+    } else if (R < 4) {
+        hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4, 0, true, true>), grid, block, shm, st, a);
     } else if (R == 4) {
         hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 4, 0, true>), grid, block, shm, st, a);
     } else {
         hipLaunchKernelGGL((decode_splitkv_mfma_kernel<false, 8, 0, true>), grid, block, shm, st, a);
     }
 #undef OMMX_LAUNCH
+#undef OMMX_LAUNCH_PARTIAL
     return 0;
 }
 
