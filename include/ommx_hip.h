@@ -118,20 +118,20 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 plane, int8 exponents, and the dedicated FP4 map (the serving recipe) or,
  *                 with k_ms = k_mc = NULL, outliers on the base scale and zero point
  *   req_to_token  int32 or int64 (table_i64) [B, >= ceil((L+off)/ps)], row stride rt_stride
- *   req_to_group  same type [B, >= seg_group_base + ceil(L/32)], row stride rg_stride
+ *   req_to_group  same type [B, >= seg_group_base + ceil(L/group_tokens)], row stride rg_stride
  *   b_seq_len     int32[B] packed tokens per request (device; bounds the loop)
  *   attn_logits   f32 [B,Hq,>=num_splits,D+1] with strides al_stride_b/h/s: partial
  *                 o (normalised) in [0,D) and lse at D; an empty split writes o=0,
  *                 lse=-inf (paged_decode.py:2262-2284)
- * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/32)*32
- * (paged_decode.py:1429-1432).  Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64;
- * num_splits <= 256; planes 8-byte aligned.  scale_bf16 = 1: k_scale / v_scale hold the steps
- * themselves as bf16 instead of int8 exponents (plain kernel only).  group_tokens /
- * group_channels: tokens per K group and channels per V vector, 16, 32, 64 or 128; the split
- * length is rounded to group_tokens, and ommx_decode_combine must be given the same value.
- * 32 and 32 with 6 (or 0) outliers is the matrix-core shape; k_outliers up to 16 otherwise.
- * v_bf16 = 1: v_main is bf16 [P,ps,H,D] and v_scale / v_zp are ignored (plain kernel only).  head_dim 128 with r = 4 or 8 and 6 (or 0)
- * outliers runs on the matrix-core kernel, every other supported shape on the plain fp32 kernel.
+ * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/gt)*gt with
+ * gt = group_tokens (paged_decode.py:1429-1432); ommx_decode_combine must be given the same gt.
+ * Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64; num_splits <= 256; planes 8-byte aligned.
+ *   group_tokens / group_channels   tokens per K group and channels per V vector: 16, 32, 64, 128
+ *   scale_bf16 = 1   k_scale / v_scale hold the steps themselves as bf16, not int8 exponents
+ *   v_bf16 = 1       v_main is bf16 [P,ps,H,D]; v_scale / v_zp are ignored
+ * The matrix-core kernel runs head_dim 128, 32-token groups, 32-channel V vectors, INT2 V, int8
+ * exponents and 6 (or 0) outliers, with either index plane and either outlier map; every other
+ * supported shape or recipe (k_outliers up to 16) runs on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
