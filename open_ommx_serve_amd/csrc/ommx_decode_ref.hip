@@ -21,7 +21,7 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
     float* s_q = s_K + (32 * KS > TS * R * D ? 32 * KS : TS * R * D);   // [R][D]
     float* s_sc = s_q + R * D;            // [2][D]  (two K groups per tile when groups are 16 tokens)
     float* s_zp = s_sc + 2 * D;           // [2][D]
-    float* s_p = s_zp + D;                // [R][32]
+    float* s_p = s_zp + 2 * D;            // [R][32]
     float* s_al = s_p + R * 32;           // [R]
     int64_t* s_row = reinterpret_cast<int64_t*>(s_al + 8);   // [32]
 

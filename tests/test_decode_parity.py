@@ -248,6 +248,39 @@ def test_bf16_v_rows(kw):
         _check(_run(case, num_kv_splits=S), want, f"bf16 V {kw} S{S}")
 
 
+def test_randomised_recipes_against_the_oracle():
+    """Forty random draws over the whole recipe space the kernels accept (group sizes, outlier
+    count, index plane, outlier map, step mode, V format, head shapes, table dtype, splits,
+    ragged lengths cut inside the last group), each against the fp64 oracle."""
+    g = torch.Generator().manual_seed(2024)
+
+    def pick(*xs):
+        return xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+
+    for it in range(40):
+        gt, gc = pick(16, 32, 64, 128), pick(16, 32, 64)
+        D = pick(64, 128)
+        rep = pick("bitmap", "relidx7")
+        k = pick(0, 1, 3, 6, 8) if rep == "bitmap" else pick(0, 2, 6, 10, 16)
+        k = min(k, gt)
+        hkv = pick(1, 2, 4)
+        r = pick(1, 2, 4, 8)
+        recipe = dict(group_tokens=gt, group_channels=gc, outliers_per_vector=k, outlier_repr=rep,
+                      kv_outlier_map=pick(True, False), use_pow2=pick(True, True, False),
+                      kv_int8_scale=pick(True, False), v_format=pick("i2", "i2", "bf16"))
+        B = pick(1, 2, 3)
+        lens = [int(torch.randint(1, 1400, (1,), generator=g)) for _ in range(B)]
+        case = build_decode_case(lens, q_heads=hkv * r, kv_heads=hkv, head_dim=D, seed=3000 + it,
+                                 permute_tables=pick(True, False), sparse_frac=pick(0.0, 0.01),
+                                 table_dtype=pick(torch.int32, torch.int64), **recipe)
+        if pick(0, 1):
+            cut = torch.tensor([max(0, n - int(torch.randint(0, gt, (1,), generator=g)))
+                                for n in case.b_seq_len.tolist()], dtype=torch.int32)
+            case.b_seq_len.copy_(cut)
+        S = pick(None, 1, 3, 16, 200)
+        _check(_run(case, num_kv_splits=S), _oracle(case), f"case {it}: lens={lens} D={D} r={r} hkv={hkv} S={S} {recipe}")
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_no_outliers_recipe(ref_kernel):
     case = build_decode_case([1000], q_heads=8, kv_heads=2, seed=10, outliers_per_vector=0)
