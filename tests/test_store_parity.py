@@ -189,6 +189,53 @@ def test_store_bf16_v_rows(kw, fp32):
         assert np.array_equal(bits_of(got[n]), bits_of(want[n])), n
 
 
+def test_store_randomised_recipes():
+    """Sixty random draws over the recipe space (group sizes, outlier count / selection / index
+    plane / map, step mode, V format, page size, head shapes, input dtype, value patterns with
+    ties): every plane bit for bit against the oracle."""
+    g = torch.Generator().manual_seed(77)
+
+    def pick(*xs):
+        return xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+
+    for it in range(60):
+        gt, gc = pick(16, 32, 64, 128), pick(16, 32, 64, 128)
+        D = pick(32, 64, 128, 256)
+        gc = min(gc, D)
+        H = pick(1, 2, 5, 8)
+        ps = pick(8, 16, 32)
+        T = gt * pick(1, 2, 5)
+        while T % ps:
+            T += gt
+        rep = pick("bitmap", "relidx7")
+        k = min(pick(0, 1, 2, 3, 6, 7, 8, 11, 16), gt)
+        recipe = dict(group_tokens=gt, group_channels=gc, outliers_per_vector=k, outlier_repr=rep,
+                      outlier_select=pick("signed", "abs"), kv_outlier_map=pick(True, False),
+                      use_pow2=pick(True, False), kv_int8_scale=pick(True, False),
+                      v_format=pick("i2", "i2", "bf16"), page_size=ps)
+        K, V = synth_kv(T, H, D, 4000 + it, outlier_channels=min(4, D // 8), sparse_frac=pick(0.0, 0.02))
+        if pick(0, 1, 2) == 0:                      # a block of heavy ties between values of both signs
+            lv = torch.tensor([-3.0, -1.0, 1.0, 0.5, -0.5, 2.0, -2.0, 3.0, 0.25])
+            n = min(T, 2 * gt)
+            K[:n] = lv[torch.randint(0, 9, (n, H, D), generator=g)].to(torch.bfloat16)
+            V[:n] = lv[torch.randint(0, 9, (n, H, D), generator=g)].to(torch.bfloat16)
+        if pick(0, 1):
+            K, V = K.float() * 1.0009765625, V.float() * 0.99951171875
+        what = f"case {it}: T={T} H={H} D={D} {K.dtype} {recipe}"
+        want = O.pack_kv(K, V, **recipe)
+        got = _hip(K, V, **recipe)
+        for n in ("k_base", "k_scale", "k_zp", "k_obmp", "k_oidx", "k_oval", "k_fp4_mapscale",
+                  "k_fp4_mapcenter", "v_main", "v_scale", "v_zp"):
+            if want[n] is None:
+                assert got[n] is None, (what, n)
+                continue
+            assert got[n].dtype == want[n].dtype and got[n].shape == want[n].shape, (what, n)
+            a, b = bits_of(got[n]), bits_of(want[n])
+            if n in ("k_zp", "k_fp4_mapcenter", "v_zp"):        # the sign of a zero is free (conftest)
+                a, b = np.where(a == 0x8000, 0, a), np.where(b == 0x8000, 0, b)
+            assert np.array_equal(a, b), f"{what}: plane {n}"
+
+
 @pytest.mark.parametrize("k", [0, 1, 2, 5, 8])
 def test_store_other_outlier_counts(k):
     K, V = synth_kv(128, 2, 64, 10 + k)
