@@ -325,21 +325,20 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int tok_off = a.gbase * 32 + a.off;
     const char* const rt_b = static_cast<const char*>(a.rt) + ((b * a.rt_s) << tsh);
     const char* const rg_b = static_cast<const char*>(a.rg) + ((b * a.rg_s + a.gbase) << tsh);
-    const uint8_t* const kb_lane = a.k_base + kvh * 32 + 8 * kq;
-    const uint8_t* const vb_lane = a.v_main + kvh * 32 + 8 * kq;
+    const uint8_t* const kb_head = a.k_base + kvh * 32;      // a lane loads its own token's 32-byte rows
+    const uint8_t* const vb_head = a.v_main + kvh * 32;
     const int8_t* const vs_head = a.v_scale + kvh * 4;
     const uint16_t* const vz_head = a.v_zp + kvh * 4;
 
     // The loop is software-pipelined by hand: table entries are fetched two iterations
     // ahead, plane data one iteration ahead, each into the registers its previous use
     // has just released.
-    int rows[4], gsl[2];                  // physical token rows / group slots of the NEXT data loads
+    int row1, gsl[2];                     // physical row of token n + lane / group slots, of the NEXT data loads
     auto fetch_tables = [&](int n) {
-#pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-            const int p = min(n + 16 * tb + j, last) + tok_off;
+        {
+            const int p = min(n + lane, last) + tok_off;
             const int pg = *reinterpret_cast<const int*>(rt_b + ((uint32_t)(p >> ps_sh) << tsh));
-            rows[tb] = (pg << ps_sh) + (p & ps_mask);
+            row1 = (pg << ps_sh) + (p & ps_mask);
         }
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -347,17 +346,16 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             gsl[g] = *reinterpret_cast<const int*>(rg_b + ((uint32_t)gi << tsh));
         }
     };
-    u32x2 kw[4], vw[4], vzp;
+    u32x4 kr[2], vr[2];
+    u32x2 vzp;
     uint32_t vsc;
     auto fetch_kv = [&]() {
-#pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-            const uint64_t ro = (uint64_t)(uint32_t)rows[tb] * row_bytes;
-            kw[tb] = *reinterpret_cast<const u32x2*>(kb_lane + ro);
-            vw[tb] = *reinterpret_cast<const u32x2*>(vb_lane + ro);
-        }
-        // this lane's own token (n + lane) is column j of token block kq
-        const uint32_t my_row = kq == 0 ? rows[0] : (kq == 1 ? rows[1] : (kq == 2 ? rows[2] : rows[3]));
+        const uint64_t ro = (uint64_t)(uint32_t)row1 * row_bytes;
+        kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
+        kr[1] = *reinterpret_cast<const u32x4*>(kb_head + ro + 16);
+        vr[0] = *reinterpret_cast<const u32x4*>(vb_head + ro);
+        vr[1] = *reinterpret_cast<const u32x4*>(vb_head + ro + 16);
+        const uint32_t my_row = row1;
         vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
         vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
     };
@@ -481,12 +479,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 
         // ---------------------------------------------------------------- stage to LDS
         // K code rows (for the outlier pass), transposed V dwords
+        {   // row of token lane: 32 code bytes of K (rows are 8-byte aligned), 8 dwords of V
+            u32x2* krow = reinterpret_cast<u32x2*>(sm + OFF_KT + lane * KT_ROW);
+            krow[0] = u32x2{kr[0][0], kr[0][1]};
+            krow[1] = u32x2{kr[0][2], kr[0][3]};
+            krow[2] = u32x2{kr[1][0], kr[1][1]};
+            krow[3] = u32x2{kr[1][2], kr[1][3]};
+            uint32_t* vt = reinterpret_cast<uint32_t*>(sm + OFF_VT) + lane;
 #pragma unroll
-        for (int tb = 0; tb < 4; ++tb) {
-            *reinterpret_cast<u32x2*>(sm + OFF_KT + (16 * tb + j) * KT_ROW + 8 * kq) = kw[tb];
-            uint32_t* vt = reinterpret_cast<uint32_t*>(sm + OFF_VT);
-            vt[(2 * kq) * VT_COL + 16 * tb + j] = vw[tb][0];
-            vt[(2 * kq + 1) * VT_COL + 16 * tb + j] = vw[tb][1];
+            for (int c = 0; c < 8; ++c) vt[c * VT_COL] = vr[c >> 2][c & 3];
         }
         // V scales / zero points of this lane's token as f16, [group][token]
         {
