@@ -425,7 +425,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
                 const float qs = k_class(4 * (ks & 1) + rr) == 1 ? 32.0f : 8.0f;    // 2^(7-2k)
                 const float lo = qs * q_at(cl), hi = qs * q_at(cl + 8);
-                aq_pair[ks][rr] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
+                // bf16 pair (lo, hi): the upper halves of the two fp32 words (exact products)
+                aq_pair[ks][rr] = __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
                 aq_nat[ks][rr] = pack_f16x2(4.0f * q_at(8 * ks + 2 * rr), 4.0f * q_at(8 * ks + 2 * rr + 1));
             }
         }
@@ -817,7 +818,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             for (int r = 0; r < 4; ++r) {
                 if (r >= heads) break;
                 float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
-                const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+                const float inv = l_tot[r] > 0.0f ? __builtin_amdgcn_rcpf(l_tot[r]) : 0.0f;    // 1 ulp
 #pragma unroll
                 for (int y = 0; y < 8; ++y)
                     dst[ch0 + y] = (((y & 1) ? 4.0f : 16.0f) * (acc[y][r] - pvs[r]) + pvz[r]) * inv;
@@ -838,7 +839,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 float* dst = a.al + b * a.al_b + (int64_t)(qh0 + 4 * hg + r) * a.al_h + (int64_t)sp * a.al_s;
-                const float inv = l_tot[r] > 0.0f ? 1.0f / l_tot[r] : 0.0f;
+                const float inv = l_tot[r] > 0.0f ? __builtin_amdgcn_rcpf(l_tot[r]) : 0.0f;    // 1 ulp
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     const int ch0 = 16 * (4 * s + (j & 3)) + 4 * bsel;
