@@ -1,32 +1,36 @@
-// Split combine with the bf16 sink/recent tail folded in: one workgroup of 8*D threads per
-// (request, q head).  Follows ommx_gpu_serve/attention/paged_decode.py:2366-2500: valid
+// Split combine with the bf16 sink/recent tail folded in: four workgroups of 1024 threads per
+// (request, q head), one per quarter of the head's channels.  Follows ommx_gpu_serve/attention/paged_decode.py:2366-2500: valid
 // splits are recomputed from the packed length with the stage-1 rounding; the tail is one
 // more softmax part computed here from k_tail/v_tail; o = sum w_i o_i / sum w_i,
 // lse = max + ln sum w_i; nothing attended gives o = 0, lse = -inf.
 //
 // The kernel is latency bound (B*Hq small workgroups, a few KB each), so every global load
 // is issued before the first wait: thread (d, sg) owns channel d of the splits
-// sg, sg+8, ... and of the tail rows sg, sg+8, ...; for the tail logits the same threads
+// sg, sg+NSG, ... and of the tail rows sg, sg+NSG, ...; for the tail logits the same threads
 // regroup as (row, 16 parts of the row).
 #include "ommx_decode_args.h"
 
 namespace ommx {
 
 template <int D>
-__global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
-    constexpr int NT = 8 * D;
+__global__ void __launch_bounds__(1024) combine_kernel(CombineArgs a) {
+    constexpr int NT = 1024;
+    constexpr int CH = D / 4;            // channels of this workgroup (a quarter of the head)
+    constexpr int NSG = NT / CH;         // split groups: thread (d, sg) owns splits sg, sg + NSG, ...
     constexpr int MAXS = 256;            // split slots (the launcher refuses more)
-    constexpr int ROWS = NT / 16;        // tail rows handled per chunk (64 at D=128)
-    constexpr int PER = ROWS / 8;        // tail rows per thread in the P.V step
-    constexpr int NSP = MAXS / 8;        // split partials per thread, upper bound
+    constexpr int NSP = MAXS / NSG;      // split partials per thread, upper bound
+    constexpr int ROWS = NT / 16;        // tail rows handled per chunk (64)
+    constexpr int PER = ROWS / NSG;      // tail rows per thread in the P.V step
+    static_assert(PER >= 1 && NSP % 4 == 0, "thread layout");
     __shared__ float s_q[D];
     __shared__ __attribute__((aligned(16))) float s_logit[ROWS];
-    __shared__ float s_acc[8][D];        // per-sg sums of the split part
-    __shared__ float s_tacc[8][D];       // per-sg sums of the tail part
-    __shared__ float s_w[8], s_tl[8], s_wmax[MAXS / 64];
-    __shared__ __attribute__((aligned(16))) float s_wT[8][NSP];   // weight of split sg + 8*i at [sg][i]
-    const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int d = tid % D, sg = tid / D;
+    __shared__ float s_acc[NSG][CH];     // per-sg sums of the split part
+    __shared__ float s_tacc[NSG][CH];    // per-sg sums of the tail part
+    __shared__ float s_w[NSG], s_tl[NSG], s_wmax[MAXS / 64];
+    __shared__ __attribute__((aligned(16))) float s_wT[NSG][NSP];   // weight of split sg + NSG*i at [sg][i]
+    const int b = blockIdx.x, h = blockIdx.y, cq = blockIdx.z, tid = threadIdx.x;
+    const int dl = tid % CH, sg = tid / CH;
+    const int d = cq * CH + dl;          // this thread's channel of the head
     const int kvh = h / (a.Hq / a.Hkv);
     const float* base = a.al + b * a.al_b + (int64_t)h * a.al_h;
     // the two scalars that everything after the split loads waits for: requested first
@@ -35,25 +39,25 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
 
     // ---- all loads of the split part --------------------------------------------------
     // They depend on the arguments only, so they go out before anything is read from
-    // memory; one pointer per thread, advanced by 8 split slots per load.  (A uniform trip
+    // memory; one pointer per thread, advanced by NSG split slots per load.  (A uniform trip
     // count and a clamped last address keep the loads free of per-lane branches, so they
     // are all in flight together.)
     float pv[NSP];
-    const int n_i = (a.S + 7) >> 3;
+    const int n_i = (a.S + NSG - 1) / NSG;
     {
         const float* p = base + (int64_t)sg * a.al_s + d;
-        const int64_t step = 8 * a.al_s;
+        const int64_t step = NSG * a.al_s;
 #pragma unroll
         for (int i = 0; i < NSP; ++i) {
             pv[i] = 0.0f;
             if (i < n_i) {
-                const bool inside = sg + 8 * i < a.S;          // only the last trip can fall outside
+                const bool inside = sg + NSG * i < a.S;        // only the last trip can fall outside
                 pv[i] = *(inside ? p : base + (int64_t)(a.S - 1) * a.al_s + d);
                 p += step;
             }
         }
     }
-    const uint32_t q_raw = a.q ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + d] : 0u;
+    const uint32_t q_raw = (a.q && tid < D) ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + tid] : 0u;
     const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:2407
     float my_lse = -INFINITY;
     if (tid < MAXS) {
@@ -70,6 +74,8 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
     }
 
     // ---- tail: chunks of ROWS rows (one chunk in practice: sink + recent <= 72 rows) ----
+    // Every quarter computes all the logits (they need the whole q and K rows) and its own
+    // channels of P.V.
     float t_m = -INFINITY, t_l = 0.0f, t_acc = 0.0f;
     for (int r0 = 0; r0 < tail; r0 += ROWS) {
         const int nr = min(ROWS, tail - r0);
@@ -81,7 +87,7 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
         uint32_t vv[PER];
 #pragma unroll
         for (int i = 0; i < PER; ++i)
-            vv[i] = a.vt[b * a.vt_b + (int64_t)(r0 + min(sg + 8 * i, nr - 1)) * a.vt_t +
+            vv[i] = a.vt[b * a.vt_b + (int64_t)(r0 + min(sg + NSG * i, nr - 1)) * a.vt_t +
                          (int64_t)kvh * a.vt_h + d];
         __syncthreads();                              // s_q ready (and previous chunk consumed)
         float dot = 0.0f;
@@ -110,7 +116,7 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
         t_acc *= alpha;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int r = sg + 8 * i;
+            const int r = sg + NSG * i;
             if (r < nr) {
                 const float p = __expf(s_logit[r] - m_new);
                 t_l += p;
@@ -123,12 +129,12 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
 
     // ---- split part: weights from the lse column -----------------------------------------
     // One thread per split turns its lse into a weight; the weights are laid out so that
-    // thread (d, sg) reads the ones of its splits sg, sg+8, ... as float4.
+    // thread (d, sg) reads the ones of its splits sg, sg+NSG, ... as float4.
     float g_max = s_wmax[0];
 #pragma unroll
     for (int w = 1; w < MAXS / 64; ++w) g_max = fmaxf(g_max, s_wmax[w]);
     const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
-    if (tid < MAXS) s_wT[tid & 7][tid >> 3] = my_lse == -INFINITY ? 0.0f : __expf(my_lse - g_safe);
+    if (tid < MAXS) s_wT[tid % NSG][tid / NSG] = my_lse == -INFINITY ? 0.0f : __expf(my_lse - g_safe);
     __syncthreads();
     float acc = 0.0f, wsum = 0.0f;
 #pragma unroll
@@ -141,14 +147,14 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
             acc = w[k] > 0.0f ? fmaf(w[k], pv[4 * i4 + k], acc) : acc;
         }
     }
-    s_acc[sg][d] = acc;
-    s_tacc[sg][d] = t_acc;
-    if (d == 0) { s_w[sg] = wsum; s_tl[sg] = t_l; }
+    s_acc[sg][dl] = acc;
+    s_tacc[sg][dl] = t_acc;
+    if (dl == 0) { s_w[sg] = wsum; s_tl[sg] = t_l; }
     __syncthreads();
     if (sg == 0) {
         float A = 0.0f, W = 0.0f, TA = 0.0f, TL = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) { A += s_acc[k][d]; W += s_w[k]; TA += s_tacc[k][d]; TL += s_tl[k]; }
+        for (int k = 0; k < NSG; ++k) { A += s_acc[k][dl]; W += s_w[k]; TA += s_tacc[k][dl]; TL += s_tl[k]; }
         const float tail_lse = TL > 0.0f ? t_m + __logf(TL) : -INFINITY;
         const float n_max = fmaxf(g_max, tail_lse);
         const float n_safe = (n_max == -INFINITY) ? 0.0f : n_max;
@@ -167,9 +173,9 @@ __global__ void __launch_bounds__(8 * D) combine_kernel(CombineArgs a) {
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
-    const dim3 grid(a.B, a.Hq);
+    const dim3 grid(a.B, a.Hq, 4);
     if (D == 128) hipLaunchKernelGGL(combine_kernel<128>, grid, dim3(1024), 0, st, a);
-    else if (D == 64) hipLaunchKernelGGL(combine_kernel<64>, grid, dim3(512), 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL(combine_kernel<64>, grid, dim3(1024), 0, st, a);
     else return -1;
     return 0;
 }
