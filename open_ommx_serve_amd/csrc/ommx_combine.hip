@@ -12,10 +12,10 @@
 
 namespace ommx {
 
-template <int D>
+template <int D, int Q>
 __global__ void __launch_bounds__(1024) combine_kernel(CombineArgs a) {
     constexpr int NT = 1024;
-    constexpr int CH = D / 4;            // channels of this workgroup (a quarter of the head)
+    constexpr int CH = D / Q;            // channels of this workgroup (one of Q pieces of the head)
     constexpr int NSG = NT / CH;         // split groups: thread (d, sg) owns splits sg, sg + NSG, ...
     constexpr int MAXS = 256;            // split slots (the launcher refuses more)
     constexpr int NSP = MAXS / NSG;      // split partials per thread, upper bound
@@ -173,9 +173,10 @@ __global__ void __launch_bounds__(1024) combine_kernel(CombineArgs a) {
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
-    const dim3 grid(a.B, a.Hq, 4);
-    if (D == 128) hipLaunchKernelGGL(combine_kernel<128>, grid, dim3(1024), 0, st, a);
-    else if (D == 64) hipLaunchKernelGGL(combine_kernel<64>, grid, dim3(1024), 0, st, a);
+    constexpr int Q = 4;             // 2 and 8 pieces measured slower
+    const dim3 grid(a.B, a.Hq, Q);
+    if (D == 128) hipLaunchKernelGGL((combine_kernel<128, Q>), grid, dim3(1024), 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL((combine_kernel<64, 4>), dim3(a.B, a.Hq, 4), dim3(1024), 0, st, a);
     else return -1;
     return 0;
 }
