@@ -275,7 +275,10 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 // base scale and zero point (level * 2^e + zp), and there are no map planes.
 // PARTIAL (HR = 4 only): the kv head serves 1 or 2 q heads; the spare head slots repeat the
 // last head and are not written out.
-template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false>
+// GTS: K groups of 32 << GTS tokens (position streams only).  The kernel keeps working in
+// 32-token pieces: piece v of a longer group reads the group's parameters again and takes the
+// outliers whose position falls into it.  The V vectors may then be 32, 64 or 128 channels wide.
+template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -296,7 +299,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int qh0 = kvh * heads;          // first of this wave's q heads
     const int b = blockIdx.z, sp = blockIdx.x;
     const int L = a.seq[b];
-    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
+    constexpr int GT = 32 << GTS;
+    static_assert(GTS == 0 || IDX == 1, "longer groups are read through position streams");
+    const int per = ((((L + a.S - 1) / a.S) + GT - 1) / GT) * GT;
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
     const float c_log2e = 1.4426950408889634f;
@@ -322,13 +327,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int last = n_end - 1;
     const int ps_sh = __ffs(a.ps) - 1, ps_mask = a.ps - 1;     // page_size is a power of two
     const int tsh = a.i64 ? 3 : 2;                             // low dword of an int64 entry
-    const int tok_off = a.gbase * 32 + a.off;
+    const int tok_off = a.gbase * GT + a.off;
     const char* const rt_b = static_cast<const char*>(a.rt) + ((b * a.rt_s) << tsh);
     const char* const rg_b = static_cast<const char*>(a.rg) + ((b * a.rg_s + a.gbase) << tsh);
     const uint8_t* const kb_head = a.k_base + kvh * 32;      // a lane loads its own token's 32-byte rows
     const uint8_t* const vb_head = a.v_main + kvh * 32;
-    const int8_t* const vs_head = a.v_scale + kvh * 4;
-    const uint16_t* const vz_head = a.v_zp + kvh * 4;
+    // V vectors per token: 4 of 32 channels, or fewer of 64 / 128 (longer-group recipes only)
+    const int ngv = GTS == 0 ? 4 : D / a.gc;
+    const int8_t* const vs_head = a.v_scale + kvh * ngv;
+    const uint16_t* const vz_head = a.v_zp + kvh * ngv;
 
     // The loop is software-pipelined by hand: table entries are fetched two iterations
     // ahead, plane data one iteration ahead, each into the registers its previous use
@@ -342,7 +349,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         }
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            const int gi = min(n / 32 + g, last / 32);
+            const int gi = min((n + 32 * g) / GT, last / GT);
             gsl[g] = *reinterpret_cast<const int*>(rg_b + ((uint32_t)gi << tsh));
         }
     };
@@ -356,8 +363,20 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         vr[0] = *reinterpret_cast<const u32x4*>(vb_head + ro);
         vr[1] = *reinterpret_cast<const u32x4*>(vb_head + ro + 16);
         const uint32_t my_row = row1;
-        vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
-        vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
+        if (GTS == 0 || ngv == 4) {
+            vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
+            vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 4));
+        } else if (ngv == 2) {      // two 64-channel vectors: each serves two 32-channel quarters
+            const uint32_t e2 = *reinterpret_cast<const uint16_t*>(vs_head + (uint64_t)my_row * (uint32_t)(Hkv * 2));
+            const uint32_t z2 = *reinterpret_cast<const uint32_t*>(vz_head + (uint64_t)my_row * (uint32_t)(Hkv * 2));
+            vsc = __builtin_amdgcn_perm(0u, e2, 0x01010000u);
+            vzp = u32x2{(z2 & 0xFFFFu) * 0x10001u, (z2 >> 16) * 0x10001u};
+        } else {                    // one 128-channel vector
+            const uint32_t e1 = *reinterpret_cast<const uint8_t*>(vs_head + (uint64_t)my_row * (uint32_t)Hkv);
+            const uint32_t z1 = *(vz_head + (uint64_t)my_row * (uint32_t)Hkv);
+            vsc = e1 * 0x01010101u;
+            vzp = u32x2{z1 * 0x10001u, z1 * 0x10001u};
+        }
     };
     // channel pair (2*lane, 2*lane+1) parameters of both groups
     uint32_t g_sc[2], g_zp[2], g_ms[2] = {0, 0}, g_mc[2] = {0, 0};
@@ -551,6 +570,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                 // RES = false: the walk every group takes.  RES = true: a second walk that only
                 // adds f16 rounding residuals of large deltas onto the logits.
                 float dl_max[2] = {0.0f, 0.0f};
+                const int piece = ((n0 >> 5) + g) & ((1 << GTS) - 1);     // 32-token piece of the group
                 auto walk = [&](auto RES, auto U) {
                     constexpr int u = decltype(U)::value;
                     {
@@ -591,24 +611,33 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                             if constexpr (IDX == 0) {
                                 pos = __builtin_ctz(bm) & 31;           // v_ffbl_b32
                                 bm &= bm - 1;
-                            } else {                                    // bits [7s, 7s+5) of the stream
-                                pos = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
-                                    : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
-                                                : ((ix_hi >> 3) & 31);
+                            } else {                                    // bits [7s, 7s+7) of the stream
+                                constexpr int PM = GT - 1;              // (5 bits suffice for 32-token groups)
+                                pos = sidx < 4 ? ((ix_lo >> (7 * sidx)) & PM)
+                                    : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & PM)
+                                                : ((ix_hi >> 3) & PM);
+                            }
+                            // a longer group: only the outliers of this 32-token piece
+                            bool here = true;
+                            if constexpr (GTS > 0) {
+                                here = (pos >> 5) == piece;
+                                pos &= 31;
                             }
                             const float dl0 = fmaf(lv[sidx], a1, b1);
                             const bool top = dl0 > thr;
                             const float dl = top ? dl0 - s34 : dl0;
                             const _Float16 hi = static_cast<_Float16>(dl);
                             if constexpr (!decltype(RES)::value) {
-                                dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
-                                // K row dword = (dword & ~field) | (top ? field : 0)
-                                asm volatile("ds_mskor_b32 %0, %1, %2"
-                                             :: "v"(kt + pos * KT_ROW), "v"(field), "v"(top ? field : 0u)
-                                             : "memory");
-                                dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
+                                if (here) {
+                                    dt[pos * (DT_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
+                                    // K row dword = (dword & ~field) | (top ? field : 0)
+                                    asm volatile("ds_mskor_b32 %0, %1, %2"
+                                                 :: "v"(kt + pos * KT_ROW), "v"(field), "v"(top ? field : 0u)
+                                                 : "memory");
+                                    dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
+                                }
                             } else {
-                                if (fabsf(dl) >= big_thr[u]) {
+                                if (here && fabsf(dl) >= big_thr[u]) {
                                     const float lo = dl - static_cast<float>(hi);
 #pragma unroll
                                     for (int r = 0; r < HR; ++r)
@@ -864,7 +893,12 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
     if (a.scale_bf16) return 1;      // operands are exact only for power-of-two steps
-    if (a.gt != 32 || a.gc != 32 || a.v_bf16) return 1;
+    if (a.v_bf16) return 1;
+    // longer K groups (and wider V vectors with them): position streams, 6 outliers, 4 or 8 heads
+    const bool longer = a.gt == 64 || a.gt == 128;
+    if (longer && !(a.idx_repr == 1 && a.kout == 6 && (R == 4 || R == 8) &&
+                    (a.gc == 32 || a.gc == 64 || a.gc == 128))) return 1;
+    if (!longer && (a.gt != 32 || a.gc != 32)) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);    // one wave per kv head
@@ -876,7 +910,20 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a)
 #define OMMX_LAUNCH_PARTIAL(IDX, MAP) \
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, IDX, MAP, true>), grid, block, shm, st, a)
-    if (a.kout == 6 && R < 4) {
+#define OMMX_LAUNCH_LONG(HR, MAP, GTS) \
+    hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, 1, MAP, false, GTS>), grid, block, shm, st, a)
+    if (longer) {
+        switch ((R == 8 ? 4 : 0) | (a.gt == 128 ? 2 : 0) | (own_map ? 1 : 0)) {
+            case 0: OMMX_LAUNCH_LONG(4, false, 1); break;
+            case 1: OMMX_LAUNCH_LONG(4, true, 1); break;
+            case 2: OMMX_LAUNCH_LONG(4, false, 2); break;
+            case 3: OMMX_LAUNCH_LONG(4, true, 2); break;
+            case 4: OMMX_LAUNCH_LONG(8, false, 1); break;
+            case 5: OMMX_LAUNCH_LONG(8, true, 1); break;
+            case 6: OMMX_LAUNCH_LONG(8, false, 2); break;
+            default: OMMX_LAUNCH_LONG(8, true, 2); break;
+        }
+    } else if (a.kout == 6 && R < 4) {
         switch ((a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
             case 0: OMMX_LAUNCH_PARTIAL(0, false); break;
             case 1: OMMX_LAUNCH_PARTIAL(0, true); break;
@@ -904,6 +951,7 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     }
 #undef OMMX_LAUNCH
 #undef OMMX_LAUNCH_PARTIAL
+#undef OMMX_LAUNCH_LONG
     return 0;
 }
 
