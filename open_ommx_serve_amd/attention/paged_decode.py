@@ -31,7 +31,7 @@ def _cu_count(device: torch.device) -> int:
 
 
 def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256,
-                       q_per_kv: int = 4) -> int:
+                       q_per_kv: int = 4, group_tokens: int = 32) -> int:
     """Split count that gives every compute unit four workgroups, two resident and two queued
     behind them so that requests of different length even out (a workgroup is four waves of
     one split; a wave covers one kv head and all of its q heads, so ``q_per_kv`` does not
@@ -41,12 +41,14 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
     and the steps are dealt out evenly (the split length
     is rounded up to whole groups by the kernel, so a careless count leaves splits empty and
     others a step longer).  At most 256, the number of partial states the combine kernel keeps
-    on chip."""
+    on chip.  Splits are whole K groups (``group_tokens``), so longer groups mean coarser steps."""
     wgs_per_split = max(1, int(batch) * max(1, int(kv_heads) // 4))
     want = max(1, min(256, (4 * int(n_cu)) // wgs_per_split))
-    steps = max(1, (int(max_seq_len) + 63) // 64)
-    if want >= 2 * steps:          # plenty of idle units: splits of one 32-token group
-        return int(min(want, max(1, (int(max_seq_len) + 31) // 32)))
+    gt = max(32, int(group_tokens))
+    step_tokens = max(64, gt)
+    steps = max(1, (int(max_seq_len) + step_tokens - 1) // step_tokens)
+    if want >= 2 * steps:          # plenty of idle units: splits of one K group
+        return int(min(want, max(1, (int(max_seq_len) + gt - 1) // gt)))
     target = max(1, min(want, steps))
     # equal whole steps per split, no empty split: the slowest wave sets the kernel's time
     steps_per_split = (steps + target - 1) // target
@@ -200,7 +202,7 @@ def ommx_paged_decode_attention_canonical(
     else:
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
     if num_kv_splits is None:
-        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv)
+        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv, group_tokens)
     S = max(1, int(num_kv_splits))
     if attn_logits is None:
         attn_logits = make_attn_logits(B, Hq, S, D, q.device)

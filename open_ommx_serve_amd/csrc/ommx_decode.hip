@@ -278,7 +278,8 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 // GTS: K groups of 32 << GTS tokens (position streams only).  The kernel keeps working in
 // 32-token pieces: piece v of a longer group reads the group's parameters again and takes the
 // outliers whose position falls into it.  The V vectors may then be 32, 64 or 128 channels wide.
-template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0>
+// KO: outliers per K vector, 6, or 10 (position streams, 128-token groups: the 2.75-bit recipe).
+template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0, int KO = 6>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -301,6 +302,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int L = a.seq[b];
     constexpr int GT = 32 << GTS;
     static_assert(GTS == 0 || IDX == 1, "longer groups are read through position streams");
+    static_assert(KO == 6 || (KO == 10 && IDX == 1), "10 outliers: position streams only");
     const int per = ((((L + a.S - 1) / a.S) + GT - 1) / GT) * GT;
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
@@ -383,6 +385,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     constexpr bool own_map = OWN_MAP;
     u32x2 g_bm[2], g_ov[2];
     uint32_t g_bx[2];                     // third index dword (position streams only)
+    // 10 outliers: 18 index bytes and 10 nibble bytes per lane start at a multiple of 2; the
+    // aligned dwords that cover them are loaded and shifted into place when they are used
+    uint32_t g_ix10[2][5], g_ov10[2][3];
     // (the group index is wave-uniform: base addresses are formed on the scalar unit, the lane
     // adds a 32-bit byte offset)
     const uint32_t kvh_s = __builtin_amdgcn_readfirstlane(kvh);
@@ -401,15 +406,24 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                     g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
                     g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
                 }
-                if constexpr (IDX == 0) {
+                if constexpr (KO == 10) {
+                    const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp + gidx * 9, (18 * lane_b) & ~3u));
+#pragma unroll
+                    for (int i = 0; i < 5; ++i) g_ix10[g][i] = ixp[i];
+                    const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 5, (10 * lane_b) & ~3u));
+#pragma unroll
+                    for (int i = 0; i < 3; ++i) g_ov10[g][i] = ovp[i];
+                } else if constexpr (IDX == 0) {
                     g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
                 } else {          // 12 bytes: the streams of both channels
                     const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp + gidx * 6, 12 * lane_b));
                     g_bm[g] = u32x2{ixp[0], ixp[1]};
                     g_bx[g] = ixp[2];
                 }
-                const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
-                g_ov[g] = u32x2{ovp[0], ovp[1]};
+                if constexpr (KO == 6) {
+                    const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
+                    g_ov[g] = u32x2{ovp[0], ovp[1]};
+                }
             }
         }
     };
@@ -583,20 +597,50 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
                         const float a1 = own_map ? 0.25f * __builtin_amdgcn_rcpf(ms) : 0.25f * s;
                         const float b1 = own_map ? 0.25f * (mc - zp) : 0.0f;
-                        uint32_t bm = g_bm[g][u];
+                        uint32_t bm = 0;
+                        if constexpr (IDX == 0) bm = g_bm[g][u];
                         // position stream of this channel: 42 bits from bit 0 (u = 0) or bit 48
                         uint32_t ix_lo = 0, ix_hi = 0;
-                        if constexpr (IDX == 1) {
+                        if constexpr (IDX == 1 && KO == 6) {
                             ix_lo = u ? __builtin_amdgcn_alignbit(g_bx[g], g_bm[g][1], 16) : g_bm[g][0];
                             ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
                         }
-                        // 6 nibbles of this channel: bytes 3c..3c+2 of the block
-                        const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
-                        const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
-                        const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
-                        const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
-                        const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
-                        const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
+                        float lv[KO];
+                        uint32_t ixw[5] = {0, 0, 0, 0, 0};       // 10 outliers: index window, channel 0 at bit 0
+                        if constexpr (KO == 6) {
+                            // 6 nibbles of this channel: bytes 3c..3c+2 of the block
+                            const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
+                            const uint32_t nib = static_cast<uint32_t>(ov64 >> (8 * ((6 * lane) & 3) + 24 * u)) & 0xFFFFFFu;
+                            const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                            const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
+                            const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
+                            lv[0] = l01[0]; lv[1] = l01[1]; lv[2] = l23[0]; lv[3] = l23[1]; lv[4] = l45[0]; lv[5] = l45[1];
+                        } else {
+                            // the lane's bytes start 0 or 2 bytes into the loaded dwords (odd lanes)
+                            const uint32_t sh = (lane & 1) ? 16u : 0u;
+                            const uint32_t o0 = __builtin_amdgcn_alignbit(g_ov10[g][1], g_ov10[g][0], sh);
+                            const uint32_t o1 = __builtin_amdgcn_alignbit(g_ov10[g][2], g_ov10[g][1], sh);
+                            const uint32_t o2 = g_ov10[g][2] >> sh;
+                            // channel u: nibbles 10u .. 10u+9 = bytes 5u .. 5u+4 of (o0, o1, o2)
+#pragma unroll
+                            for (int i = 0; i < 5; ++i) {
+                                const int byte = 5 * u + i;
+                                const uint32_t w = byte < 4 ? o0 : (byte < 8 ? o1 : o2);
+                                f32x2 l2;
+                                switch (byte & 3) {
+                                    case 0: l2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); break;
+                                    case 1: l2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); break;
+                                    case 2: l2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); break;
+                                    default: l2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); break;
+                                }
+                                lv[2 * i] = l2[0];
+                                lv[2 * i + 1] = l2[1];
+                            }
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                ixw[i] = __builtin_amdgcn_alignbit(g_ix10[g][i + 1], g_ix10[g][i], sh);
+                            ixw[4] = g_ix10[g][4] >> sh;
+                        }
                         // The 2-bit base code of an outlier position is overwritten (in the staged
                         // K row) by 0 or 3, whichever base value is nearer to the outlier, so the
                         // delta left for the tile is small; the bias terms account for the rest.
@@ -606,9 +650,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
                         uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_DT) + c;
                         float* lc = reinterpret_cast<float*>(sm + OFF_LC) + g * 32 * HR;
 #pragma unroll
-                        for (int sidx = 0; sidx < 6; ++sidx) {
+                        for (int sidx = 0; sidx < KO; ++sidx) {
                             int pos;
-                            if constexpr (IDX == 0) {
+                            if constexpr (KO == 10) {          // 7-bit field at bit 72u + 7s of the window
+                                constexpr int PM = GT - 1;
+                                const int bit = 72 * u + 7 * sidx;
+                                const int wi = bit >> 5, bo = bit & 31;
+                                pos = (bo <= 25 ? (ixw[wi] >> bo)
+                                                : __builtin_amdgcn_alignbit(ixw[wi < 4 ? wi + 1 : 4], ixw[wi], bo)) & PM;
+                            } else if constexpr (IDX == 0) {
                                 pos = __builtin_ctz(bm) & 31;           // v_ffbl_b32
                                 bm &= bm - 1;
                             } else {                                    // bits [7s, 7s+7) of the stream
@@ -891,20 +941,22 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
 
 // Returns 0 when launched, 1 when the shape is not covered by the tuned kernel.
 int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
-    if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8) || !(a.kout == 6 || a.kout == 0)) return 1;
+    if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8)) return 1;
+    const bool paper = a.kout == 10 && a.gt == 128 && a.idx_repr == 1 && (R == 4 || R == 8);   // 128-token groups, 10 outliers
+    if (!(a.kout == 6 || a.kout == 0 || paper)) return 1;
     if (a.scale_bf16) return 1;      // operands are exact only for power-of-two steps
     if (a.v_bf16) return 1;
     // longer K groups (and wider V vectors with them): position streams, 6 outliers, 4 or 8 heads
     const bool longer = a.gt == 64 || a.gt == 128;
-    if (longer && !(a.idx_repr == 1 && a.kout == 6 && (R == 4 || R == 8) &&
+    if (longer && !(a.idx_repr == 1 && (a.kout == 6 || paper) && (R == 4 || R == 8) &&
                     (a.gc == 32 || a.gc == 64 || a.gc == 128))) return 1;
     if (!longer && (a.gt != 32 || a.gc != 32)) return 1;
     // the kernel reads q two channels at a time
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);    // one wave per kv head
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * (R <= 4 ? (a.kout == 6 ? LdsMap<4>::END : LdsMap<4>::DT)
-                                               : (a.kout == 6 ? LdsMap<8>::END : LdsMap<8>::DT));
+    const size_t shm = (size_t)waves * (R <= 4 ? (a.kout > 0 ? LdsMap<4>::END : LdsMap<4>::DT)
+                                               : (a.kout > 0 ? LdsMap<8>::END : LdsMap<8>::DT));
     const bool own_map = a.k_ms != nullptr;
 #define OMMX_LAUNCH(HR, IDX, MAP) \
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a)
@@ -912,7 +964,16 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, IDX, MAP, true>), grid, block, shm, st, a)
 #define OMMX_LAUNCH_LONG(HR, MAP, GTS) \
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, 1, MAP, false, GTS>), grid, block, shm, st, a)
-    if (longer) {
+#define OMMX_LAUNCH_PAPER(HR, MAP) \
+    hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, 1, MAP, false, 2, 10>), grid, block, shm, st, a)
+    if (paper) {
+        switch ((R == 8 ? 2 : 0) | (own_map ? 1 : 0)) {
+            case 0: OMMX_LAUNCH_PAPER(4, false); break;
+            case 1: OMMX_LAUNCH_PAPER(4, true); break;
+            case 2: OMMX_LAUNCH_PAPER(8, false); break;
+            default: OMMX_LAUNCH_PAPER(8, true); break;
+        }
+    } else if (longer) {
         switch ((R == 8 ? 4 : 0) | (a.gt == 128 ? 2 : 0) | (own_map ? 1 : 0)) {
             case 0: OMMX_LAUNCH_LONG(4, false, 1); break;
             case 1: OMMX_LAUNCH_LONG(4, true, 1); break;
@@ -952,6 +1013,7 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
 #undef OMMX_LAUNCH
 #undef OMMX_LAUNCH_PARTIAL
 #undef OMMX_LAUNCH_LONG
+#undef OMMX_LAUNCH_PAPER
     return 0;
 }
 

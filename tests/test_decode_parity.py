@@ -248,20 +248,22 @@ def test_bf16_v_rows(kw):
         _check(_run(case, num_kv_splits=S), want, f"bf16 V {kw} S{S}")
 
 
-@pytest.mark.parametrize("gt,gc", [(64, 64), (64, 32), (128, 128), (128, 64), (64, 128)])
-@pytest.mark.parametrize("hq,own_map", [(32, False), (64, True), (32, True)])
-def test_longer_groups_on_the_matrix_core_kernel(gt, gc, hq, own_map):
-    """K groups of 64 / 128 tokens with position streams and 6 outliers run on the matrix-core
-    kernel (32-token pieces of a group): against the oracle and against the plain kernel, ragged
+@pytest.mark.parametrize("gt,gc,k", [(64, 64, 6), (64, 32, 6), (128, 128, 6), (128, 64, 6), (64, 128, 6),
+                                     (128, 128, 10), (128, 32, 10)])
+@pytest.mark.parametrize("hq,own_map", [(32, False), (64, True), (32, True), (64, False)])
+def test_longer_groups_on_the_matrix_core_kernel(gt, gc, k, hq, own_map):
+    """K groups of 64 / 128 tokens with position streams and 6 outliers (10 with 128-token
+    groups: the reference's 2.75-bit "paper-kv" recipe) run on the matrix-core kernel as
+    32-token pieces of a group: against the oracle and against the plain kernel, ragged
     lengths, permuted tables, several split counts."""
     case = build_decode_case([2900, 700, 150], q_heads=hq, kv_heads=8, seed=81, permute_tables=True,
-                             sparse_frac=0.005, group_tokens=gt, group_channels=gc,
+                             sparse_frac=0.005, group_tokens=gt, group_channels=gc, outliers_per_vector=k,
                              outlier_repr="relidx7", kv_outlier_map=own_map)
     want = _oracle(case)
     ref = _run(case, ref_kernel=True)
     for S in (None, 1, 5):
         got = _run(case, num_kv_splits=S)
-        _check(got, want, f"gt{gt} gc{gc} S{S}")
+        _check(got, want, f"gt{gt} gc{gc} k{k} S{S}")
         assert (got[0] - ref[0]).abs().max().item() <= MAX_ABS
 
 
