@@ -129,9 +129,11 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *   group_tokens / group_channels   tokens per K group and channels per V vector: 16, 32, 64, 128
  *   scale_bf16 = 1   k_scale / v_scale hold the steps themselves as bf16, not int8 exponents
  *   v_bf16 = 1       v_main is bf16 [P,ps,H,D]; v_scale / v_zp are ignored
- * The matrix-core kernel runs head_dim 128, 32-token groups, 32-channel V vectors, INT2 V, int8
- * exponents and 6 (or 0) outliers, with either index plane and either outlier map; every other
- * supported shape or recipe (k_outliers up to 16) runs on the plain fp32 kernel.
+ * The matrix-core kernel runs head_dim 128, INT2 V, int8 exponents, either outlier map, and
+ *   32-token groups with 32-channel V vectors and 6 (or 0) outliers, either index plane;
+ *   64- or 128-token groups with 32/64/128-channel V vectors and 6 outliers, relidx7 plane;
+ *   128-token groups with 10 outliers, relidx7 plane (4 or 8 q heads per kv head).
+ * Every other supported shape or recipe (k_outliers up to 16) runs on the plain fp32 kernel.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
