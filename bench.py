@@ -217,7 +217,7 @@ def main() -> int:
     cpu = None
     parity = None
     if not args.no_cpu_baseline:
-        runs = 5 if args.ctx >= 32768 else 20
+        runs = 15 if args.ctx >= 32768 else 40          # about ten seconds of CPU work
         times, (wo, wl) = _cpu_reference(case, runs)
         err = (m["o"].cpu().double() - wo.double()).abs()
         parity = {"max_abs": float(err.max()), "mean_abs": float(err.mean())}
