@@ -1,5 +1,7 @@
 // Tuned split-KV decode kernel for gfx950: head_dim 128, 1, 2, 4 or 8 q heads per kv head, 6 (or
-// 0) outliers per K vector.  Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
+// 0) outliers per K vector of 32 tokens; with the position-stream index plane also K vectors of
+// 64 / 128 tokens (6 outliers, or 10 with 128 tokens) and V vectors of 64 / 128 channels.
+// Same operator as ommx_gpu_serve/attention/paged_decode.py:1255-2284.
 //
 // Work decomposition.  A wavefront owns one kv head (and all 4 or 8 of its q heads) of one
 // split and walks it 64 tokens (two 32-token K groups) at a time; waves never synchronise with
