@@ -352,14 +352,19 @@ def test_logit_cap_and_caller_workspace():
     assert (o[0].double() - want).abs().max().item() <= MAX_ABS
 
 
-def test_segment_partial_emit_composes_to_the_full_result():
-    """Two group-range segments plus the tail, merged with the textbook state merge."""
-    case = build_decode_case([4096], q_heads=8, kv_heads=2, seed=15)
+@pytest.mark.parametrize("gt,kw", [(32, {}), (64, dict(group_tokens=64, group_channels=64, outlier_repr="relidx7")),
+                                   (128, dict(group_tokens=128, group_channels=128, outlier_repr="relidx7",
+                                              outliers_per_vector=10)),
+                                   (16, dict(group_tokens=16, group_channels=16, outliers_per_vector=3))])
+def test_segment_partial_emit_composes_to_the_full_result(gt, kw):
+    """Two group-range segments plus the tail, merged with the textbook state merge; the segment
+    base counts K groups of the recipe's size."""
+    case = build_decode_case([4096], q_heads=8, kv_heads=2, seed=15, **kw)
     want = _oracle(case)
     L = case.b_seq_len.tolist()[0]
-    g_split = (L // 32) // 3
+    g_split = (L // gt) // 3
     parts = []
-    for gb, n in ((0, g_split * 32), (g_split, L - g_split * 32)):
+    for gb, n in ((0, g_split * gt), (g_split, L - g_split * gt)):
         case.b_seq_len.fill_(n)
         o, lse = _run(case, num_kv_splits=4, seg_group_base=gb,
                       max_tail_len=0 if gb > 0 else None)
