@@ -3,7 +3,7 @@ operator (split-KV kernel + combine kernel) on one MI355X, Llama-3.1-8B attentio
 (32 q heads, 8 kv heads, d=128), batch 1, synthetic caches, context 1K..64K.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--ctx 65536] [--no-ladder]
-                    [--no-cpu-baseline]
+                    [--no-cpu-baseline] [--batch B] [--q-heads H]
 
 One step = one decode call over one batch: the split-KV launch followed by the combine
 launch, operands resident in HBM, workspace preallocated.  Steps are replayed from HIP
@@ -140,6 +140,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--ctx", type=int, default=65536)
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--batch", type=int, default=1,
+                    help="requests per step (other workloads than the headline one, e.g. "
+                         "--batch 8 --ctx 32768 --q-heads 64 for the 8-request GQA-8 configuration)")
+    ap.add_argument("--q-heads", type=int, default=32)
     ap.add_argument("--no-ladder", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -163,7 +167,8 @@ def main() -> int:
     torch.cuda.set_device(0)
 
     def measure(ctx, steps, warmup):
-        case = build_decode_case([ctx], seed=42, permute_tables=True, sparse_frac=0.005)
+        case = build_decode_case([ctx] * args.batch, q_heads=args.q_heads, seed=42, permute_tables=True,
+                                 sparse_frac=0.005)
         step, stage1, o, lse, S = _make_runner(case, args.splits or None)
         # one model forward runs this operator once per layer inside a single graph, so the
         # steps are timed in graphs of LAYERS consecutive steps (steps is rounded up to that)
@@ -190,6 +195,9 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
+    headline = args.batch == 1 and args.q_heads == 32
+    if not headline:                   # another workload: no ladder, no CPU run (it scales with the batch)
+        args.no_ladder = args.no_cpu_baseline = True
     ladder = {}
     if not args.no_ladder:
         for ctx in (1024, 4096, 16384, 32768):
@@ -208,7 +216,7 @@ def main() -> int:
     p50 = statistics.median(m["us"])
     step_bytes = case.algorithmic_bytes()
     L = case.packed_lens[0]
-    packed_bytes = L * case.kv_heads * 132
+    packed_bytes = sum(case.packed_lens) * case.kv_heads * 132
     k1 = statistics.mean(m["us1"])
     achieved = packed_bytes / (k1 * 1e-6) / 1e9
     ladder[str(args.ctx)] = {"p50_us": round(p50, 2), "splits": m["S"], "bytes": step_bytes,
@@ -230,14 +238,15 @@ def main() -> int:
                          f"fp32 attention per q head) on {os.cpu_count()} logical CPUs"}
 
     out = {
-        "metric": "p50 decode-attn us/step/layer, 8B shape bs1",
+        "metric": "p50 decode-attn us/step/layer, 8B shape bs1" if headline
+                  else "p50 decode-attn us/step/layer",
         "value": round(p50, 3), "unit": "us/step/layer", "n_gpus": 1,
         "steps": -(-args.steps // LAYERS) * LAYERS, "warmup": -(-args.warmup // LAYERS) * LAYERS,
         "ms_per_step": round(m["wall_ms"], 6), "higher_is_better": False, "scaling": "weak",
-        "vs_baseline": round(p50 / H200_P50_US_64K, 5) if args.ctx == 65536 else None,
+        "vs_baseline": round(p50 / H200_P50_US_64K, 5) if (args.ctx == 65536 and headline) else None,
         "dtype": "u8 planes, bf16 q, f32 accumulate", "data": "synthetic",
-        "config": {"workload": f"OMMX paged decode attention, 32 q / 8 kv heads, d=128, batch 1, "
-                               f"ctx {args.ctx} ({L} packed tokens + {int(case.b_tail_len[0])} bf16 "
+        "config": {"workload": f"OMMX paged decode attention, {args.q_heads} q / 8 kv heads, d=128, "
+                               f"batch {args.batch}, ctx {args.ctx} ({L} packed tokens + {int(case.b_tail_len[0])} bf16 "
                                f"tail rows), page 16, permuted page/group tables, K outliers 4 "
                                f"channels x12 + 0.5% x8",
                    "num_kv_splits": m["S"], "launch": m["mode"],
@@ -247,7 +256,7 @@ def main() -> int:
                    "(reference Triton kernel on H200 NVL, page 32; other hardware)"},
         "roofline": {"bound": "hbm", "kernel": "decode_splitkv", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES_CTX64K if (args.ctx == 65536 and not args.splits) else None,
+                     "traffic": TRAFFIC_BYTES_CTX64K if (args.ctx == 65536 and not args.splits and headline) else None,
                      "bytes_per_launch": packed_bytes,
                      "avg_kernel_us": round(k1, 3)},
         "cpu_baseline": cpu,

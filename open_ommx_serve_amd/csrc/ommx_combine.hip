@@ -12,12 +12,13 @@
 
 namespace ommx {
 
-template <int D, int Q>
-__global__ void __launch_bounds__(1024) combine_kernel(CombineArgs a) {
-    constexpr int NT = 1024;
+// NT threads per workgroup, at most MAXS splits: 1024 / 256 in general, 512 / 64 when many
+// (request, head) pairs with few splits each fill the chip (fewer idle lanes per workgroup).
+template <int D, int Q, int NT = 1024, int MAXS = 256>
+__global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
     constexpr int CH = D / Q;            // channels of this workgroup (one of Q pieces of the head)
     constexpr int NSG = NT / CH;         // split groups: thread (d, sg) owns splits sg, sg + NSG, ...
-    constexpr int MAXS = 256;            // split slots (the launcher refuses more)
+    static_assert(MAXS <= NT && MAXS % 64 == 0, "one thread per split slot");
     constexpr int NSP = MAXS / NSG;      // split partials per thread, upper bound
     constexpr int ROWS = NT / 16;        // tail rows handled per chunk (64)
     constexpr int PER = ROWS / NSG;      // tail rows per thread in the P.V step
@@ -173,11 +174,18 @@ __global__ void __launch_bounds__(1024) combine_kernel(CombineArgs a) {
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
-    constexpr int Q = 2;             // pieces per head: 2 and 4 measured alike (36.7 us per step at 64K
-                                     // against 38.1 with one and 37.2 with eight); fewer repeat less
-    const dim3 grid(a.B, a.Hq, Q);
-    if (D == 128) hipLaunchKernelGGL((combine_kernel<128, Q>), grid, dim3(1024), 0, st, a);
-    else if (D == 64) hipLaunchKernelGGL((combine_kernel<64, Q>), grid, dim3(1024), 0, st, a);
+    // Pieces per head.  At batch 1 the kernel is latency bound and 2 pieces measured best (36.7 us
+    // per step at 64K against 38.1 with one, 36.7 with four, 37.2 with eight); with many
+    // (request, head) pairs the grid fills the chip by itself and one piece repeats no work.
+    const bool split2 = a.B * a.Hq < 256;
+    const dim3 grid(a.B, a.Hq, split2 ? 2 : 1);
+    const bool small = !split2 && a.S <= 64;
+    if (D == 128 && split2) hipLaunchKernelGGL((combine_kernel<128, 2>), grid, dim3(1024), 0, st, a);
+    else if (D == 128 && small) hipLaunchKernelGGL((combine_kernel<128, 1, 512, 64>), grid, dim3(512), 0, st, a);
+    else if (D == 128) hipLaunchKernelGGL((combine_kernel<128, 1>), grid, dim3(1024), 0, st, a);
+    else if (D == 64 && split2) hipLaunchKernelGGL((combine_kernel<64, 2>), grid, dim3(1024), 0, st, a);
+    else if (D == 64 && small) hipLaunchKernelGGL((combine_kernel<64, 1, 512, 64>), grid, dim3(512), 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL((combine_kernel<64, 1>), grid, dim3(1024), 0, st, a);
     else return -1;
     return 0;
 }
