@@ -300,8 +300,23 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     const int kvh = blockIdx.y * waves + wave;
     const int heads = PARTIAL ? a.Hq / Hkv : HR;      // q heads this kv head really serves
     const int qh0 = kvh * heads;          // first of this wave's q heads
-    const int b = blockIdx.z, sp = blockIdx.x;
-    const int L = a.seq[b];
+    const int sp = blockIdx.x;
+    // Requests are served longest first: workgroups are dispatched in grid order, so the ones that
+    // start last, when most compute units have run dry, belong to the shortest requests.
+    // blockIdx.z is the rank of the request by (length descending, index ascending); every wave
+    // finds its request from the lengths (one per lane, up to 64 requests).
+    int b = blockIdx.z, L;
+    if (a.B > 1 && a.B <= 64) {
+        const int my_len = lane < a.B ? a.seq[lane] : 0;
+        const uint32_t key = (static_cast<uint32_t>(my_len) << 6) | (63u - lane);   // distinct per lane
+        int rank = 0;
+        for (int i = 0; i < a.B; ++i)
+            rank += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key), i)) > key;
+        b = __builtin_ctzll(__ballot(lane < a.B && rank == static_cast<int>(blockIdx.z)));
+        L = __builtin_amdgcn_readlane(my_len, b);
+    } else {
+        L = a.seq[b];
+    }
     constexpr int GT = 32 << GTS;
     static_assert(GTS == 0 || IDX == 1, "longer groups are read through position streams");
     static_assert(KO == 6 || (KO == 10 && IDX == 1), "10 outliers: position streams only");

@@ -137,6 +137,23 @@ def test_ragged_batch_32_requests():
     _check(_run(case), _oracle(case), "B32")
 
 
+@pytest.mark.parametrize("batch", [2, 64, 65, 70])
+def test_longest_first_request_order(batch):
+    """The matrix-core kernel serves up to 64 requests longest first (more keep the grid order):
+    equal lengths, zero lengths and both sides of the 64-request limit give every request its
+    own result."""
+    g = torch.Generator().manual_seed(batch)
+    lens = torch.randint(40, 700, (batch,), generator=g).tolist()
+    lens[0] = lens[-1] = 500                      # ties
+    lens[batch // 2] = 9                          # nothing packed
+    if batch > 2:
+        lens[1] = lens[2] = lens[3] = 168
+    case = build_decode_case(lens, seed=batch, permute_tables=True, sparse_frac=0.005)
+    want = _oracle(case)
+    for S in (None, 3):
+        _check(_run(case, num_kv_splits=S), want, f"B{batch} S{S}")
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_gqa8_64_q_heads(ref_kernel):
     case = build_decode_case([2048, 3000], q_heads=64, kv_heads=8, seed=8, sparse_frac=0.005)
