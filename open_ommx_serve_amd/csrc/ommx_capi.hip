@@ -19,104 +19,93 @@ extern "C" int ommx_abi_version(void) { return OMMX_ABI_VERSION; }
 
 extern "C" const char* ommx_last_error(void) { return ommx::g_error.c_str(); }
 
-extern "C" int ommx_decode_splitkv(
-    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
-    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
-    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
-    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
-    int table_i64, const int32_t* b_seq_len,
-    float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int v_bf16, int num_splits,
-    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
-    void* stream) {
-    using namespace ommx;
-    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) {
-        set_error("ommx_decode_splitkv: q heads must be a positive multiple of kv heads");
-        return -1;
-    }
+// The two split-KV entry points take the same arguments and refuse the same ones.
+#define OMMX_DECODE_PARAMS                                                                          \
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,                                      \
+    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,                               \
+    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,      \
+    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,                               \
+    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,       \
+    int table_i64, const int32_t* b_seq_len,                                                        \
+    float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,              \
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,   \
+    int group_tokens, int group_channels, int v_bf16, int num_splits,                               \
+    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base, void* stream
+#define OMMX_DECODE_ARGS                                                                            \
+    q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval, v_main, v_scale, \
+    v_zp, req_to_token, rt_stride, req_to_group, rg_stride, table_i64, b_seq_len, attn_logits,      \
+    al_stride_b, al_stride_h, al_stride_s, B, Hq, Hkv, D, page_size, k_outliers, index_repr,        \
+    scale_bf16, group_tokens, group_channels, v_bf16, num_splits, sm_scale, logit_cap,              \
+    packed_start_offset, seg_group_base, stream
+
+namespace ommx {
+
+static bool is_group_size(int g) { return g == 16 || g == 32 || g == 64 || g == 128; }
+
+// Argument checks of the split-KV entry points: nullptr when the call may go ahead, else what
+// is wrong with it.  Everything a kernel assumes about shapes and alignment is checked here, on
+// the host, before anything is launched.
+static const char* check_decode(OMMX_DECODE_PARAMS) {
+    (void)q_stride_b; (void)q_stride_h; (void)rt_stride; (void)rg_stride; (void)table_i64;
+    (void)al_stride_b; (void)al_stride_h; (void)al_stride_s; (void)scale_bf16; (void)v_bf16;
+    (void)k_scale; (void)v_scale;
+    (void)sm_scale; (void)logit_cap; (void)stream;
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv)
+        return "q heads must be a positive multiple of kv heads";
     const int R = Hq / Hkv;
-    if (!(R == 1 || R == 2 || R == 4 || R == 8) || !(D == 64 || D == 128)) {
-        set_error("ommx_decode_splitkv: supported shapes are head_dim 64|128 and 1|2|4|8 q heads per kv head");
-        return -1;
-    }
-    if (!(group_tokens == 16 || group_tokens == 32 || group_tokens == 64 || group_tokens == 128) ||
-        !(group_channels == 16 || group_channels == 32 || group_channels == 64 || group_channels == 128) ||
-        D % group_channels) {
-        set_error("ommx_decode_splitkv: group_tokens / group_channels must be 16, 32, 64 or 128");
-        return -1;
-    }
-    if (page_size <= 0 || group_tokens % page_size) {
-        set_error("ommx_decode_splitkv: page_size must divide the K group");
-        return -1;
-    }
-    if (packed_start_offset < 0 || packed_start_offset >= page_size || seg_group_base < 0) {
-        set_error("ommx_decode_splitkv: packed_start_offset must be in [0,page_size), seg_group_base >= 0");
-        return -1;
-    }
-    if (k_outliers < 0 || k_outliers > 16 || k_outliers > group_tokens || num_splits < 1 || num_splits > 256 ||
-        (index_repr != 0 && index_repr != 1)) {
-        set_error("ommx_decode_splitkv: k_outliers in [0,min(16,group_tokens)], num_splits in [1,256], index_repr 0|1");
-        return -1;
-    }
+    if (!(R == 1 || R == 2 || R == 4 || R == 8) || !(D == 64 || D == 128))
+        return "supported shapes are head_dim 64|128 and 1|2|4|8 q heads per kv head";
+    if (!is_group_size(group_tokens) || !is_group_size(group_channels) || D % group_channels)
+        return "group_tokens / group_channels must be 16, 32, 64 or 128";
+    if (page_size <= 0 || group_tokens % page_size) return "page_size must divide the K group";
+    if (packed_start_offset < 0 || packed_start_offset >= page_size || seg_group_base < 0)
+        return "packed_start_offset must be in [0,page_size), seg_group_base >= 0";
+    if (k_outliers < 0 || k_outliers > 16 || k_outliers > group_tokens || num_splits < 1 ||
+        num_splits > 256 || (index_repr != 0 && index_repr != 1))
+        return "k_outliers in [0,min(16,group_tokens)], num_splits in [1,256], index_repr 0|1";
     if ((reinterpret_cast<uintptr_t>(k_base) | reinterpret_cast<uintptr_t>(v_main) |
          reinterpret_cast<uintptr_t>(v_zp) | reinterpret_cast<uintptr_t>(k_index) |
          reinterpret_cast<uintptr_t>(k_oval) | reinterpret_cast<uintptr_t>(k_zp) |
-         reinterpret_cast<uintptr_t>(k_ms) | reinterpret_cast<uintptr_t>(k_mc)) & 7) {
-        set_error("ommx_decode_splitkv: planes must be 8-byte aligned");
-        return -1;
-    }
-    if (!q || !b_seq_len || !attn_logits || !req_to_token || !req_to_group) {
-        set_error("ommx_decode_splitkv: null pointer");
-        return -1;
-    }
-    if ((k_outliers > 0 && (!k_index || !k_oval)) || (!k_ms != !k_mc)) {
-        set_error("ommx_decode_splitkv: outlier planes missing");
-        return -1;
-    }
-    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, static_cast<const int8_t*>(k_scale), k_zp, k_ms, k_mc,
-                 k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
-                 table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
-                 B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
-                 group_tokens, group_channels, v_bf16 ? 1 : 0};
+         reinterpret_cast<uintptr_t>(k_ms) | reinterpret_cast<uintptr_t>(k_mc)) & 7)
+        return "planes must be 8-byte aligned";
+    // (plane pointers may be null: an empty cache is legal when every b_seq_len is zero, and then
+    // no plane is read)
+    if (!q || !b_seq_len || !attn_logits || !req_to_token || !req_to_group) return "null pointer";
+    if ((k_outliers > 0 && (!k_index || !k_oval)) || (!k_ms != !k_mc)) return "outlier planes missing";
+    return nullptr;
+}
+
+static DecodeArgs make_decode_args(OMMX_DECODE_PARAMS) {
+    (void)D; (void)stream;
+    return DecodeArgs{q, q_stride_b, q_stride_h, k_base, static_cast<const int8_t*>(k_scale), k_zp, k_ms, k_mc,
+                      k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride,
+                      req_to_group, rg_stride, table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h,
+                      al_stride_s, B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
+                      packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
+                      group_tokens, group_channels, v_bf16 ? 1 : 0};
+}
+
+static void set_error2(const char* where, const char* what) { g_error = std::string(where) + ": " + what; }
+
+}  // namespace ommx
+
+extern "C" int ommx_decode_splitkv(OMMX_DECODE_PARAMS) {
+    using namespace ommx;
+    if (const char* bad = check_decode(OMMX_DECODE_ARGS)) { set_error2("ommx_decode_splitkv", bad); return -1; }
+    const DecodeArgs a = make_decode_args(OMMX_DECODE_ARGS);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = launch_decode_fast(a, D, R, st);
-    if (rc == 1) rc = launch_decode_ref(a, D, R, st);
+    int rc = launch_decode_fast(a, D, Hq / Hkv, st);
+    if (rc == 1) rc = launch_decode_ref(a, D, Hq / Hkv, st);      // shapes the matrix-core kernel leaves out
     if (rc != 0) { set_error("ommx_decode_splitkv: no kernel for this shape"); return -1; }
     if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_splitkv: launch failed"); return -2; }
     return 0;
 }
 
 // Same operator through the plain fp32 kernel only (cross-check entry used by tests).
-extern "C" int ommx_decode_splitkv_ref(
-    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
-    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
-    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
-    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
-    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
-    int table_i64, const int32_t* b_seq_len,
-    float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,
-    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int v_bf16, int num_splits,
-    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,
-    void* stream) {
+extern "C" int ommx_decode_splitkv_ref(OMMX_DECODE_PARAMS) {
     using namespace ommx;
-    if (B <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 || num_splits < 1 || k_outliers < 0 ||
-        k_outliers > 16 || (index_repr != 0 && index_repr != 1) ||
-        !(group_tokens == 16 || group_tokens == 32 || group_tokens == 64 || group_tokens == 128) ||
-        !(group_channels == 16 || group_channels == 32 || group_channels == 64 || group_channels == 128) ||
-        group_tokens % page_size || k_outliers > group_tokens || D % group_channels) {
-        set_error("ommx_decode_splitkv_ref: bad arguments");
-        return -1;
-    }
-    DecodeArgs a{q, q_stride_b, q_stride_h, k_base, static_cast<const int8_t*>(k_scale), k_zp, k_ms, k_mc,
-                 k_index, k_oval, v_main, static_cast<const int8_t*>(v_scale), v_zp, req_to_token, rt_stride, req_to_group, rg_stride,
-                 table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h, al_stride_s,
-                 B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
-                 packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
-                 group_tokens, group_channels, v_bf16 ? 1 : 0};
+    if (const char* bad = check_decode(OMMX_DECODE_ARGS)) { set_error2("ommx_decode_splitkv_ref", bad); return -1; }
+    const DecodeArgs a = make_decode_args(OMMX_DECODE_ARGS);
     if (launch_decode_ref(a, D, Hq / Hkv, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_splitkv_ref: unsupported shape");
         return -1;
