@@ -317,6 +317,23 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     } else {
         L = a.seq[b];
     }
+    // q is requested first: it only needs the request index, and it is long here when the A
+    // operands are built (after the first plane rows have been requested, while they travel).
+    // qw: this lane's 32 channels of q of head j % HR, 16 dwords, channel 2i in the low half of
+    // dword i; qraw: channels 2*lane, 2*lane+1 of every head (for the channel pass).
+    uint32_t qw[16], qraw[HR];
+    {
+        const uint32_t* qh = reinterpret_cast<const uint32_t*>(
+            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & (HR - 1), heads - 1)) * a.q_sh + 32 * kq);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) qw[i] = qh[i];
+        if (OUTLIERS) {
+#pragma unroll
+            for (int r = 0; r < HR; ++r)
+                qraw[r] = *reinterpret_cast<const uint32_t*>(
+                    a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
+        }
+    }
     constexpr int GT = 32 << GTS;
     static_assert(GTS == 0 || IDX == 1, "longer groups are read through position streams");
     static_assert(KO == 6 || (KO == 10 && IDX == 1), "10 outliers: position streams only");
@@ -359,12 +376,15 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // The loop is software-pipelined by hand: table entries are fetched two iterations
     // ahead, plane data one iteration ahead, each into the registers its previous use
     // has just released.
-    int row1, gsl[2];                     // physical row of token n + lane / group slots, of the NEXT data loads
+    // Page entry and slot in the page of token n + lane, group slots: of the NEXT data loads.  The
+    // entries stay as loaded until fetch_kv turns them into a row: arithmetic on them here would
+    // put a wait for the table loads (and for every older load) right behind their issue.
+    int pg1, ps1, gsl[2];
     auto fetch_tables = [&](int n) {
         {
             const int p = min(n + lane, last) + tok_off;
-            const int pg = *reinterpret_cast<const int*>(rt_b + ((uint32_t)(p >> ps_sh) << tsh));
-            row1 = (pg << ps_sh) + (p & ps_mask);
+            pg1 = *reinterpret_cast<const int*>(rt_b + ((uint32_t)(p >> ps_sh) << tsh));
+            ps1 = p & ps_mask;
         }
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -376,6 +396,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     u32x2 vzp;
     uint32_t vsc;
     auto fetch_kv = [&]() {
+        const int row1 = (pg1 << ps_sh) + ps1;              // physical row of this lane's token
         const uint64_t ro = (uint64_t)(uint32_t)row1 * row_bytes;
         kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
         kr[1] = *reinterpret_cast<const u32x4*>(kb_head + ro + 16);
@@ -445,12 +466,23 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         }
     };
     auto fetch_params = [&]() { fetch_params_g(0); fetch_params_g(1); };
-    if (n_begin < n_end) {
-        fetch_tables(n_begin);
-        fetch_kv();
-        fetch_params();
-        fetch_tables(n_begin + 64);
+    if (n_begin >= n_end) {
+        // An empty split leaves the state of nothing attended (o = 0, lse = -inf) and is done.
+        // (Leaving here, rather than running the rest with an empty loop, also keeps the loads
+        // below on every path that reaches the A operands: the waits placed there then let the
+        // plane rows travel while the operands are built.)
+        for (int r = 0; r < heads; ++r) {
+            float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
+            dst[lane] = 0.0f;
+            dst[64 + lane] = 0.0f;
+            if (lane == 0) dst[D] = -INFINITY;
+        }
+        return;
     }
+    fetch_tables(n_begin);
+    fetch_kv();
+    fetch_params();
+    fetch_tables(n_begin + 64);
 
     // ---- A operands: scaled q of head j % HR for this lane's 32-channel quarter ---------
     // (pair order: q * 2^(7-2k) with k the code position of the pair, see k_pair; natural
@@ -459,12 +491,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // natural order (outlier tile): k=(ks,kq,r) <-> channel 32kq + 8ks + r
     u32x4 aq_pair[4], aq_nat[4];
     {
-        // this lane's 32 channels of q: 16 dwords, channel 2i in the low half of dword i
-        const uint32_t* qh = reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & (HR - 1), heads - 1)) * a.q_sh + 32 * kq);
-        uint32_t qw[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) qw[i] = qh[i];
         auto q_at = [&](int c) {          // channel c of the quarter as fp32 (exact)
             return __uint_as_float((c & 1) ? (qw[c >> 1] & 0xFFFF0000u) : (qw[c >> 1] << 16));
         };
@@ -484,7 +510,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // q of every head for the channel pass, channels 2*lane and 2*lane+1: as fp32 with 4
     // heads, left as the bf16 pair with 8 (registers are short there, and the residual walk
     // that reads them is rare)
-    uint32_t qraw[HR];
     float qf[2][4];
     auto q4_at = [&](int u, int r) {      // 4*q
         if constexpr (HR == 4) return qf[u][r];
@@ -493,10 +518,6 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // per channel: the |delta/4| from which the residual matters (infinite for q = 0)
     float big_thr[2] = {0.0f, 0.0f};
     if (OUTLIERS) {
-#pragma unroll
-        for (int r = 0; r < HR; ++r)
-            qraw[r] = *reinterpret_cast<const uint32_t*>(
-                a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
         if constexpr (HR == 4) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
