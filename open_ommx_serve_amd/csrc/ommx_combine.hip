@@ -174,8 +174,8 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
-    // Pieces per head.  At batch 1 the kernel is latency bound and 2 pieces measured best (36.7 us
-    // per step at 64K against 38.1 with one, 36.7 with four, 37.2 with eight); with many
+    // Pieces per head.  At batch 1 the kernel is latency bound and 2 pieces measured best (1.4 us
+    // per step at 64K less than one, the same as four, 0.5 us less than eight); with many
     // (request, head) pairs the grid fills the chip by itself and one piece repeats no work.
     const bool split2 = a.B * a.Hq < 256;
     const dim3 grid(a.B, a.Hq, split2 ? 2 : 1);
