@@ -29,7 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the split-KV kernel at the default workload (ctx 65536, 255
+# HBM bytes per launch of the split-KV kernel at the default workload (ctx 65536, 256
 # splits), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 256 MiB copy kernel
 # (profiles/decode_ctx64k_hbm_traffic.txt); counters cannot be read from inside this script.
 TRAFFIC_BYTES_CTX64K = 74.03e6
@@ -85,7 +85,11 @@ def _make_runner(case, splits=None):
     dev = case.q.device
     kw = case.decode_kwargs()
     n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
-    S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu, Hq // case.kv_heads)
+    # the lengths of the synthetic requests are known on the host: pass their mean as the hint a
+    # serving caller would take from its own bookkeeping
+    mean_len = sum(case.packed_lens) / len(case.packed_lens)
+    S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu, Hq // case.kv_heads,
+                                     mean_seq_len=mean_len)
     ws = make_attn_logits(B, Hq, S, D, dev)
     o = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)

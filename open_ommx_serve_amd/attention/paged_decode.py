@@ -31,11 +31,17 @@ def _cu_count(device: torch.device) -> int:
 
 
 def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256,
-                       q_per_kv: int = 4, group_tokens: int = 32) -> int:
+                       q_per_kv: int = 4, group_tokens: int = 32,
+                       mean_seq_len: Optional[float] = None) -> int:
     """Split count that gives every compute unit four workgroups, two resident and two queued
     behind them so that requests of different length even out (a workgroup is four waves of
     one split; a wave covers one kv head and all of its q heads, so ``q_per_kv`` does not
-    enter), but never less than one
+    enter) -- or only the two resident ones when ``mean_seq_len`` says that the requests are
+    about equally long (at least 0.9 of the longest) and a workgroup would get at most eight
+    64-token steps: little is left to even out then, and a second round of workgroups mostly
+    pays the start-up of a workgroup (about one step) again, 10 % of the whole on short splits;
+    with longer splits the second round still wins, by absorbing the spread of the
+    workgroups' own run times -- but never less than one
     64-token step per split (one 32-token group when even that leaves units idle): a wave's time
     is a fixed part plus ~5 us per step, so while compute units are idle more splits are faster;
     and the steps are dealt out evenly (the split length
@@ -47,6 +53,9 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
     gt = max(32, int(group_tokens))
     step_tokens = max(64, gt)
     steps = max(1, (int(max_seq_len) + step_tokens - 1) // step_tokens)
+    equal = mean_seq_len is not None and float(mean_seq_len) >= 0.9 * float(max_seq_len)
+    if equal and (steps + min(want, steps) - 1) // min(want, steps) <= 8:
+        want = max(1, min(256, (2 * int(n_cu)) // wgs_per_split))
     if want >= 2 * steps:          # plenty of idle units: splits of one K group
         return int(min(want, max(1, (int(max_seq_len) + gt - 1) // gt)))
     target = max(1, min(want, steps))
@@ -92,12 +101,17 @@ def ommx_paged_decode_attention_canonical(
     packed_start_offset: int = 0,
     seg_group_base: int = 0,
     _force_reference_kernel: bool = False,
+    mean_seq_len: Optional[float] = None,
 ) -> None:
     """Canonical-KV paged decode attention.  Writes ``o [B,Hq,D]`` / ``lse [B,Hq]`` in place.
 
     Plane layouts, tables and the tail are as documented for the reference launcher
     (``paged_decode.py:2856-2887``).  ``seg_group_base > 0`` emits the un-merged state of a
     group-range segment without the tail (``:2892-2902``).
+
+    ``mean_seq_len`` (not in the reference's signature) is a hint for the automatic split count
+    only: a caller that passes ``max_seq_len`` to avoid the host sync may also say how long the
+    requests are on average, see :func:`auto_num_kv_splits`.
     """
     pages, ngroups = int(k_base.shape[0]), int(k_scale.shape[0])
     ps = int(page_size)
@@ -199,10 +213,16 @@ def ommx_paged_decode_attention_canonical(
     _hip.require_gpu(q.device)
     if max_seq_len is not None:
         max_seq = max(1, int(max_seq_len))
+    elif num_kv_splits is None and int(b_seq_len.numel()) > 0:
+        lens = b_seq_len.tolist()                      # the one host sync of this path
+        max_seq = max(1, max(lens))
+        if mean_seq_len is None:
+            mean_seq_len = sum(lens) / len(lens)
     else:
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
     if num_kv_splits is None:
-        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv, group_tokens)
+        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv, group_tokens,
+                                           mean_seq_len)
     S = max(1, int(num_kv_splits))
     if attn_logits is None:
         attn_logits = make_attn_logits(B, Hq, S, D, q.device)
