@@ -3,7 +3,7 @@ operator (split-KV kernel + combine kernel) on one MI355X, Llama-3.1-8B attentio
 (32 q heads, 8 kv heads, d=128), batch 1, synthetic caches, context 1K..64K.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--ctx 65536] [--no-ladder]
-                    [--no-cpu-baseline] [--batch B] [--q-heads H]
+                    [--no-cpu-baseline] [--batch B] [--q-heads H] [--ragged]
 
 One step = one decode call over one batch: the split-KV launch followed by the combine
 launch, operands resident in HBM, workspace preallocated.  Steps are replayed from HIP
@@ -148,6 +148,9 @@ def main() -> int:
                     help="requests per step (other workloads than the headline one, e.g. "
                          "--batch 8 --ctx 32768 --q-heads 64 for the 8-request GQA-8 configuration)")
     ap.add_argument("--q-heads", type=int, default=32)
+    ap.add_argument("--ragged", action="store_true",
+                    help="with --batch: request lengths uniform in [1024, ctx] (seeded) instead of "
+                         "all ctx, e.g. --batch 32 --ctx 16384 --ragged")
     ap.add_argument("--no-ladder", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -171,7 +174,11 @@ def main() -> int:
     torch.cuda.set_device(0)
 
     def measure(ctx, steps, warmup):
-        case = build_decode_case([ctx] * args.batch, q_heads=args.q_heads, seed=42, permute_tables=True,
+        lens = [ctx] * args.batch
+        if args.ragged:
+            g = torch.Generator().manual_seed(4)
+            lens = torch.randint(1024, ctx + 1, (args.batch,), generator=g).tolist()
+        case = build_decode_case(lens, q_heads=args.q_heads, seed=42, permute_tables=True,
                                  sparse_frac=0.005)
         step, stage1, o, lse, S = _make_runner(case, args.splits or None)
         # one model forward runs this operator once per layer inside a single graph, so the
@@ -250,7 +257,9 @@ def main() -> int:
         "vs_baseline": round(p50 / H200_P50_US_64K, 5) if (args.ctx == 65536 and headline) else None,
         "dtype": "u8 planes, bf16 q, f32 accumulate", "data": "synthetic",
         "config": {"workload": f"OMMX paged decode attention, {args.q_heads} q / 8 kv heads, d=128, "
-                               f"batch {args.batch}, ctx {args.ctx} ({L} packed tokens + {int(case.b_tail_len[0])} bf16 "
+                               f"batch {args.batch}, ctx {'1024..' if args.ragged else ''}{args.ctx} "
+                               f"({sum(case.packed_lens) if args.ragged else L} packed tokens"
+                               f"{' in all' if args.ragged else ''} + {int(case.b_tail_len[0])} bf16 "
                                f"tail rows), page 16, permuted page/group tables, K outliers 4 "
                                f"channels x12 + 0.5% x8",
                    "num_kv_splits": m["S"], "launch": m["mode"],
