@@ -304,7 +304,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // Requests are served longest first: workgroups are dispatched in grid order, so the ones that
     // start last, when most compute units have run dry, belong to the shortest requests.
     // blockIdx.z is the rank of the request by (length descending, index ascending); every wave
-    // finds its request from the lengths (one per lane, up to 64 requests).
+    // finds its request from the lengths: up to 64 requests by counting, lane by lane, the keys
+    // above its own; up to 256 (four keys per lane) by a radix select of the key of that rank,
+    // one bit per round; more keep the grid order.
     int b = blockIdx.z, L;
     if (a.B > 1 && a.B <= 64) {
         const int my_len = lane < a.B ? a.seq[lane] : 0;
@@ -314,6 +316,29 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             rank += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key), i)) > key;
         b = __builtin_ctzll(__ballot(lane < a.B && rank == static_cast<int>(blockIdx.z)));
         L = __builtin_amdgcn_readlane(my_len, b);
+    } else if (a.B <= 256) {
+        // key = (length + 1, 255 - index): distinct, and above the zero of an unused slot
+        uint32_t key[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = 64 * r + lane;
+            key[r] = idx < a.B ? (static_cast<uint32_t>(a.seq[idx] + 1) << 8) | (255u - idx) : 0u;
+        }
+        // the largest value that more than blockIdx.z keys reach is the key of rank blockIdx.z
+        uint32_t want = 0;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = want | (1u << bit);
+            int reach = 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) reach += __popcll(__ballot(key[r] >= cand));
+            if (reach > static_cast<int>(blockIdx.z)) want = cand;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint64_t hit = __ballot(key[r] == want);
+            if (hit) b = 64 * r + __builtin_ctzll(hit);
+        }
+        L = static_cast<int>(want >> 8) - 1;
     } else {
         L = a.seq[b];
     }

@@ -137,11 +137,11 @@ def test_ragged_batch_32_requests():
     _check(_run(case), _oracle(case), "B32")
 
 
-@pytest.mark.parametrize("batch", [2, 64, 65, 70])
+@pytest.mark.parametrize("batch", [2, 64, 65, 70, 130, 256, 257])
 def test_longest_first_request_order(batch):
-    """The matrix-core kernel serves up to 64 requests longest first (more keep the grid order):
-    equal lengths, zero lengths and both sides of the 64-request limit give every request its
-    own result."""
+    """The matrix-core kernel serves up to 256 requests longest first (by counting up to 64, by a
+    radix select beyond; more keep the grid order): equal lengths, zero lengths and both sides
+    of the two limits give every request its own result."""
     g = torch.Generator().manual_seed(batch)
     lens = torch.randint(40, 700, (batch,), generator=g).tolist()
     lens[0] = lens[-1] = 500                      # ties
