@@ -84,13 +84,14 @@ def test_split_heuristic_bounds():
     assert auto_num_kv_splits(960, 1, 8, 256) >= 1
     assert auto_num_kv_splits(65472, 1, 8, 256) == 256
     assert auto_num_kv_splits(960, 1, 8, 256) == 30          # one 32-token group per split
-    assert auto_num_kv_splits(65472, 32, 8, 256) == 16
+    assert auto_num_kv_splits(16320, 32, 8, 256) == 16
+    assert auto_num_kv_splits(65472, 32, 8, 256) == 32         # long splits, lengths may differ: finer
     # equal lengths (mean close to the longest) and short splits: two workgroups per compute unit
     # instead of four
     assert auto_num_kv_splits(8128, 32, 8, 256, mean_seq_len=8128) == 8
     assert auto_num_kv_splits(8128, 32, 8, 256) == 16
     assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=65472) == 16      # long splits: stay
-    assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=30000) == 16
+    assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=30000) == 32
     assert auto_num_kv_splits(32704, 8, 8, 256, 8, mean_seq_len=32704) == 32
     assert auto_num_kv_splits(65472, 1, 8, 256, mean_seq_len=65472) == 256
     assert 1 <= auto_num_kv_splits(1, 1, 1, 256) <= 256
