@@ -172,6 +172,204 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
     }
 }
 
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// The same merge for a whole kv head at a time: one workgroup of 512 threads per (request, kv
+// head) serves the R = 4 or 8 q heads of that kv head, so the bf16 tail rows -- most of the bytes
+// when there are few splits -- are read once instead of once per q head.  Used when (request, kv
+// head) pairs alone fill the chip twice over (then nothing is gained by one workgroup per q
+// head) and there are at most 64 splits.  Wave r < R owns the scalars of head r (split weights, running tail maximum
+// and sum); the channel work is dealt out as (head, channel) for the splits and as (channel
+// pair, row group) for the tail's P.V.
+template <int D, int R>
+__global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
+    constexpr int NT = 512, MAXS = 64;
+    constexpr int ROWS = 128;              // tail rows per pass (two per thread of the logit layout)
+    constexpr int CHP = D / 8;             // channels per thread of a K row (8 threads per row)
+    constexpr int NRG = NT / (D / 2);      // row groups of the P.V layout
+    constexpr int HD = (R * D + NT - 1) / NT;   // (head, channel) items per thread
+    __shared__ __attribute__((aligned(16))) float s_q[R][D];
+    __shared__ float s_w[R][MAXS];
+    __shared__ float s_gmax[R], s_W[R], s_alpha[R], s_tm[R], s_tl[R];
+    __shared__ float s_logit[R][ROWS];
+    __shared__ float s_p[R][ROWS];
+    __shared__ float s_red[NRG][R][D];
+    const int b = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int h0 = kvh * R;
+    const float* base = a.al + b * a.al_b + (int64_t)h0 * a.al_h;
+    const int L = a.seq[b];
+    const int tail = a.tail ? a.tail[b] : 0;
+
+    // ---- split weights: wave r, lane s ----------------------------------------------------
+    if (a.q) {
+        for (int i = tid; i < R * D / 2; i += NT) {
+            const int r = i / (D / 2), c2 = i % (D / 2);
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(
+                a.q + b * a.q_sb + (int64_t)(h0 + r) * a.q_sh + 2 * c2);
+            s_q[r][2 * c2] = __uint_as_float(w << 16);
+            s_q[r][2 * c2 + 1] = __uint_as_float(w & 0xFFFF0000u);
+        }
+    }
+    const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:2407
+    if (wave < R) {
+        const bool valid = lane < a.S && min(per * lane + per, L) > per * lane;
+        const float my_lse = valid ? base[(int64_t)wave * a.al_h + (int64_t)lane * a.al_s + D] : -INFINITY;
+        const float g_max = wave_max_f32(my_lse);
+        const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
+        const float w = my_lse == -INFINITY ? 0.0f : __expf(my_lse - g_safe);
+        const float W = wave_sum_f32(w);
+        s_w[wave][lane] = w;
+        if (lane == 0) { s_gmax[wave] = g_max; s_W[wave] = W; }
+    }
+    __syncthreads();
+
+    // ---- split part: item (head, channel), absent splits are not read ----------------------
+    float A[HD];
+#pragma unroll
+    for (int k = 0; k < HD; ++k) {
+        A[k] = 0.0f;
+        const int i = tid + k * NT;
+        if (i < R * D) {
+            const int r = i / D, d = i % D;
+            const float* p = base + (int64_t)r * a.al_h + d;
+            float acc = 0.0f;
+#pragma unroll 8
+            for (int sp = 0; sp < a.S; ++sp) {
+                const float w = s_w[r][sp];
+                if (w > 0.0f) acc = fmaf(w, p[(int64_t)sp * a.al_s], acc);
+            }
+            A[k] = acc;
+        }
+    }
+
+    // ---- tail: passes of up to ROWS rows, online over passes ------------------------------
+    float m_run = -INFINITY, l_run = 0.0f;          // of head `wave` (waves < R)
+    float acc[R][2];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r][0] = acc[r][1] = 0.0f;
+    const int dp = tid % (D / 2), rg = tid / (D / 2);
+    for (int r0 = 0; r0 < tail; r0 += ROWS) {
+        const int nr = min(ROWS, tail - r0);
+        {   // logits: thread (row, part) takes CHP channels of rows row and row + 64
+            const int part = tid & 7, row = tid >> 3;
+#pragma unroll
+            for (int rr = 0; rr < ROWS; rr += 64) {
+                const int t = row + rr;
+                float dot[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) dot[r] = 0.0f;
+                if (t < nr) {
+                    const uint16_t* kp = a.kt + b * a.kt_b + (int64_t)(r0 + t) * a.kt_t +
+                                         (int64_t)kvh * a.kt_h + part * CHP;
+#pragma unroll
+                    for (int c8 = 0; c8 < CHP / 8; ++c8) {
+                        const uint4 ku = reinterpret_cast<const uint4*>(kp)[c8];
+                        const uint32_t w[4] = {ku.x, ku.y, ku.z, ku.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float k0 = __uint_as_float(w[i] << 16);
+                            const float k1 = __uint_as_float(w[i] & 0xFFFF0000u);
+                            const int c = part * CHP + 8 * c8 + 2 * i;
+#pragma unroll
+                            for (int r = 0; r < R; ++r)
+                                dot[r] = fmaf(s_q[r][c + 1], k1, fmaf(s_q[r][c], k0, dot[r]));
+                        }
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int o = 1; o < 8; o <<= 1) dot[r] += __shfl_xor(dot[r], o);
+                }
+                if (part == 0) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        s_logit[r][t] = t < nr ? apply_cap(dot[r] * a.sm_scale, a.cap) : -INFINITY;
+                }
+            }
+        }
+        __syncthreads();
+        if (wave < R) {   // softmax bookkeeping of head `wave`: rows lane and lane + 64
+            const float x0 = s_logit[wave][lane], x1 = s_logit[wave][lane + 64];
+            const float m_new = fmaxf(m_run, wave_max_f32(fmaxf(x0, x1)));
+            const float alpha = (m_run == -INFINITY) ? 0.0f : __expf(m_run - m_new);
+            const float p0 = x0 == -INFINITY ? 0.0f : __expf(x0 - m_new);
+            const float p1 = x1 == -INFINITY ? 0.0f : __expf(x1 - m_new);
+            l_run = l_run * alpha + wave_sum_f32(p0 + p1);
+            m_run = m_new;
+            s_p[wave][lane] = p0;
+            s_p[wave][lane + 64] = p1;
+            if (lane == 0) s_alpha[wave] = alpha;
+        }
+        __syncthreads();
+        {   // P.V: thread (channel pair, row group)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float al = s_alpha[r];
+                acc[r][0] *= al;
+                acc[r][1] *= al;
+            }
+            for (int t = rg; t < nr; t += NRG) {
+                const uint32_t vv = *reinterpret_cast<const uint32_t*>(
+                    a.vt + b * a.vt_b + (int64_t)(r0 + t) * a.vt_t + (int64_t)kvh * a.vt_h + 2 * dp);
+                const float v0 = __uint_as_float(vv << 16), v1 = __uint_as_float(vv & 0xFFFF0000u);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float p = s_p[r][t];
+                    acc[r][0] = fmaf(p, v0, acc[r][0]);
+                    acc[r][1] = fmaf(p, v1, acc[r][1]);
+                }
+            }
+        }
+        // (the next pass writes s_logit before its first barrier and s_p after it: both are
+        // past every read of this pass)
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        s_red[rg][r][2 * dp] = acc[r][0];
+        s_red[rg][r][2 * dp + 1] = acc[r][1];
+    }
+    if (wave < R && lane == 0) { s_tm[wave] = m_run; s_tl[wave] = l_run; }
+    __syncthreads();
+
+    // ---- both parts together, item (head, channel) ------------------------------------------
+#pragma unroll
+    for (int k = 0; k < HD; ++k) {
+        const int i = tid + k * NT;
+        if (i < R * D) {
+            const int r = i / D, d = i % D;
+            float TA = 0.0f;
+#pragma unroll
+            for (int g = 0; g < NRG; ++g) TA += s_red[g][r][d];
+            const float TL = s_tl[r], t_m = s_tm[r], g_max = s_gmax[r];
+            float W = s_W[r], Av = A[k];
+            const float tail_lse = TL > 0.0f ? t_m + __logf(TL) : -INFINITY;
+            const float n_max = fmaxf(g_max, tail_lse);
+            const float n_safe = (n_max == -INFINITY) ? 0.0f : n_max;
+            const float rs = (g_max == -INFINITY) ? 0.0f : __expf(g_max - n_safe);
+            W *= rs;
+            Av *= rs;
+            if (TL > 0.0f) {
+                const float w = __expf(tail_lse - n_safe);
+                W += w;
+                Av = fmaf(w, TA / TL, Av);
+            }
+            a.o[b * a.o_b + (int64_t)(h0 + r) * a.o_h + d] = W > 0.0f ? Av / W : 0.0f;
+            if (d == 0) a.lse[b * a.lse_b + h0 + r] = W > 0.0f ? n_max + __logf(W) : -INFINITY;
+        }
+    }
+}
+
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     if (a.S > 256) return -1;
     // Pieces per head.  At batch 1 the kernel is latency bound and 2 pieces measured best (1.4 us
@@ -180,6 +378,18 @@ int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     const bool split2 = a.B * a.Hq < 256;
     const dim3 grid(a.B, a.Hq, split2 ? 2 : 1);
     const bool small = !split2 && a.S <= 64;
+    const int R = a.Hq / a.Hkv;
+    // a whole kv head per workgroup once those alone are two per compute unit (128 requests of 8
+    // kv heads: 29 against 47 us; with fewer, one workgroup per q head spreads the work better)
+    if (small && (R == 4 || R == 8) && a.Hq == R * a.Hkv && a.B * a.Hkv >= 512) {
+        const dim3 g2(a.B, a.Hkv);
+        if (D == 128 && R == 4) hipLaunchKernelGGL((combine_grouped_kernel<128, 4>), g2, dim3(512), 0, st, a);
+        else if (D == 128) hipLaunchKernelGGL((combine_grouped_kernel<128, 8>), g2, dim3(512), 0, st, a);
+        else if (D == 64 && R == 4) hipLaunchKernelGGL((combine_grouped_kernel<64, 4>), g2, dim3(512), 0, st, a);
+        else if (D == 64) hipLaunchKernelGGL((combine_grouped_kernel<64, 8>), g2, dim3(512), 0, st, a);
+        else return -1;
+        return 0;
+    }
     if (D == 128 && split2) hipLaunchKernelGGL((combine_kernel<128, 2>), grid, dim3(1024), 0, st, a);
     else if (D == 128 && small) hipLaunchKernelGGL((combine_kernel<128, 1, 512, 64>), grid, dim3(512), 0, st, a);
     else if (D == 128) hipLaunchKernelGGL((combine_kernel<128, 1>), grid, dim3(1024), 0, st, a);

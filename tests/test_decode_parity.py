@@ -154,6 +154,50 @@ def test_longest_first_request_order(batch):
         _check(_run(case, num_kv_splits=S), want, f"B{batch} S{S}")
 
 
+def _run_one(case, i, **over):
+    """Request i of a batch as a one-request call (same planes and tables, row i of the rest)."""
+    B, Hq, D = case.q.shape
+    o = torch.full((1, Hq, D), float("nan"), dtype=torch.float32, device=case.q.device)
+    lse = torch.full((1, Hq), float("nan"), dtype=torch.float32, device=case.q.device)
+    args = list(case.decode_args(o, lse))
+    for k in (0, 9, 10, 11, 14, 15, 16):          # q, tails, tables, lengths
+        args[k] = args[k][i:i + 1].contiguous()
+    kw = case.decode_kwargs()
+    kw.update(over)
+    ommx_paged_decode_attention_canonical(*args, **kw)
+    torch.cuda.synchronize()
+    return o.cpu()[0], lse.cpu()[0]
+
+
+@pytest.mark.parametrize("hq,hkv,D,kw", [
+    (32, 8, 128, {}), (64, 8, 128, {}), (16, 4, 64, {}), (32, 4, 64, {}),
+    (32, 8, 128, dict(group_tokens=128, group_channels=128, outlier_repr="relidx7")),   # tails past 128 rows
+])
+def test_batches_combine_per_kv_head(hq, hkv, D, kw):
+    """With 512 or more (request, kv head) pairs and at most 64 splits the combine serves a whole
+    kv head per workgroup: against the oracle over split counts, and -- capped logits, segment
+    form -- against the same requests sent one by one (which take the per-head kernel)."""
+    B = 512 // hkv + 3
+    pool = [9, 40, 71, 72, 200, 1000, 1500, 333, 2047, 640, 4100, 136, 168, 900, 77]
+    lens = [pool[i % len(pool)] + 3 * (i // len(pool)) for i in range(B)]
+    case = build_decode_case(lens, q_heads=hq, kv_heads=hkv, head_dim=D, seed=31 + hq + D,
+                             permute_tables=True, sparse_frac=0.005, **kw)
+    assert B * hkv >= 512
+    if kw:
+        assert max(case.b_tail_len.tolist()) > 128
+    want = _oracle(case)
+    for S in (None, 1, 5, 64):
+        _check(_run(case, num_kv_splits=S), want, f"S{S}")
+    for over in (dict(logit_cap=4.0), dict(seg_group_base=0, max_tail_len=0)):
+        o, lse = _run(case, num_kv_splits=6, **over)
+        for i in (0, 1, 5, B - 1):
+            o1, l1 = _run_one(case, i, num_kv_splits=6, **over)
+            assert torch.equal(torch.isfinite(lse[i]), torch.isfinite(l1))
+            fin = torch.isfinite(l1)
+            assert (o[i] - o1).abs().max().item() <= 2e-5, (over, i)
+            assert (lse[i][fin] - l1[fin]).abs().max().item() <= 2e-5 if fin.any() else True
+
+
 @pytest.mark.parametrize("ref_kernel", [False, True])
 def test_gqa8_64_q_heads(ref_kernel):
     case = build_decode_case([2048, 3000], q_heads=64, kv_heads=8, seed=8, sparse_frac=0.005)
