@@ -233,7 +233,9 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
     }
     __syncthreads();
 
-    // ---- split part: item (head, channel), absent splits are not read ----------------------
+    // ---- split part: item (head, channel) ---------------------------------------------------
+    // Every split slot is read (it exists; an absent split's content is stale and is dropped by
+    // the select), so that the loads carry no branch and go out eight at a time.
     float A[HD];
 #pragma unroll
     for (int k = 0; k < HD; ++k) {
@@ -243,10 +245,15 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
             const int r = i / D, d = i % D;
             const float* p = base + (int64_t)r * a.al_h + d;
             float acc = 0.0f;
-#pragma unroll 8
-            for (int sp = 0; sp < a.S; ++sp) {
-                const float w = s_w[r][sp];
-                if (w > 0.0f) acc = fmaf(w, p[(int64_t)sp * a.al_s], acc);
+            for (int s0 = 0; s0 < a.S; s0 += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = p[(int64_t)min(s0 + u, a.S - 1) * a.al_s];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const float w = s0 + u < a.S ? s_w[r][s0 + u] : 0.0f;
+                    acc = w > 0.0f ? fmaf(w, v[u], acc) : acc;
+                }
             }
             A[k] = acc;
         }
