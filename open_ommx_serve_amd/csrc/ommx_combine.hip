@@ -1,13 +1,16 @@
-// Split combine with the bf16 sink/recent tail folded in: Q workgroups of 1024 threads per
-// (request, q head), one per piece of the head's channels.  Follows ommx_gpu_serve/attention/paged_decode.py:2366-2500: valid
-// splits are recomputed from the packed length with the stage-1 rounding; the tail is one
-// more softmax part computed here from k_tail/v_tail; o = sum w_i o_i / sum w_i,
-// lse = max + ln sum w_i; nothing attended gives o = 0, lse = -inf.
+// Split combine with the bf16 sink/recent tail folded in.  Follows
+// ommx_gpu_serve/attention/paged_decode.py:2366-2500: valid splits are recomputed from the
+// packed length with the stage-1 rounding; the tail is one more softmax part computed here from
+// k_tail/v_tail; o = sum w_i o_i / sum w_i, lse = max + ln sum w_i; nothing attended gives
+// o = 0, lse = -inf.
 //
-// The kernel is latency bound (B*Hq small workgroups, a few KB each), so every global load
-// is issued before the first wait: thread (d, sg) owns channel d of the splits
-// sg, sg+NSG, ... and of the tail rows sg, sg+NSG, ...; for the tail logits the same threads
-// regroup as (row, 16 parts of the row).
+// Two kernels.  combine_kernel: Q workgroups per (request, q head), one per piece of the head's
+// channels.  It is latency bound (few small workgroups, a few KB each), so every global load is
+// issued before the first wait: thread (d, sg) owns channel d of the splits sg, sg+NSG, ... and
+// of the tail rows sg, sg+NSG, ...; for the tail logits the same threads regroup as (row, 16
+// parts of the row).  combine_grouped_kernel (further down): one workgroup per (request, kv head)
+// for large batches, where the tail rows are most of the bytes and are read once for all the
+// q heads of the kv head.
 #include "ommx_decode_args.h"
 
 namespace ommx {
