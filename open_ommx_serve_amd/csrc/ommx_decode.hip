@@ -281,7 +281,11 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 // 32-token pieces: piece v of a longer group reads the group's parameters again and takes the
 // outliers whose position falls into it.  The V vectors may then be 32, 64 or 128 channels wide.
 // KO: outliers per K vector, 6, or 10 (position streams, 128-token groups: the 2.75-bit recipe).
-template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0, int KO = 6>
+// MANYREQ: the request order of 65..256 requests (a radix select at the start).  A separate
+// instantiation, because its mere presence in the code costs the others 1.7 us at batch 1
+// (register allocation and scheduling of the start-up shift).
+template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0, int KO = 6,
+          bool MANYREQ = false>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -306,7 +310,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // blockIdx.z is the rank of the request by (length descending, index ascending); every wave
     // finds its request from the lengths: up to 64 requests by counting, lane by lane, the keys
     // above its own; up to 256 (four keys per lane) by a radix select of the key of that rank,
-    // one bit per round; more keep the grid order.
+    // one bit per round (the serving recipe's instantiations only); more keep the grid order.
     int b = blockIdx.z, L;
     if (a.B > 1 && a.B <= 64) {
         const int my_len = lane < a.B ? a.seq[lane] : 0;
@@ -316,7 +320,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             rank += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key), i)) > key;
         b = __builtin_ctzll(__ballot(lane < a.B && rank == static_cast<int>(blockIdx.z)));
         L = __builtin_amdgcn_readlane(my_len, b);
-    } else if (a.B <= 256) {
+    } else if (MANYREQ && a.B <= 256) {
         // key = (length + 1, 255 - index): distinct, and above the zero of an unused slot
         uint32_t key[4];
 #pragma unroll
@@ -1021,8 +1025,14 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     const size_t shm = (size_t)waves * (R <= 4 ? (a.kout > 0 ? LdsMap<4>::END : LdsMap<4>::DT)
                                                : (a.kout > 0 ? LdsMap<8>::END : LdsMap<8>::DT));
     const bool own_map = a.k_ms != nullptr;
-#define OMMX_LAUNCH(HR, IDX, MAP) \
-    hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a)
+#define OMMX_LAUNCH(HR, IDX, MAP)                                                                          \
+    do {                                                                                                   \
+        if (a.B > 64 && a.B <= 256)                                                                        \
+            hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP, false, 0, 6, true>), grid,  \
+                               block, shm, st, a);                                                         \
+        else                                                                                               \
+            hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a); \
+    } while (0)
 #define OMMX_LAUNCH_PARTIAL(IDX, MAP) \
     hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, 4, IDX, MAP, true>), grid, block, shm, st, a)
 #define OMMX_LAUNCH_LONG(HR, MAP, GTS) \
