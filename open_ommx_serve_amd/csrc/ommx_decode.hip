@@ -281,11 +281,12 @@ __device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t one_f16x2) {
 // 32-token pieces: piece v of a longer group reads the group's parameters again and takes the
 // outliers whose position falls into it.  The V vectors may then be 32, 64 or 128 channels wide.
 // KO: outliers per K vector, 6, or 10 (position streams, 128-token groups: the 2.75-bit recipe).
-// MANYREQ: the request order of 65..256 requests (a radix select at the start).  A separate
-// instantiation, because its mere presence in the code costs the others 1.7 us at batch 1
-// (register allocation and scheduling of the start-up shift).
+// ORDER: which request orders the code holds: 0 none (one request), 1 up to 64 requests, 2 up to
+// 256 as well (a radix select at the start).  Separate instantiations, because the mere presence
+// of that code costs the others at batch 1 (register allocation and scheduling of the start-up
+// shift): 1.7 us for the radix select, 0.4 us for the 64-request loop.
 template <bool OUTLIERS, int HR, int IDX, bool OWN_MAP, bool PARTIAL = false, int GTS = 0, int KO = 6,
-          bool MANYREQ = false>
+          int ORDER = 1>
 __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -312,7 +313,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     // above its own; up to 256 (four keys per lane) by a radix select of the key of that rank,
     // one bit per round (the serving recipe's instantiations only); more keep the grid order.
     int b = blockIdx.z, L;
-    if (a.B > 1 && a.B <= 64) {
+    if (ORDER >= 1 && a.B > 1 && a.B <= 64) {
         const int my_len = lane < a.B ? a.seq[lane] : 0;
         const uint32_t key = (static_cast<uint32_t>(my_len) << 6) | (63u - lane);   // distinct per lane
         int rank = 0;
@@ -320,7 +321,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
             rank += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key), i)) > key;
         b = __builtin_ctzll(__ballot(lane < a.B && rank == static_cast<int>(blockIdx.z)));
         L = __builtin_amdgcn_readlane(my_len, b);
-    } else if (MANYREQ && a.B <= 256) {
+    } else if (ORDER == 2 && a.B > 1 && a.B <= 256) {
         // key = (length + 1, 255 - index): distinct, and above the zero of an unused slot
         uint32_t key[4];
 #pragma unroll
@@ -1027,8 +1028,11 @@ int launch_decode_fast(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
     const bool own_map = a.k_ms != nullptr;
 #define OMMX_LAUNCH(HR, IDX, MAP)                                                                          \
     do {                                                                                                   \
-        if (a.B > 64 && a.B <= 256)                                                                        \
-            hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP, false, 0, 6, true>), grid,  \
+        if (a.B == 1)                                                                                      \
+            hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP, false, 0, 6, 0>), grid,     \
+                               block, shm, st, a);                                                         \
+        else if (a.B > 64 && a.B <= 256)                                                                   \
+            hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP, false, 0, 6, 2>), grid,     \
                                block, shm, st, a);                                                         \
         else                                                                                               \
             hipLaunchKernelGGL((decode_splitkv_mfma_kernel<true, HR, IDX, MAP>), grid, block, shm, st, a); \
