@@ -530,6 +530,18 @@ class MultiSeqKVPool:
         self._gather(kt, vt, tail_idx=tidx_dev, slots=sel)
         return self._bundle(sel, b_seq_len, b_tail_len, kt, vt, max_seq_len)
 
+    def decode_inputs_seq(self, sel: torch.Tensor, seq: torch.Tensor, b_seq_len: torch.Tensor,
+                          b_tail_len: torch.Tensor, max_seq_len: int) -> dict:
+        """Decode bundle from caller-owned fixed buffers that hold the pool slots (``sel``,
+        int64 ``[B]``) and the CURRENT sequence lengths (``seq``, int64 ``[B]``): the gather
+        launch derives the tail positions and writes ``b_seq_len`` / ``b_tail_len`` (int32
+        ``[B]``).  Device-only work; the reference's counterpart takes a host-filled ``[B, T]``
+        position matrix (kv_pool.py:886-936)."""
+        B = int(sel.shape[0])
+        d = self._decode_buffers(B)
+        self._gather(d["kt"], d["vt"], seq=seq, slots=sel, b_tail=b_tail_len, b_seq=b_seq_len)
+        return self._bundle(sel, b_seq_len, b_tail_len, d["kt"], d["vt"], max_seq_len)
+
     def decode_inputs_batched(self, slots: Sequence[int]) -> dict:
         """Decode bundle for ``slots`` from the host sequence lengths (kv_pool.py:938-1013):
         one small host-to-device copy, then one gather launch."""
