@@ -33,14 +33,14 @@ class _Request:
 
 
 class _Engine:
-    def __init__(self, max_context, **state):
+    def __init__(self, max_context, recipe=None, **state):
         self.state = BK.reset_worker_state(**state)
         self.builder = BK.OMMXCanonicalMetadataBuilder()
         self.layers = [NS() for _ in range(LAYERS)]
         self.impls = [BK.OMMXCanonicalImpl(HQ, D, SCALE, HKV) for _ in range(LAYERS)]
         for im in self.impls:
             im._ommx_serving_cfg = OMMXServingConfig(max_context=max_context, head_dim=D,
-                                                     n_q_heads=HQ, n_kv_heads=HKV)
+                                                     n_q_heads=HQ, n_kv_heads=HKV, **(recipe or {}))
         self.win = WindowSpec()
 
     def step(self, batch, check):
@@ -211,4 +211,33 @@ def test_batched_graph_route_replays_from_a_hip_graph():
     for p in eng.state.bmanager.pools.values():
         p.check_errors()
         assert sorted(p.seq_len) == sorted(r.seq for r in reqs)
+    BK.reset_worker_state()
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_ring_history_and_the_position_stream_recipe_through_the_backend(graph, monkeypatch):
+    """``OMMX_KV_RING=1`` (the pools and stores keep 104 bf16 rows per request instead of the
+    whole history) with the relidx7 index plane chosen through the serving config.  The two
+    index planes name the same outlier positions, so the dequantised history — and the oracle —
+    is the one of the bitmap recipe."""
+    monkeypatch.setenv("OMMX_KV_RING", "1")
+    recipe = {"outlier_repr": "relidx7"}
+    eng = _Engine(700, recipe=recipe, graph=False, batched=True, batched_graph=graph, max_num_seqs=2)
+    a, b = _Request(8, 420, 520, 1500), _Request(9, 75, 180, 1600)
+    eng.step([a, b], check=True)
+    for s in range(80):
+        eng.step([b, a] if s % 2 else [a, b], check=(s % 10 == 0 or s == 79))
+    pool = next(iter(eng.state.bmanager.pools.values()))
+    assert pool.kv_ring and pool.k_hist.shape[1] == 104 and pool.k_oidx is not None and pool.k_obmp is None
+    for p in eng.state.bmanager.pools.values():
+        p.check_errors()
+    eng = _Engine(700, recipe=recipe, graph=False, batched=False, batched_graph=False)
+    c = _Request(4, 200, 300, 1700)
+    eng.step([c], check=True)
+    for s in range(90):
+        eng.step([c], check=(s % 10 == 0 or s == 89))
+    st = eng.layers[0]._ommx_store_obj
+    assert st.kv_ring and st.k_hist.shape[0] == 104
+    assert eng.state.manager.kv_ring and not eng.state.manager.dead
+    st.check_errors()
     BK.reset_worker_state()
