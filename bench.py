@@ -11,6 +11,7 @@ graphs of 32 consecutive steps (the 32 layers of one model forward; eager launch
 capture fails), so K is rounded up to a multiple of 32.  Prints ONE JSON line.  ``value`` is the p50 over the K timed
 steps at the headline context; ``roofline`` is the split-KV kernel alone (algorithmic bytes
 of the packed planes it must read over its average duration, against 8 TB/s);
+``store`` is the quantize-on-store kernel over the same cache (its own roofline figures);
 ``cpu_baseline`` is the CPU checker (dequantise-then-attend, torch on the host cores) on
 the same workload, a bounded number of runs, used here also for the post-timing parity
 check.
@@ -34,6 +35,7 @@ HBM_PEAK_GBPS = 8000.0
 # (profiles/decode_ctx64k_hbm_traffic.txt); counters cannot be read from inside this script.
 TRAFFIC_BYTES_CTX64K = 74.03e6
 STAGE1_REP = 20
+STORE_REP = 8
 LAYERS = 32                  # decode steps (layers) per graph replay
 H200_P50_US_64K = 563.0      # reference Triton kernel, H200 NVL, B=1 ctx 65536 (other hardware)
 
@@ -120,6 +122,35 @@ def _make_runner(case, splits=None):
     return step, stage1, o, lse, S
 
 
+def _time_store(ctx, kv_heads=8, head_dim=128):
+    """Quantize-on-store kernel over one ctx-token cache (bf16 K and V resident in HBM, serving
+    recipe, identity tables): launches replayed from a graph of STORE_REP, HIP events around each
+    replay.  Algorithmic bytes per (token, kv head): 512 read + 132 written."""
+    import torch
+    from open_ommx_serve_amd.attention.kv_window import WindowSpec
+    from open_ommx_serve_amd.attention.pack import alloc_planes, store_pack_into
+    from open_ommx_serve_amd.synth import synth_kv
+    T = WindowSpec().packed_len(ctx)
+    K, V = synth_kv(T, kv_heads, head_dim, seed=42, sparse_frac=0.005)
+    K, V = K.cuda(), V.cuda()
+    planes = alloc_planes(T // 16, T // 32, kv_heads, head_dim, device="cuda")
+    err = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def rep():
+        for _ in range(STORE_REP):
+            store_pack_into(K, V, planes, err_flag=err)
+    run, mode = _graph_or_eager(rep)
+    _, us = _time_steps(run, 10, 2, per_call=STORE_REP)
+    if int(err.item()):
+        raise RuntimeError(f"store kernel reported error bits {int(err.item())}")
+    k = statistics.mean(us)
+    nbytes = T * kv_heads * (4 * head_dim + 132)
+    gbps = nbytes / (k * 1e-6) / 1e9
+    return {"kernel": "store_pack", "bound": "hbm", "tokens": T, "bytes_per_launch": nbytes,
+            "avg_kernel_us": round(k, 2), "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "launch": mode}
+
+
 def _cpu_reference(case, runs):
     """Dequantise-then-attend on the host cores; (seconds per step list, o, lse)."""
     import torch
@@ -153,6 +184,8 @@ def main() -> int:
                          "all ctx, e.g. --batch 32 --ctx 16384 --ragged")
     ap.add_argument("--no-ladder", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-store", action="store_true",
+                    help="skip the timing of the quantize-on-store kernel (headline workload only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy kernel (3 times), the known-size "
                          "reference that scales the FETCH_SIZE / WRITE_SIZE counters")
@@ -233,6 +266,10 @@ def main() -> int:
     ladder[str(args.ctx)] = {"p50_us": round(p50, 2), "splits": m["S"], "bytes": step_bytes,
                              "hbm_frac": round(step_bytes / (p50 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
 
+    store = None
+    if headline and not args.no_store:
+        store = _time_store(args.ctx)
+
     cpu = None
     parity = None
     if not args.no_cpu_baseline:
@@ -274,6 +311,7 @@ def main() -> int:
                      "avg_kernel_us": round(k1, 3)},
         "cpu_baseline": cpu,
         "parity_after_timing": parity,
+        "store": store,
     }
     print(json.dumps(out))
     return 0
