@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 3   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments */
+#define OMMX_ABI_VERSION 4   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion */
 
 /* step of the INT2 quantisers and the dtype of the k_scale / v_scale planes */
 #define OMMX_SCALE_POW2_INT8  0
@@ -37,6 +37,9 @@ extern "C" {
 #define OMMX_INDEX_BITMAP   0   /* k_index u8[G,H,D,4]: bit p of the frame = position p (codec.py:330-372) */
 #define OMMX_INDEX_RELIDX7  1   /* k_index u8[G,H,D,ceil(7k/8)]: ascending positions, 7 bits each,
                                    least significant bit first (pack.py:128-164) */
+#define OMMX_INDEX_COMBINADIC 2 /* k_index u8[G,H,D,ceil(log2 C(gt,k)/8)]: rank sum_i C(p_i, i) of the ascending
+                                   positions, little endian (pack.py:179-206, codec.py:131-180); accepted by
+                                   ommx_index_convert only: store and decode work on the other two planes */
 
 /* number of floats in the store decision table: 256 pow2 thresholds + 8 FP4 slots */
 #define OMMX_STORE_TABLE_FLOATS 264
@@ -48,6 +51,9 @@ extern "C" {
 #define OMMX_ERR_EXP_RANGE     8   /* scale exponent does not fit the int8 plane */
 /* error bit OR-ed into *err_flag by ommx_ring_write / ommx_tail_gather */
 #define OMMX_ERR_RING_RANGE   16   /* row outside the history (kv_store_ops.py:33-34,52-53) */
+/* error bit OR-ed into *err_flag by ommx_index_convert */
+#define OMMX_ERR_INDEX_PLANE  32   /* a vector that does not name exactly k positions below group_tokens
+                                      (codec.py:173-178 raises ValueError there) */
 
 int ommx_abi_version(void);
 const char* ommx_last_error(void);
@@ -256,6 +262,28 @@ int ommx_merge_states(const float* o_parts, const float* lse_parts, const int32_
                       float* o, float* lse, int P, int R, int D,
                       int64_t op_stride_p, int64_t op_stride_r, int64_t lp_stride_p,
                       int64_t o_stride_r, void* stream);
+
+/*
+ * Bytes per K vector of an outlier index plane, 0 if the combination is not supported
+ * (1..16 outliers, group_tokens <= 128, combinadic ranks of at most 64 bits).  Replaces
+ * combinadic_index_bytes, ommx_gpu_serve/attention/codec.py:131-143, and the plane widths of
+ * pack.py:128-164 (position streams) and codec.py:330-372 (bitmask).
+ */
+int ommx_index_plane_bytes(int index_repr, int group_tokens, int k);
+
+/*
+ * Convert the outlier index plane of K groups between the three encodings (bitmask, position
+ * streams, combinadic rank).  Replaces _pack_combinadic_frames / _unpack_combinadic_frames
+ * (pack.py:179-223), combinadic_to_bitmap (codec.py:239-255) and the plane rewrite of
+ * derive_relidx7_from_combinadic (pack.py:662-699), which run on the host one vector at a time.
+ *   src / dst  u8 [slots, vectors_per_group, bytes(repr)] contiguous, bytes as ommx_index_plane_bytes
+ *   groups     NULL (slots 0..n_groups-1) or int32[n_groups] slots to convert
+ * A vector that does not decode to exactly k distinct positions below group_tokens is written
+ * as zeros and sets OMMX_ERR_INDEX_PLANE in *err_flag (may be NULL).
+ */
+int ommx_index_convert(const uint8_t* src, uint8_t* dst, const int32_t* groups, int n_groups,
+                       int vectors_per_group, int group_tokens, int k, int src_repr, int dst_repr,
+                       int32_t* err_flag, void* stream);
 
 #ifdef __cplusplus
 }

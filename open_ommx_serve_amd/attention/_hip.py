@@ -16,8 +16,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
-ABI_VERSION = 3
-INDEX_BITMAP, INDEX_RELIDX7 = 0, 1
+ABI_VERSION = 4
+INDEX_BITMAP, INDEX_RELIDX7, INDEX_COMBINADIC = 0, 1, 2
 SCALE_POW2_INT8, SCALE_POW2_BF16, SCALE_BF16 = 0, 1, 2
 
 
@@ -28,6 +28,7 @@ def scale_mode(use_pow2: bool, kv_int8_scale: bool) -> int:
         return SCALE_BF16
     return SCALE_POW2_INT8 if kv_int8_scale else SCALE_POW2_BF16
 ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
+ERR_INDEX_PLANE = 32
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -56,6 +57,8 @@ _SIGNATURES = {
     "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
                              _I, _I, _I, _I, _I, _P, _P]),
     "ommx_merge_states": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P]),
+    "ommx_index_plane_bytes": (_I, [_I, _I, _I]),
+    "ommx_index_convert": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]),
     "ommx_tail_gather": (_I, [_P, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P,
                               _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
 }

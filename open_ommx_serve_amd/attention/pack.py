@@ -137,7 +137,21 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
                               or int(t.numel()) < n or t.device != K.device):
             raise ValueError("index tables must be contiguous int32 device tensors of the right length")
     k = int(outliers_per_vector)
-    index_repr, index_plane = _index_plane(planes, outlier_repr, k, gt)
+    combinadic = k > 0 and str(outlier_repr).lower() == "combinadic"
+    if combinadic:
+        # the store kernel writes the flat bitmask into a scratch plane kept beside k_crank;
+        # the ranks of the groups just written come from one conversion launch after it
+        crank = planes.get("k_crank")
+        fb = index_plane_bytes("combinadic", gt, k)
+        if crank is None or int(crank.shape[-1]) != fb:
+            raise ValueError(f"combinadic needs a k_crank plane of {fb} bytes per frame")
+        scratch = planes.get("_k_obmp_scratch")
+        if scratch is None or tuple(scratch.shape[:3]) != tuple(crank.shape[:3]):
+            scratch = torch.zeros(*crank.shape[:3], (gt + 7) // 8, dtype=torch.uint8, device=crank.device)
+            planes["_k_obmp_scratch"] = scratch
+        index_repr, index_plane = _hip.INDEX_BITMAP, scratch
+    else:
+        index_repr, index_plane = _index_plane(planes, outlier_repr, k, gt)
     sel = str(outlier_select).lower()
     if sel not in ("signed", "abs"):
         raise ValueError(f"outlier_select must be signed|abs; got {outlier_select!r}")
@@ -161,6 +175,90 @@ def store_pack_into(K: torch.Tensor, V: torch.Tensor, planes: Dict[str, Any], *,
             planes["v_main"].data_ptr(), planes["v_scale"].data_ptr(), planes["v_zp"].data_ptr(),
             _hip.ptr(err_flag), _hip.current_stream_ptr(K.device))
     _hip.check(rc, "ommx_store_pack")
+    if combinadic and T >= gt:
+        convert_index_plane(index_plane, planes["k_crank"], group_tokens=gt, k=k, src_repr="bitmap",
+                            dst_repr="combinadic", groups=dst_groups, n_groups=T // gt, err_flag=err_flag)
+
+
+_REPR_CODE = {"bitmap": _hip.INDEX_BITMAP, "relidx7": _hip.INDEX_RELIDX7, "combinadic": _hip.INDEX_COMBINADIC}
+
+
+def index_plane_bytes(outlier_repr: str, group_tokens: int, k: int) -> int:
+    """Bytes per K vector of an index plane: ``group_tokens/8`` (bitmap), ``ceil(7k/8)`` (relidx7),
+    ``ceil(log2 C(group_tokens, k) / 8)`` (combinadic; reference ``codec.py:131-143``).  Raises
+    ``NotImplementedError`` for what the library does not convert (more than 16 outliers, ranks
+    wider than 64 bits)."""
+    if int(k) <= 0:
+        return 0
+    n = _hip.load().ommx_index_plane_bytes(_REPR_CODE[str(outlier_repr).lower()], int(group_tokens), int(k))
+    if n <= 0:
+        raise NotImplementedError(f"index plane {outlier_repr!r} with group_tokens={group_tokens}, k={k}")
+    return int(n)
+
+
+def convert_index_plane(src: torch.Tensor, dst: torch.Tensor, *, group_tokens: int, k: int,
+                        src_repr: str, dst_repr: str, groups: Optional[torch.Tensor] = None,
+                        n_groups: Optional[int] = None, err_flag: Optional[torch.Tensor] = None) -> None:
+    """Rewrite the outlier index plane ``src [slots, H, D, bytes]`` in another encoding into
+    ``dst`` (same slots), one launch on the current stream; ``groups`` int32 names the slots to
+    convert (default: the first ``n_groups``, default all).  A vector that does not hold exactly
+    ``k`` positions sets ``ERR_INDEX_PLANE`` in ``err_flag`` and is written as zeros."""
+    gt, k = int(group_tokens), int(k)
+    sb, db = index_plane_bytes(src_repr, gt, k), index_plane_bytes(dst_repr, gt, k)
+    for name, t, nb in (("src", src, sb), ("dst", dst, db)):
+        if t.dtype != torch.uint8 or t.dim() != 4 or int(t.shape[-1]) != nb or not t.is_contiguous():
+            raise ValueError(f"{name} index plane must be contiguous u8 [slots, H, D, {nb}]")
+    if tuple(src.shape[:3]) != tuple(dst.shape[:3]) or src.device != dst.device:
+        raise ValueError("src and dst index planes must cover the same slots on one device")
+    _hip.require_gpu(src.device)
+    if groups is not None:
+        if groups.dtype != torch.int32 or not groups.is_contiguous() or groups.device != src.device:
+            raise ValueError("groups must be a contiguous int32 device tensor")
+        n = int(groups.numel()) if n_groups is None else int(n_groups)
+        if n > int(groups.numel()):
+            raise ValueError("n_groups exceeds the slot list")
+    else:
+        n = int(src.shape[0]) if n_groups is None else int(n_groups)
+        if n > int(src.shape[0]):
+            raise ValueError("n_groups exceeds the plane")
+    with torch.cuda.device(src.device):
+        rc = _hip.load().ommx_index_convert(
+            src.data_ptr(), dst.data_ptr(), _hip.ptr(groups), n, int(src.shape[1]) * int(src.shape[2]),
+            gt, k, _REPR_CODE[str(src_repr).lower()], _REPR_CODE[str(dst_repr).lower()],
+            _hip.ptr(err_flag), _hip.current_stream_ptr(src.device))
+    _hip.check(rc, "ommx_index_convert")
+
+
+def _derive(planes: dict, dst_repr: str) -> dict:
+    if str(planes.get("outlier_repr")) != "combinadic" or planes.get("k_crank") is None:
+        return planes
+    k, gt = int(planes["outliers_per_vector"]), int(planes.get("group_tokens", 32))
+    crank = planes["k_crank"]
+    dev = crank.device if crank.device.type == "cuda" else torch.device("cuda", torch.cuda.current_device())
+    src = crank.to(dev).contiguous()
+    dst = torch.empty(*src.shape[:3], index_plane_bytes(dst_repr, gt, k), dtype=torch.uint8, device=dev)
+    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    convert_index_plane(src, dst, group_tokens=gt, k=k, src_repr="combinadic", dst_repr=dst_repr, err_flag=err)
+    if int(err.item()) & _hip.ERR_INDEX_PLANE:
+        raise ValueError(f"invalid combinadic rank for k={k}, tile={gt}")          # codec.py:173-178
+    out = dict(planes)
+    out["k_oidx" if dst_repr == "relidx7" else "k_obmp"] = dst.to(crank.device)
+    out["outlier_repr"] = dst_repr
+    out["k_field_bytes"] = int(dst.shape[-1]) if dst_repr == "bitmap" else 0
+    out["outlier_repr_storage"] = "combinadic"
+    return out
+
+
+def derive_relidx7_from_combinadic(planes: dict) -> dict:
+    """Combinadic-stored outliers -> a new pack dict with the position-stream plane ``k_oidx`` the
+    decode kernels read; ``k_crank`` stays as the stored form (reference ``pack.py:662-699``, which
+    unranks on the host).  A pack with another index plane is returned unchanged."""
+    return _derive(planes, "relidx7")
+
+
+def derive_bitmap_from_combinadic(planes: dict) -> dict:
+    """Same, to the flat bitmask plane ``k_obmp``."""
+    return _derive(planes, "bitmap")
 
 
 def _index_plane(planes: Dict[str, Any], outlier_repr: str, k: int, gt: int = 32):
@@ -204,6 +302,9 @@ def alloc_planes(num_pages: int, num_group_slots: int, n_kv_heads: int, head_dim
     if k > 0:
         if str(outlier_repr).lower() == "relidx7":      # pack.py:128-164: ceil(7k/8) bytes per frame
             out["k_oidx"] = torch.empty(G, H, D, (7 * k + 7) // 8, dtype=u8, device=dev)
+        elif str(outlier_repr).lower() == "combinadic":  # pack.py:552-557: one rank per frame
+            out["k_crank"] = torch.empty(G, H, D, index_plane_bytes("combinadic", int(group_tokens), k),
+                                         dtype=u8, device=dev)
         else:
             out["k_obmp"] = torch.empty(G, H, D, (int(group_tokens) + 7) // 8, dtype=u8, device=dev)
         out["k_oval"] = torch.empty(G, H, D, (k + 1) // 2, dtype=u8, device=dev)
@@ -224,6 +325,8 @@ def raise_for_store_errors(bits: int) -> None:
         raise ValueError("encode_fp4_e2m1f: non-finite input")               # codec.py:55-57
     if bits & _hip.ERR_EXP_RANGE:
         raise ValueError("KV pack: a scale exponent does not fit the int8 plane")
+    if bits & _hip.ERR_INDEX_PLANE:
+        raise ValueError("outlier index plane: a vector does not name exactly k positions")
 
 
 def ommx_pack_kv_canonical_block(
@@ -284,8 +387,9 @@ def ommx_pack_kv_canonical_block(
         raise ValueError(f"v_format must be i2|bf16; got {v_format!r}")
 
     unsupported = []
-    if k > 0 and repr_l not in ("bitmap", "relidx7"):
-        unsupported.append(f"outlier_repr={repr_l!r}")
+    if 0 < k <= 16 and repr_l == "combinadic" and \
+            _hip.load().ommx_index_plane_bytes(_hip.INDEX_COMBINADIC, gt, k) <= 0:
+        unsupported.append(f"combinadic ranks wider than 64 bits (group_tokens={gt}, k={k})")
     if str(outlier_select).lower() not in ("signed", "abs"):
         unsupported.append(f"outlier_select={outlier_select!r}")
     if k > 16:
@@ -332,7 +436,11 @@ def ommx_pack_kv_canonical_block(
     out = {name: _to(planes[name]) for name in (
         "k_base", "k_scale", "k_zp", "k_oidx", "k_oval", "k_crank", "k_obmp",
         "k_fp4_mapscale", "k_fp4_mapcenter")}
-    out["k_field_bytes"] = (gt + 7) // 8 if (k > 0 and repr_l == "bitmap") else 0    # pack.py:468,568
+    out["k_field_bytes"] = 0                                                      # pack.py:468,557,568
+    if k > 0 and repr_l == "bitmap":
+        out["k_field_bytes"] = (gt + 7) // 8
+    elif k > 0 and repr_l == "combinadic":
+        out["k_field_bytes"] = int(planes["k_crank"].shape[-1])
     out.update({name: _to(planes[name]) for name in ("v_main", "v_scale", "v_zp")})
     out.update(
         req_to_token=torch.arange(pages, dtype=torch.int32, device=device).reshape(1, pages),
@@ -348,4 +456,5 @@ def ommx_pack_kv_canonical_block(
 
 __all__ = ["CANONICAL_GROUP_TOKENS", "CANONICAL_GROUP_CHANNELS", "OUTLIER_REPRS",
            "ommx_pack_kv_canonical_block", "store_pack_into", "alloc_planes",
-           "measure_store_table", "store_table", "raise_for_store_errors"]
+           "measure_store_table", "store_table", "raise_for_store_errors", "index_plane_bytes",
+           "convert_index_plane", "derive_relidx7_from_combinadic", "derive_bitmap_from_combinadic"]

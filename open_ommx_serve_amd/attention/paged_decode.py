@@ -179,8 +179,6 @@ def ommx_paged_decode_attention_canonical(
         raise ValueError("kv_outlier_map=True requires k_fp4_mapscale + k_fp4_mapcenter planes.")
 
     unsupported = []
-    if k > 0 and combinadic_read:
-        unsupported.append("combinadic outlier index plane")
     if k > 16:
         unsupported.append("more than 16 outliers per vector")
     # int8 exponent planes (kv_int8_scale) or the steps themselves as bf16 (paged_decode.py:1846-1855)
@@ -197,6 +195,22 @@ def ommx_paged_decode_attention_canonical(
     if unsupported:
         raise NotImplementedError(
             "the HIP decode kernel implements the serving recipe only; not: " + ", ".join(unsupported))
+    if combinadic_read and k > 0:
+        # The kernels read positions, not ranks: the rank plane is unranked into a position plane
+        # by one launch ahead of the decode (paged_decode.py:969-1010 unranks inside the tile loop
+        # and is 2.3-4.5x slower for it, pack.py:668).  A caller that decodes the same planes step
+        # after step converts once with pack.derive_bitmap_from_combinadic instead.
+        from .pack import convert_index_plane, index_plane_bytes
+        if k_crank.dtype != torch.uint8 or tuple(k_crank.shape[:3]) != tuple(k_scale.shape) \
+                or int(k_crank.shape[-1]) != index_plane_bytes("combinadic", group_tokens, k):
+            raise ValueError("k_crank must be u8 [group_slots, Hkv, D, ceil(log2 C(group_tokens, k) / 8)]")
+        to = "bitmap" if k <= 8 else "relidx7"          # the bitmask read serves up to 8 outliers
+        plane = torch.empty(*k_crank.shape[:3], index_plane_bytes(to, group_tokens, k), dtype=torch.uint8,
+                            device=k_crank.device)
+        convert_index_plane(k_crank.contiguous(), plane, group_tokens=group_tokens, k=k,
+                            src_repr="combinadic", dst_repr=to)
+        bitmap_read = to == "bitmap"
+        k_obmp, k_oidx = (plane, k_oidx) if bitmap_read else (k_obmp, plane)
     # which index plane the kernels read (paged_decode.py:945-968 bitmap, :843-913 relidx7)
     k_index, index_repr = (k_obmp, _hip.INDEX_BITMAP) if bitmap_read else (k_oidx, _hip.INDEX_RELIDX7)
     if k > 0 and (k_index.dtype != torch.uint8 or tuple(k_index.shape[:3]) != tuple(k_scale.shape)

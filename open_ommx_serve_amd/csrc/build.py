@@ -25,6 +25,7 @@ SOURCES = {
     "ommx_combine.hip": [],
     "ommx_ring.hip": [],
     "ommx_merge.hip": [],
+    "ommx_index.hip": [],
     "ommx_capi.hip": [],
 }
 COMMON = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}",

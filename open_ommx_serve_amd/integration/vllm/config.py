@@ -146,11 +146,10 @@ def resolve_serving_config(*, head_dim: Optional[int] = None, n_q_heads: Optiona
     if cfg.combinadic_read and cfg.outlier_repr != "combinadic":
         raise ValueError("OMMX_ATTN_COMBINADIC_READ=1 needs OMMX_ATTN_OUTLIER_REPR=combinadic: the "
                          f"store allocates no k_crank plane under outlier_repr={cfg.outlier_repr!r}")
-    # The reference refuses the bitmap plane above 8 outliers because its kernel stages a
-    # group's nibbles in one int32 (config.py:458-465); the kernels here read up to 16.
-    if cfg.resolved_bitmap_read() and cfg.outliers_per_vector > 16:
-        raise ValueError(f"outlier_repr=bitmap serves at most 16 outliers per vector; got "
-                         f"{cfg.outliers_per_vector}")
+    if cfg.resolved_bitmap_read() and cfg.outliers_per_vector > 8:
+        raise ValueError(f"outlier_repr=bitmap cannot serve outliers_per_vector={cfg.outliers_per_vector}: "
+                         "the bitmask read is limited to k <= 8 (config.py:458-465).  Set "
+                         "OMMX_ATTN_OUTLIER_REPR=relidx7, or lower OMMX_ATTN_OUTLIERS / OMMX_OUTLIER_PERCENT.")
     return cfg
 
 

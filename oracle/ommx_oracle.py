@@ -19,6 +19,10 @@ Parity status of each function (what pins it, besides reading):
   relidx7_pack / relidx7_unpack  closed form (7-bit LSB-first stream) against big-integer
                                arithmetic and hand-computed bytes; positions equal the
                                bitmap's for the same input     (tests/test_oracle_codec.py)
+  combinadic_pack / _unpack    the combinatorial number system: every k-subset of a small set
+                               enumerated in colexicographic order takes the ranks 0, 1, 2 ...
+                               in turn; first / last subset, a hand-computed rank, field widths
+                               of the reference's recipes      (tests/test_oracle_pins.py)
   pow2_exponent                rule 2^rint(log2(x)) incl. exact-tie vectors
   select_outliers_signed       brute-force rank counting on small vectors with ties
   select_outliers_abs          the same, on magnitudes
@@ -148,11 +152,62 @@ def relidx7_unpack(plane: torch.Tensor, k: int) -> torch.Tensor:
     return (bits * (1 << torch.arange(7, dtype=torch.int64))).sum(-1)
 
 
+def combinadic_bytes(k: int, n: int = GROUP_TOKENS) -> int:
+    """Bytes of one combinadic rank: ``ceil(log2 C(n, k))`` bits, at least one.
+    codec.py:131-143."""
+    if k <= 0 or k >= n:
+        return 0
+    return (max(1, (math.comb(n, k) - 1).bit_length()) + 7) // 8
+
+
+def combinadic_pack(pos: torch.Tensor, n: int = GROUP_TOKENS) -> torch.Tensor:
+    """Ascending distinct positions ``[..., k]`` -> ``[..., combinadic_bytes]`` little-endian
+    ranks: the rank of ``p_1 < ... < p_k`` is ``sum_i C(p_i, i)`` (the combinatorial number
+    system; codec.py:146-158 sums ``C(c_j, k-j)`` over the descending order, the same terms).
+    Python integers, so no width limit.  pack.py:179-206."""
+    k = int(pos.shape[-1])
+    nb = combinadic_bytes(k, n)
+    flat = pos.reshape(-1, k).tolist()
+    out = torch.zeros(len(flat), nb, dtype=torch.uint8)
+    for r, cols in enumerate(flat):
+        cols = sorted(int(c) for c in cols)
+        if len(set(cols)) != k or cols[0] < 0 or cols[-1] >= n:
+            raise ValueError("combinadic_pack: positions must be distinct and inside the group")
+        rank = sum(math.comb(c, i + 1) for i, c in enumerate(cols))
+        out[r] = torch.tensor(list(rank.to_bytes(nb, "little")), dtype=torch.uint8)
+    return out.reshape(*pos.shape[:-1], nb)
+
+
+def combinadic_unpack(plane: torch.Tensor, k: int, n: int = GROUP_TOKENS) -> torch.Tensor:
+    """Ranks ``[..., bytes]`` -> ascending positions ``[..., k]`` by the greedy inverse: for
+    ``i = k .. 1`` take the largest ``c`` with ``C(c, i) <= rest``.  codec.py:161-180,
+    pack.py:209-223."""
+    flat = plane.reshape(-1, int(plane.shape[-1])).tolist()
+    out = torch.zeros(len(flat), k, dtype=torch.int64)
+    for r, bs in enumerate(flat):
+        rem = int.from_bytes(bytes(bs), "little")
+        cols = []
+        for i in range(k, 0, -1):
+            c = n - 1
+            while c >= i - 1 and math.comb(c, i) > rem:
+                c -= 1
+            if c < i - 1:
+                raise ValueError("invalid combinadic rank")
+            rem -= math.comb(c, i)
+            cols.append(c)
+        if rem != 0 or len(set(cols)) != k:
+            raise ValueError("invalid combinadic rank")
+        out[r] = torch.tensor(sorted(cols), dtype=torch.int64)
+    return out.reshape(*plane.shape[:-1], k)
+
+
 def outlier_positions(planes: Dict[str, object], gsel, k: int, gt: int = GROUP_TOKENS) -> torch.Tensor:
     """Ascending outlier positions ``[n, H, D, k]`` of the group slots ``gsel`` from whichever
     index plane the pack carries (both decode to the same positions, pack.py:323-326)."""
     if str(planes.get("outlier_repr", "bitmap")).lower() == "relidx7":
         return relidx7_unpack(planes["k_oidx"][gsel], k)
+    if str(planes.get("outlier_repr", "bitmap")).lower() == "combinadic":
+        return combinadic_unpack(planes["k_crank"][gsel], k, gt)
     return bitmap_unpack(planes["k_obmp"][gsel], k, gt)
 
 
@@ -272,9 +327,9 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
     code = torch.round((gw - zp) / scale).clamp(0, 3).to(torch.int64)
 
     repr_l = str(outlier_repr).lower()
-    if repr_l not in ("bitmap", "relidx7"):
-        raise ValueError("outlier_repr must be bitmap or relidx7")
-    planes: Dict[str, object] = {"k_oidx": None}
+    if repr_l not in ("bitmap", "relidx7", "combinadic"):
+        raise ValueError("outlier_repr must be bitmap, relidx7 or combinadic")
+    planes: Dict[str, object] = {"k_oidx": None, "k_crank": None}
     if k > 0:
         if kv_outlier_map:                                  # pack.py:486-498
             omn, omx = _masked_min_max(gw, omask)
@@ -294,6 +349,9 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         oval = oval.permute(2, 0, 1, 3).contiguous()
         if repr_l == "bitmap":                              # pack.py:559-573
             planes["k_obmp"] = bitmap_pack(pos, gt)
+        elif repr_l == "combinadic":                        # pack.py:552-557
+            planes["k_obmp"] = None
+            planes["k_crank"] = combinadic_pack(pos, gt)
         else:
             planes["k_obmp"] = None
             planes["k_oidx"] = relidx7_pack(pos)
@@ -343,7 +401,8 @@ def _finish_planes(planes: Dict[str, object], v: Dict[str, object]) -> Dict[str,
     """Identity tables and the metadata keys of pack.py:628-654."""
     gt, k = v["gt"], v["k"]
     planes.update(
-        k_crank=None, k_field_bytes=(gt + 7) // 8 if (k > 0 and v["repr_l"] == "bitmap") else 0,
+        k_field_bytes=((gt + 7) // 8 if v["repr_l"] == "bitmap" else
+                       combinadic_bytes(k, gt) if v["repr_l"] == "combinadic" else 0) if k > 0 else 0,
         req_to_token=torch.arange(v["pages"], dtype=torch.int32).reshape(1, v["pages"]),
         req_to_group=torch.arange(v["G"], dtype=torch.int32).reshape(1, v["G"]),
         head_dim=v["D"], n_kv_heads=v["H"], num_tokens=v["T"], n_groups=v["G"], page_size=int(v["page_size"]),

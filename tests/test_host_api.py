@@ -33,7 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     for n in names:
         assert getattr(raw, n) is not None, n
     assert set(_hip.exported_symbols()) == set(names)
-    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 3
+    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 4
 
 
 def test_default_decision_table_is_the_exact_arithmetic_one():
@@ -116,8 +116,9 @@ def test_pack_argument_errors_match_the_reference():
         P(K, K, **{**good, "outliers_per_vector": 33})
     with pytest.raises(ValueError):
         P(K, K, **{**good, "v_format": "fp8"})
-    with pytest.raises(NotImplementedError):
-        P(K, K, **{**good, "outlier_repr": "combinadic"})
+    with pytest.raises(NotImplementedError, match="64 bits"):      # C(128, 16) does not fit a 64-bit rank
+        P(torch.zeros(128, 2, 64), torch.zeros(128, 2, 64),
+          **{**good, "outlier_repr": "combinadic", "group_tokens": 128, "outliers_per_vector": 16})
     with pytest.raises(NotImplementedError):
         P(K, K, **{**good, "scale_dtype": torch.float16})
     with pytest.raises(NotImplementedError):
@@ -178,9 +179,9 @@ def test_decode_argument_errors_precede_any_launch():
     with pytest.raises(ValueError, match="contiguous"):
         bad = list(args); bad[6] = args[6][:, ::2]
         D(*bad, **{**kw, "page_size": 8})
-    with pytest.raises(NotImplementedError, match="serving recipe"):
+    with pytest.raises(ValueError, match="k_crank must be"):          # the rank plane's own shape check
         D(*args, **{**kw, "combinadic_read": True, "bitmap_read": False,
-                    "k_crank": torch.zeros(2, 2, 64, 3, dtype=torch.uint8)})
+                    "k_crank": torch.zeros(2, 2, 64, 4, dtype=torch.uint8)})
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="no CPU fallback"):
             D(*args, **kw)

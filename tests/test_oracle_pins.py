@@ -165,6 +165,51 @@ def test_relidx7_pack_carries_the_same_positions_and_values_as_the_bitmap_pack()
     assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
 
 
+def test_combinadic_ranks_are_the_combinatorial_number_system():
+    """Pins independent of the formula: the k-subsets of a small set, enumerated in
+    colexicographic order (compare the largest elements first), take the ranks 0, 1, 2, ... in
+    turn - so the map is a bijection onto [0, C(n, k)); the first subset ranks 0 and the last
+    C(n, k) - 1; one rank worked by hand; the plane widths of the reference's recipes."""
+    import itertools
+    for n, k in ((8, 3), (10, 4), (7, 1), (9, 8)):
+        subsets = sorted(itertools.combinations(range(n), k), key=lambda c: tuple(reversed(c)))
+        assert len(subsets) == math.comb(n, k)
+        planes = O.combinadic_pack(torch.tensor(subsets), n)
+        nb = planes.shape[-1]
+        ranks = [int.from_bytes(bytes(r), "little") for r in planes.tolist()]
+        assert ranks == list(range(len(subsets))), (n, k)
+        assert torch.equal(O.combinadic_unpack(planes, k, n), torch.tensor(subsets))
+        assert nb == O.combinadic_bytes(k, n) == (max(1, (len(subsets) - 1).bit_length()) + 7) // 8
+    # {1, 4, 6}: C(1,1) + C(4,2) + C(6,3) = 1 + 6 + 20
+    assert O.combinadic_pack(torch.tensor([[1, 4, 6]]), 32).tolist() == [[27, 0]]
+    assert O.combinadic_pack(torch.tensor([[6, 1, 4]]), 32).tolist() == [[27, 0]]      # order is irrelevant
+    last = torch.arange(26, 32).reshape(1, 6)
+    assert int.from_bytes(bytes(O.combinadic_pack(last, 32)[0].tolist()), "little") == 906192 - 1
+    # widths: 32 choose 6 needs 20 bits, 128 choose 10 needs 48 (codec.py:131-143)
+    assert (O.combinadic_bytes(6, 32), O.combinadic_bytes(10, 128), O.combinadic_bytes(3, 32),
+            O.combinadic_bytes(16, 32), O.combinadic_bytes(0, 32)) == (3, 6, 2, 4, 0)
+    with pytest.raises(ValueError):
+        O.combinadic_unpack(torch.tensor([[0xD0, 0xD3, 0x0D]], dtype=torch.uint8), 6, 32)   # = C(32, 6)
+    with pytest.raises(ValueError):
+        O.combinadic_pack(torch.tensor([[1, 1, 2]]), 32)
+
+
+def test_combinadic_pack_carries_the_same_positions_as_the_bitmap_pack():
+    from open_ommx_serve_amd.synth import synth_kv
+    K, V = synth_kv(128, 2, 64, 78, sparse_frac=0.02)
+    a = O.pack_kv(K, V, outlier_repr="bitmap")
+    c = O.pack_kv(K, V, outlier_repr="combinadic")
+    assert c["k_obmp"] is None and c["k_oidx"] is None and a["k_crank"] is None
+    assert c["k_crank"].shape == (4, 2, 64, 3) and c["k_field_bytes"] == 3
+    assert torch.equal(O.combinadic_unpack(c["k_crank"], 6), O.bitmap_unpack(a["k_obmp"], 6))
+    for n in ("k_base", "k_scale", "k_zp", "k_oval", "k_fp4_mapscale", "k_fp4_mapcenter",
+              "v_main", "v_scale", "v_zp"):
+        assert torch.equal(a[n], c[n]), n
+    Ka, _ = O.dequant_kv(a)
+    Kc, _ = O.dequant_kv(c)
+    assert torch.equal(Ka, Kc)
+
+
 def test_base_shared_outliers_hand_built_vector():
     """kv_outlier_map=False (pack.py:502-506, dequant :756-757), every stored value derived on
     paper.  Channel 0 over 32 tokens: base lanes 0, 1, 2, 3 repeating -> min 0, max 3, scale
