@@ -29,6 +29,32 @@ constexpr Binom make_binom() {
 }
 __device__ const Binom kBinom = make_binom();
 
+// 128-bit values as two named halves: a dynamically indexed two-element array would live in
+// scratch memory
+struct U128 { uint64_t lo, hi; };
+__device__ __forceinline__ void or_shifted(U128& v, uint64_t x, int bit) {     // v |= x << bit
+    if (bit < 64) {
+        v.lo |= x << bit;
+        if (bit > 0) v.hi |= x >> (64 - bit);
+    } else {
+        v.hi |= x << (bit - 64);
+    }
+}
+__device__ __forceinline__ uint32_t bits_at(const U128& v, int bit) {         // low 32 bits of v >> bit
+    if (bit >= 64) return static_cast<uint32_t>(v.hi >> (bit - 64));
+    uint64_t r = v.lo >> bit;
+    if (bit > 32) r |= v.hi << (64 - bit);
+    return static_cast<uint32_t>(r);
+}
+__device__ __forceinline__ U128 load_bytes(const uint8_t* s, int n) {
+    U128 v{0, 0};
+    for (int i = 0; i < n; ++i) or_shifted(v, s[i], 8 * i);
+    return v;
+}
+__device__ __forceinline__ void store_bytes(uint8_t* d, int n, const U128& v) {
+    for (int i = 0; i < n; ++i) d[i] = static_cast<uint8_t>(bits_at(v, 8 * i));
+}
+
 struct IndexArgs {
     const uint8_t* src;
     uint8_t* dst;
@@ -38,6 +64,14 @@ struct IndexArgs {
 };
 
 __global__ void __launch_bounds__(256) index_convert_kernel(IndexArgs a) {
+    // the binomials this launch can touch, C(c, i) for c < group_tokens and i <= k, staged in LDS:
+    // the unranking loop reads them at lane-dependent indices
+    __shared__ uint64_t tab[MAX_POS * (MAX_K + 1)];
+    const int tw = a.k + 1;
+    if (a.src_repr == OMMX_INDEX_COMBINADIC || a.dst_repr == OMMX_INDEX_COMBINADIC) {
+        for (int e = threadIdx.x; e < a.gt * tw; e += blockDim.x) tab[e] = kBinom.c[e / tw][e % tw];
+        __syncthreads();
+    }
     const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= static_cast<int64_t>(a.n_groups) * a.vecs) return;
     const int gi = static_cast<int>(t / a.vecs);
@@ -46,35 +80,34 @@ __global__ void __launch_bounds__(256) index_convert_kernel(IndexArgs a) {
     const uint8_t* s = a.src + vec * a.src_bytes;
     uint8_t* d = a.dst + vec * a.dst_bytes;
     // ---- positions of the vector as a 128-bit occupancy mask ------------------------
-    uint64_t occ[2] = {0, 0};
+    U128 occ{0, 0};
     bool bad = false;
+    const U128 w = load_bytes(s, a.src_bytes);
     if (a.src_repr == OMMX_INDEX_BITMAP) {
-        for (int i = 0; i < a.src_bytes; ++i) occ[i >> 3] |= static_cast<uint64_t>(s[i]) << (8 * (i & 7));
+        occ = w;
     } else if (a.src_repr == OMMX_INDEX_RELIDX7) {
-        uint64_t w[2] = {0, 0};
-        for (int i = 0; i < a.src_bytes; ++i) w[i >> 3] |= static_cast<uint64_t>(s[i]) << (8 * (i & 7));
         for (int i = 0; i < a.k; ++i) {
-            const int bit = 7 * i;
-            uint64_t f = w[bit >> 6] >> (bit & 63);
-            if ((bit & 63) > 57) f |= w[1] << (64 - (bit & 63));
-            const int p = static_cast<int>(f & 127u);
+            const int p = static_cast<int>(bits_at(w, 7 * i) & 127u);
             if (p >= a.gt) bad = true;
-            else occ[p >> 6] |= 1ull << (p & 63);
+            else or_shifted(occ, 1, p);
         }
-    } else {   // combinadic rank: greedy unranking, largest position first
-        uint64_t rem = 0;
-        for (int i = 0; i < a.src_bytes; ++i) rem |= static_cast<uint64_t>(s[i]) << (8 * i);
-        int c = a.gt - 1;
-        for (int i = a.k; i >= 1 && !bad; --i) {
-            while (c >= i - 1 && kBinom.c[c][i] > rem) --c;
-            if (c < i - 1) { bad = true; break; }
-            rem -= kBinom.c[c][i];
-            occ[c >> 6] |= 1ull << (c & 63);
-            --c;
+    } else {   // combinadic rank (at most 64 bits): greedy unranking, largest position first
+        // One pass down the positions with the level i as lane state (every lane makes the same
+        // group_tokens steps): position c is taken at level i iff C(c, i) still fits the rest,
+        // which is the largest such c below the position taken before it.
+        uint64_t rem = w.lo;
+        int i = a.k;
+        for (int c = a.gt - 1; c >= 0; --c) {
+            const uint64_t b = tab[c * tw + i];
+            if (i >= 1 && b <= rem) {
+                rem -= b;
+                or_shifted(occ, 1, c);
+                --i;
+            }
         }
-        if (rem != 0) bad = true;
+        if (rem != 0 || i != 0) bad = true;
     }
-    if (__popcll(occ[0]) + __popcll(occ[1]) != a.k) bad = true;   // a vector holds exactly k outliers
+    if (__popcll(occ.lo) + __popcll(occ.hi) != a.k) bad = true;   // a vector holds exactly k outliers
     if (bad) {
         if (a.err) atomicOr(a.err, OMMX_ERR_INDEX_PLANE);
         for (int i = 0; i < a.dst_bytes; ++i) d[i] = 0;
@@ -82,27 +115,22 @@ __global__ void __launch_bounds__(256) index_convert_kernel(IndexArgs a) {
     }
     // ---- write the destination plane ---------------------------------------------------
     if (a.dst_repr == OMMX_INDEX_BITMAP) {
-        for (int i = 0; i < a.dst_bytes; ++i) d[i] = static_cast<uint8_t>(occ[i >> 3] >> (8 * (i & 7)));
+        store_bytes(d, a.dst_bytes, occ);
         return;
     }
-    uint64_t out[2] = {0, 0};
+    U128 out{0, 0};
     int i = 0;
     for (int half = 0; half < 2; ++half) {
-        uint64_t m = occ[half];
+        uint64_t m = half ? occ.hi : occ.lo;
         while (m) {
             const int p = 64 * half + __builtin_ctzll(m);
             m &= m - 1;
-            if (a.dst_repr == OMMX_INDEX_RELIDX7) {
-                const int bit = 7 * i;
-                out[bit >> 6] |= static_cast<uint64_t>(p) << (bit & 63);
-                if ((bit & 63) > 57) out[1] |= static_cast<uint64_t>(p) >> (64 - (bit & 63));
-            } else {
-                out[0] += kBinom.c[p][i + 1];
-            }
+            if (a.dst_repr == OMMX_INDEX_RELIDX7) or_shifted(out, static_cast<uint64_t>(p), 7 * i);
+            else out.lo += tab[p * tw + i + 1];
             ++i;
         }
     }
-    for (int b = 0; b < a.dst_bytes; ++b) d[b] = static_cast<uint8_t>(out[b >> 3] >> (8 * (b & 7)));
+    store_bytes(d, a.dst_bytes, out);
 }
 
 // bytes per vector of an index plane; 0 = unsupported
