@@ -509,10 +509,11 @@ class MultiSeqKVPool:
         return {k: (v[:B] if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
 
     def _bundle(self, sel: torch.Tensor, b_seq: torch.Tensor, b_tail: torch.Tensor,
-                kt: torch.Tensor, vt: torch.Tensor, max_seq_len: int) -> dict:
+                kt: torch.Tensor, vt: torch.Tensor, max_seq_len: int, tables=None) -> dict:
         planes = dict(self.pool_planes())
-        planes["req_to_token"] = self._req_to_token.index_select(0, sel)
-        planes["req_to_group"] = self._req_to_group.index_select(0, sel)
+        if tables is None:
+            tables = (self._req_to_token.index_select(0, sel), self._req_to_group.index_select(0, sel))
+        planes["req_to_token"], planes["req_to_group"] = tables
         return {
             "planes": planes, "k_tail": kt, "v_tail": vt,
             "b_tail_len": b_tail, "b_seq_len": b_seq,
@@ -531,16 +532,18 @@ class MultiSeqKVPool:
         return self._bundle(sel, b_seq_len, b_tail_len, kt, vt, max_seq_len)
 
     def decode_inputs_seq(self, sel: torch.Tensor, seq: torch.Tensor, b_seq_len: torch.Tensor,
-                          b_tail_len: torch.Tensor, max_seq_len: int) -> dict:
+                          b_tail_len: torch.Tensor, max_seq_len: int, tables=None) -> dict:
         """Decode bundle from caller-owned fixed buffers that hold the pool slots (``sel``,
         int64 ``[B]``) and the CURRENT sequence lengths (``seq``, int64 ``[B]``): the gather
         launch derives the tail positions and writes ``b_seq_len`` / ``b_tail_len`` (int32
         ``[B]``).  Device-only work; the reference's counterpart takes a host-filled ``[B, T]``
-        position matrix (kv_pool.py:886-936)."""
+        position matrix (kv_pool.py:886-936).  ``tables``: the ``(req_to_token, req_to_group)`` rows
+        of ``sel`` when the caller already holds them (pools of one geometry share them: every
+        layer of a model), else they are selected here."""
         B = int(sel.shape[0])
         d = self._decode_buffers(B)
         self._gather(d["kt"], d["vt"], seq=seq, slots=sel, b_tail=b_tail_len, b_seq=b_seq_len)
-        return self._bundle(sel, b_seq_len, b_tail_len, d["kt"], d["vt"], max_seq_len)
+        return self._bundle(sel, b_seq_len, b_tail_len, d["kt"], d["vt"], max_seq_len, tables)
 
     def decode_inputs_batched(self, slots: Sequence[int]) -> dict:
         """Decode bundle for ``slots`` from the host sequence lengths (kv_pool.py:938-1013):

@@ -479,8 +479,11 @@ class OMMXCanonicalImpl(_ImplBase):
         if pool is None:
             raise RuntimeError("[ommx] batched decode before any write reached this layer's pool")
         B = int(mgr.cur_B)
+        # every layer's pool has the same slot geometry: the page / group table rows of this
+        # step's slots are selected by the first layer that runs and shared by the others
         bundle = pool.decode_inputs_seq(mgr.b_sel[:B], mgr.b_cur_seq[:B], mgr.b_seq_len[:B],
-                                        mgr.b_tail_len[:B], mgr.max_seq_len)
+                                        mgr.b_tail_len[:B], mgr.max_seq_len, tables=mgr.step_tables)
+        mgr.step_tables = (bundle["req_to_token"], bundle["req_to_group"])
         self._decode(layer, q[:B], out, bundle, mgr.max_seq_len)
         _STATE.fires["batched"] += 1
 

@@ -310,6 +310,7 @@ class OMMXBatchedStepManager:
         self.b_seq_len = torch.zeros(cap, dtype=torch.int32, device=dev)
         self.b_tail_len = torch.zeros(cap, dtype=torch.int32, device=dev)
         self.cur_B = 0
+        self.step_tables = None
         self.capturing = False
         self._key_to_slot: Dict[int, int] = {}
         self._free_slots: List[int] = list(range(self.num_seqs))
@@ -341,6 +342,7 @@ class OMMXBatchedStepManager:
         self._free_slots = list(range(self.num_seqs))
         self._keys_are_row_index = False
         self.cur_B = 0
+        self.step_tables = None
 
     # ── host seam ────────────────────────────────────────────────────────────────
 
@@ -380,10 +382,11 @@ class OMMXBatchedStepManager:
         self.is_uniform_decode = bool(
             q_start is not None and len(q_start) == B + 1
             and all(q_start[i + 1] - q_start[i] == 1 for i in range(B)))
-        if B and self.is_uniform_decode:
-            self.planner.plan(seq_lens, self.slots)
-            if self.graph:
-                self._refresh_graph_buffers(seq_lens, self.slots)
+        # (The reference also runs its planner here, every step, for per-slot regroup deltas that
+        # only its own pools read; the pools here count their packed groups themselves, and the
+        # planner's position matrix costs more host time than the rest of the seam.)
+        if B and self.is_uniform_decode and self.graph:
+            self._refresh_graph_buffers(seq_lens, self.slots)
 
     def _refresh_graph_buffers(self, seq_lens: List[int], slots: List[int]) -> None:
         """Advance every pool to this step's lengths, pack what completed, refresh the device
@@ -393,7 +396,7 @@ class OMMXBatchedStepManager:
         means rows nobody wrote would be packed, and the manager stops instead."""
         B = len(seq_lens)
         win = self.window
-        h = self._ctl_host
+        cols: List[int] = []
         for i in range(B):
             r, seq = int(slots[i]), int(seq_lens[i])
             for pool in self.pools.values():
@@ -410,9 +413,12 @@ class OMMXBatchedStepManager:
                 pool.seq_len[r] = seq
                 if win.num_groups(seq) > pool.packed_groups[r]:
                     pool.regroup(r)
-            h[0, i], h[1, i], h[2, i] = r, max(0, seq - 1), seq
+            cols.append(max(0, seq - 1))
         self.cur_B = B
-        self._ctl[:, :B].copy_(h[:, :B], non_blocking=True)
+        self.step_tables = None        # (req_to_token, req_to_group) rows of this step, set by the first layer
+        self._ctl_host[:, :B] = torch.tensor([[int(r) for r in slots], cols, [int(x) for x in seq_lens]],
+                                             dtype=torch.long)
+        self._ctl[:, :B].copy_(self._ctl_host[:, :B], non_blocking=True)
 
     def _seq_lens(self, common: Any) -> List[int]:
         lst = _first_field(common, _SEQ_FIELDS)
