@@ -364,7 +364,7 @@ def test_store_refuses_nonfinite_and_bad_arguments():
     with pytest.raises(ValueError):
         _hip(K, V, outliers_per_vector=33)
     with pytest.raises(NotImplementedError):
-        _hip(K, V, outlier_repr="combinadic")
+        _hip(K, V, outliers_per_vector=17, outlier_repr="relidx7")
     _hip(K, V)                                     # and a good call still works afterwards
 
 
