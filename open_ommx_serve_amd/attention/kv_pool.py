@@ -30,7 +30,7 @@ import torch
 from . import _hip
 from .kv_store_ops import gather_tails, ring_slot, write_tokens
 from .kv_window import CANONICAL_GROUP_TOKENS, WindowSpec
-from .pack import raise_for_store_errors, store_pack_into
+from .pack import index_plane_bytes, raise_for_store_errors, store_pack_into
 
 _FALSE = {"0", "false", "off", "no"}
 
@@ -59,8 +59,8 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
     bad = []
     if str(v_format).lower() != "i2":
         bad.append(f"v_format={v_format!r}")
-    if k > 0 and str(outlier_repr).lower() not in ("bitmap", "relidx7"):
-        bad.append(f"outlier_repr={outlier_repr!r}")
+    if str(outlier_repr).lower() == "combinadic" and k > 8:
+        bad.append("combinadic ranks with more than 8 outliers (their decode twin is the bitmask plane)")
     if k > 0 and str(outlier_select).lower() not in ("signed", "abs"):
         bad.append(f"outlier_select={outlier_select!r}")
     if scale_dtype != torch.bfloat16:
@@ -70,7 +70,7 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
     if bad:
         raise NotImplementedError(
             "the HIP KV store implements the serving recipe and its near variants only (i2f4, "
-            "signed or abs selection, bitmap or relidx7 index plane, power-of-two or plain bf16 steps, "
+            "signed or abs selection, bitmap, relidx7 or combinadic index plane, power-of-two or plain bf16 steps, "
             "dedicated or base-shared FP4 outliers, bf16 zero points, 0..16 outliers); "
             "unsupported: " + ", ".join(bad))
 
@@ -160,6 +160,13 @@ class MultiSeqKVPool:
             if self.outlier_repr == "relidx7":
                 self.k_obmp = None
                 self.k_oidx = z(self.G_cap, self.H, self.D, (7 * self.k + 7) // 8, dtype=torch.uint8, device=dev)
+            elif self.outlier_repr == "combinadic":
+                # The ranks are the stored form (pack.py:552-557).  The store kernel writes the flat
+                # bitmask first and one launch ranks it, so the bitmask plane stays beside the ranks
+                # as their decode-ready twin: the decode kernels read positions, not ranks.
+                self.k_crank = z(self.G_cap, self.H, self.D, index_plane_bytes("combinadic", self.gt, self.k),
+                                 dtype=torch.uint8, device=dev)
+                self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             else:
                 self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             self.k_oval = z(self.G_cap, self.H, self.D, (self.k + 1) // 2, dtype=torch.uint8, device=dev)
@@ -224,6 +231,8 @@ class MultiSeqKVPool:
         return {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
                 "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
                 "k_obmp": self.k_obmp, "k_oidx": self.k_oidx, "k_oval": self.k_oval,
+                "k_crank": self.k_crank,
+                "_k_obmp_scratch": self.k_obmp if self.outlier_repr == "combinadic" else None,
                 "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp}
 
     def _as_rows(self, t: torch.Tensor, what: str) -> torch.Tensor:
@@ -450,7 +459,7 @@ class MultiSeqKVPool:
 
         return {
             "k_base": sel(self.k_base, pidx), "k_scale": sel(self.k_scale, gidx),
-            "k_zp": sel(self.k_zp, gidx), "k_oidx": sel(self.k_oidx, gidx), "k_crank": None,
+            "k_zp": sel(self.k_zp, gidx), "k_oidx": sel(self.k_oidx, gidx), "k_crank": sel(self.k_crank, gidx),
             "k_oval": sel(self.k_oval, gidx), "k_obmp": sel(self.k_obmp, gidx),
             "k_fp4_mapscale": sel(self.k_fp4_mapscale, gidx),
             "k_fp4_mapcenter": sel(self.k_fp4_mapcenter, gidx),

@@ -21,7 +21,7 @@ from . import _hip
 from .kv_pool import _env_flag, check_serving_recipe
 from .kv_store_ops import gather_tail, ring_slot, write_token
 from .kv_window import CANONICAL_GROUP_TOKENS, WindowSpec
-from .pack import raise_for_store_errors, store_pack_into
+from .pack import index_plane_bytes, raise_for_store_errors, store_pack_into
 
 
 class CanonicalKVStore:
@@ -107,6 +107,13 @@ class CanonicalKVStore:
             if self.outlier_repr == "relidx7":
                 self.k_obmp = None
                 self.k_oidx = z(self.G_cap, self.H, self.D, (7 * self.k + 7) // 8, dtype=torch.uint8, device=dev)
+            elif self.outlier_repr == "combinadic":
+                # The ranks are the stored form (pack.py:552-557).  The store kernel writes the flat
+                # bitmask first and one launch ranks it, so the bitmask plane stays beside the ranks
+                # as their decode-ready twin: the decode kernels read positions, not ranks.
+                self.k_crank = z(self.G_cap, self.H, self.D, index_plane_bytes("combinadic", self.gt, self.k),
+                                 dtype=torch.uint8, device=dev)
+                self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             else:
                 self.k_obmp = z(self.G_cap, self.H, self.D, (self.gt + 7) // 8, dtype=torch.uint8, device=dev)
             self.k_oval = z(self.G_cap, self.H, self.D, (self.k + 1) // 2, dtype=torch.uint8, device=dev)
@@ -256,6 +263,8 @@ class CanonicalKVStore:
         return {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
                 "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
                 "k_obmp": self.k_obmp, "k_oidx": self.k_oidx, "k_oval": self.k_oval,
+                "k_crank": self.k_crank,
+                "_k_obmp_scratch": self.k_obmp if self.outlier_repr == "combinadic" else None,
                 "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp}
 
     def _regroup_pack_range(self, g0: int, g1: int) -> None:
@@ -302,7 +311,7 @@ class CanonicalKVStore:
             return None if t is None else t[:n]
 
         out = {"k_base": self.k_base[:P], "k_scale": self.k_scale[:G], "k_zp": self.k_zp[:G],
-               "k_oidx": cut(self.k_oidx, G), "k_crank": None, "k_oval": cut(self.k_oval, G),
+               "k_oidx": cut(self.k_oidx, G), "k_crank": cut(self.k_crank, G), "k_oval": cut(self.k_oval, G),
                "k_obmp": cut(self.k_obmp, G), "k_fp4_mapscale": cut(self.k_fp4_mapscale, G),
                "k_fp4_mapcenter": cut(self.k_fp4_mapcenter, G),
                "v_main": self.v_main[:P], "v_scale": self.v_scale[:P], "v_zp": self.v_zp[:P],
@@ -315,7 +324,7 @@ class CanonicalKVStore:
     def decode_planes_full(self) -> dict:
         """Full-capacity, fixed-address plane dict (kv_store.py:651-676)."""
         out = {"k_base": self.k_base, "k_scale": self.k_scale, "k_zp": self.k_zp,
-               "k_oidx": self.k_oidx, "k_oval": self.k_oval, "k_crank": None, "k_obmp": self.k_obmp,
+               "k_oidx": self.k_oidx, "k_oval": self.k_oval, "k_crank": self.k_crank, "k_obmp": self.k_obmp,
                "k_fp4_mapscale": self.k_fp4_mapscale, "k_fp4_mapcenter": self.k_fp4_mapcenter,
                "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp,
                "req_to_token": self._req_to_token_full, "req_to_group": self._req_to_group_full}

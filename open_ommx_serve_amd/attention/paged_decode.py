@@ -205,10 +205,14 @@ def ommx_paged_decode_attention_canonical(
                 or int(k_crank.shape[-1]) != index_plane_bytes("combinadic", group_tokens, k):
             raise ValueError("k_crank must be u8 [group_slots, Hkv, D, ceil(log2 C(group_tokens, k) / 8)]")
         to = "bitmap" if k <= 8 else "relidx7"          # the bitmask read serves up to 8 outliers
-        plane = torch.empty(*k_crank.shape[:3], index_plane_bytes(to, group_tokens, k), dtype=torch.uint8,
-                            device=k_crank.device)
-        convert_index_plane(k_crank.contiguous(), plane, group_tokens=group_tokens, k=k,
-                            src_repr="combinadic", dst_repr=to)
+        plane = k_obmp if to == "bitmap" else k_oidx
+        if plane is None or plane.dtype != torch.uint8 or tuple(plane.shape) != (
+                *k_crank.shape[:3], index_plane_bytes(to, group_tokens, k)):
+            # no unranked twin came with the ranks (the pool and store classes keep one)
+            plane = torch.empty(*k_crank.shape[:3], index_plane_bytes(to, group_tokens, k),
+                                dtype=torch.uint8, device=k_crank.device)
+            convert_index_plane(k_crank.contiguous(), plane, group_tokens=group_tokens, k=k,
+                                src_repr="combinadic", dst_repr=to)
         bitmap_read = to == "bitmap"
         k_obmp, k_oidx = (plane, k_oidx) if bitmap_read else (k_obmp, plane)
     # which index plane the kernels read (paged_decode.py:945-968 bitmap, :843-913 relidx7)

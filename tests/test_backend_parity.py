@@ -214,21 +214,32 @@ def test_batched_graph_route_replays_from_a_hip_graph():
     BK.reset_worker_state()
 
 
-@pytest.mark.parametrize("graph", [False, True])
-def test_ring_history_and_the_position_stream_recipe_through_the_backend(graph, monkeypatch):
+@pytest.mark.parametrize("graph,outlier_repr", [(False, "relidx7"), (True, "relidx7"), (True, "combinadic")])
+def test_ring_history_and_the_other_index_planes_through_the_backend(graph, outlier_repr, monkeypatch):
     """``OMMX_KV_RING=1`` (the pools and stores keep 104 bf16 rows per request instead of the
-    whole history) with the relidx7 index plane chosen through the serving config.  The two
-    index planes name the same outlier positions, so the dequantised history — and the oracle —
-    is the one of the bitmap recipe."""
+    whole history) with the relidx7 or the combinadic index plane chosen through the serving
+    config.  The index planes name the same outlier positions, so the dequantised history — and
+    the oracle — is the one of the bitmap recipe; the stored ranks are compared with the oracle's."""
     monkeypatch.setenv("OMMX_KV_RING", "1")
-    recipe = {"outlier_repr": "relidx7"}
+    recipe = {"outlier_repr": outlier_repr}
     eng = _Engine(700, recipe=recipe, graph=False, batched=True, batched_graph=graph, max_num_seqs=2)
     a, b = _Request(8, 420, 520, 1500), _Request(9, 75, 180, 1600)
     eng.step([a, b], check=True)
     for s in range(80):
         eng.step([b, a] if s % 2 else [a, b], check=(s % 10 == 0 or s == 79))
     pool = next(iter(eng.state.bmanager.pools.values()))
-    assert pool.kv_ring and pool.k_hist.shape[1] == 104 and pool.k_oidx is not None and pool.k_obmp is None
+    assert pool.kv_ring and pool.k_hist.shape[1] == 104
+    if outlier_repr == "relidx7":
+        assert pool.k_oidx is not None and pool.k_obmp is None and pool.k_crank is None
+    else:
+        assert pool.k_crank.shape[-1] == 3 and pool.k_oidx is None
+        slot = eng.state.bmanager._key_to_slot[a.key]
+        got = pool.request_planes(slot)
+        edge = eng.win.boundary(a.seq)
+        want = O.pack_kv(a.K[0][8:edge], a.V[0][8:edge], outlier_repr="combinadic")
+        assert got["outlier_repr"] == "combinadic" and got["num_tokens"] == edge - 8
+        assert torch.equal(got["k_crank"].cpu(), want["k_crank"])
+        assert torch.equal(got["k_obmp"].cpu(), O.bitmap_pack(O.combinadic_unpack(want["k_crank"], 6)))
     for p in eng.state.bmanager.pools.values():
         p.check_errors()
     eng = _Engine(700, recipe=recipe, graph=False, batched=False, batched_graph=False)

@@ -219,8 +219,11 @@ def test_store_classes_refuse_other_recipes_and_the_cpu():
                 outlier_repr="bitmap", use_pow2=True)
     check_serving_recipe(**good, kv_outlier_map=True, kv_int8_scale=True, group_tokens=32,
                          group_channels=32, scale_dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError, match="combinadic"):
-        MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "outlier_repr": "combinadic"})
+    with pytest.raises(NotImplementedError, match="combinadic"):      # the bitmask twin serves up to 8
+        MultiSeqKVPool(128, 8, 2, 256, device="cpu",
+                       **{**good, "outlier_repr": "combinadic", "outliers_per_vector": 10})
+    check_serving_recipe(**{**good, "outlier_repr": "combinadic"}, kv_outlier_map=True, kv_int8_scale=True,
+                         group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
     check_serving_recipe(**{**good, "outlier_repr": "relidx7"}, kv_outlier_map=True, kv_int8_scale=True,
                          group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError, match="v_format"):
