@@ -151,6 +151,100 @@ def _time_store(ctx, kv_heads=8, head_dim=128):
             "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "launch": mode}
 
 
+def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
+    """One decode step of a serving loop on MultiSeqKVPool (ring history): the new K/V row of every
+    request is written (the launch advances the device sequence counter), the sink + recent rows are
+    gathered with the window arithmetic on the device, then split-KV + combine.  These four launches
+    are one HIP graph; after each replay the host advances its mirror and packs the groups that
+    completed (one store launch, outside the timed replay).  Every request gets the same synthetic
+    rows (the kernels do not care).  Returns the JSON object."""
+    import torch
+    from open_ommx_serve_amd.attention import MultiSeqKVPool, WindowSpec, gather_tails, write_tokens
+    from open_ommx_serve_amd.attention.paged_decode import (auto_num_kv_splits, make_attn_logits,
+                                                            ommx_paged_decode_attention_canonical)
+    from open_ommx_serve_amd.synth import synth_kv, synth_q
+    H, D, B = 8, 128, batch
+    win = WindowSpec()
+    total = steps + warmup + 2
+    pool = MultiSeqKVPool(D, H, num_seqs=B, max_seq_len=ctx + total + 64, window=win, device="cuda",
+                          kv_ring=True, k_format="i2f4", outliers_per_vector=6, outlier_select="signed",
+                          outlier_repr="bitmap", use_pow2=True)
+    K, V = synth_kv(ctx + total, H, D, seed=42, sparse_frac=0.005)
+    Kd, Vd = K.cuda(), V.cuda()
+    for r in range(B):
+        pool.append_block(r, Kd[:ctx], Vd[:ctx])
+    pool.decode_seed_seq_device(range(B))
+    d = pool._decode_buffers(B)
+    pl = pool.pool_planes()
+    newK = torch.zeros(B, H, D, dtype=torch.bfloat16, device="cuda")
+    newV = torch.zeros_like(newK)
+    q = synth_q(B, q_heads, D, 42).cuda()
+    o = torch.empty(B, q_heads, D, dtype=torch.float32, device="cuda")
+    lse = torch.empty(B, q_heads, dtype=torch.float32, device="cuda")
+    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    max_seq = win.packed_len(ctx + total)
+    S = splits or auto_num_kv_splits(max_seq, B, H, n_cu, q_heads // H, mean_seq_len=win.packed_len(ctx))
+    ws = make_attn_logits(B, q_heads, S, D, "cuda")
+
+    def step():
+        write_tokens(pool.k_hist, pool.v_hist, d["seq_dev"], newK, newV, pool._ring_sink, pool._ring_rec,
+                     slots=d["rows"], pos_next=d["seq_dev"], err_flag=pool.err_flag)
+        gather_tails(pool.k_hist, pool.v_hist, d["kt"], d["vt"], pool._ring_sink, pool._ring_rec,
+                     seq=d["seq_dev"], slots=d["sel"], b_tail_len=d["b_tail"], b_seq_len=d["b_seq"],
+                     window_sink=win.sink_tokens, window_recent=win.recent_window,
+                     group_tokens=win.group_tokens, err_flag=pool.err_flag)
+        ommx_paged_decode_attention_canonical(
+            q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"], pl["v_main"], pl["v_scale"],
+            pl["v_zp"], d["kt"], d["vt"], d["b_tail"], o, lse, pl["req_to_token"], pl["req_to_group"],
+            d["b_seq"], sm_scale=D ** -0.5, page_size=win.page_size, k_outliers_per_vector=6,
+            bitmap_read=True, k_obmp=pl["k_obmp"], k_fp4_mapscale=pl["k_fp4_mapscale"],
+            k_fp4_mapcenter=pl["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
+            max_seq_len=max_seq, max_tail_len=pool.max_tail_len, num_kv_splits=S, attn_logits=ws)
+
+    seq0 = d["seq_dev"].clone()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+    torch.cuda.current_stream().wait_stream(stream)
+    d["seq_dev"].copy_(seq0)                      # capture ran no kernel
+    us, packed = [], 0
+    t0 = time.perf_counter()
+    for s in range(warmup + steps):
+        newK.copy_(Kd[ctx + s].unsqueeze(0).expand(B, H, D))
+        newV.copy_(Vd[ctx + s].unsqueeze(0).expand(B, H, D))
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        graph.replay()
+        b.record()
+        packed += pool._advance_host_and_pack(range(B))      # host mirror + pack of completed groups
+        torch.cuda.synchronize()
+        if s == warmup:
+            t0 = time.perf_counter()
+        if s >= warmup:
+            us.append(a.elapsed_time(b) * 1e3)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / max(1, steps - 1)
+    pool.check_errors()
+    if not bool(torch.isfinite(o).all()):
+        raise RuntimeError("pool step produced non-finite output")
+    p50 = statistics.median(us)
+    nbytes = B * (win.packed_len(ctx) * H * 132 + 64 * H * D * 2 * 2)
+    return {"metric": "p50 serving-step us/layer (ring write + tail gather + split-KV + combine)",
+            "value": round(p50, 3), "unit": "us/step/layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(wall_ms, 6), "higher_is_better": False, "scaling": "weak",
+            "vs_baseline": None, "dtype": "u8 planes, bf16 q, f32 accumulate", "data": "synthetic",
+            "config": {"workload": f"MultiSeqKVPool serving step, {q_heads} q / 8 kv heads, d=128, batch {B}, "
+                                   f"ctx {ctx} growing by one token per step, ring history, page 16",
+                       "num_kv_splits": S, "launch": "hip_graph", "bytes_per_step": nbytes,
+                       "hbm_frac_step": round(nbytes / (p50 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                       "groups_packed_between_replays": packed,
+                       "note": "ms_per_step is wall time per step including the host mirror, the pack "
+                               "launches and a synchronisation per step"},
+            "roofline": None, "cpu_baseline": None}
+
+
 def _cpu_reference(case, runs):
     """Dequantise-then-attend on the host cores; (seconds per step list, o, lse)."""
     import torch
@@ -186,6 +280,11 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-store", action="store_true",
                     help="skip the timing of the quantize-on-store kernel (headline workload only)")
+    ap.add_argument("--pool-step", action="store_true",
+                    help="measure the launch-only serving step of MultiSeqKVPool instead: ring write of "
+                         "one new row per request + tail gather + split-KV + combine, replayed from a "
+                         "HIP graph while the host packs completed groups between replays "
+                         "(e.g. --pool-step --batch 8 --ctx 32768 --q-heads 64)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy kernel (3 times), the known-size "
                          "reference that scales the FETCH_SIZE / WRITE_SIZE counters")
@@ -205,6 +304,9 @@ def main() -> int:
         import __graft_entry__
         __graft_entry__.build()
     torch.cuda.set_device(0)
+    if args.pool_step:
+        print(json.dumps(_pool_step(args.batch, args.ctx, args.q_heads, args.steps, args.warmup, args.splits)))
+        return 0
 
     def measure(ctx, steps, warmup):
         lens = [ctx] * args.batch
