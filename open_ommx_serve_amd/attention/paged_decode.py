@@ -37,11 +37,11 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
     behind them so that requests of different length even out (a workgroup is four waves of
     one split; a wave covers one kv head and all of its q heads, so ``q_per_kv`` does not
     enter) -- or only the two resident ones when ``mean_seq_len`` says that the requests are
-    about equally long (at least 0.9 of the longest) and a workgroup would get at most eight
-    64-token steps: little is left to even out then, and a second round of workgroups mostly
-    pays the start-up of a workgroup (about one step) again, 10 % of the whole on short splits;
-    with longer splits the second round still wins, by absorbing the spread of the
-    workgroups' own run times; and eight per unit when the requests differ in length and a
+    about equally long (at least 0.9 of the longest): little is left to even out then, and a
+    second round of workgroups mostly pays the start-up of a workgroup (about one step) again,
+    10 % of the whole on short splits and still 6 % at 16 steps per split (2 x 64K tokens, 8 x 32K
+    with 8 q heads per kv head; 8 x 64K, 16 x 32K and 32 x 16K measure the same either way); and
+    eight per unit when the requests differ in length and a
     workgroup would otherwise run for more than sixteen steps -- but never less than one
     64-token step per split (one 32-token group when even that leaves units idle): a wave's time
     is a fixed part plus ~5 us per step, so while compute units are idle more splits are faster;
@@ -56,7 +56,7 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
     steps = max(1, (int(max_seq_len) + step_tokens - 1) // step_tokens)
     equal = mean_seq_len is not None and float(mean_seq_len) >= 0.9 * float(max_seq_len)
     steps_per_split = (steps + min(want, steps) - 1) // min(want, steps)
-    if equal and steps_per_split <= 8:
+    if equal:
         want = max(1, min(256, (2 * int(n_cu)) // wgs_per_split))
     elif not equal and int(batch) > 1 and steps_per_split > 16:
         # long splits of requests of different length: eight per unit even out better (3-6 %

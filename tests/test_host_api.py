@@ -90,7 +90,7 @@ def test_split_heuristic_bounds():
     # instead of four
     assert auto_num_kv_splits(8128, 32, 8, 256, mean_seq_len=8128) == 8
     assert auto_num_kv_splits(8128, 32, 8, 256) == 16
-    assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=65472) == 16      # long splits: stay
+    assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=65472) == 8       # long splits too
     assert auto_num_kv_splits(65472, 32, 8, 256, mean_seq_len=30000) == 32
     assert auto_num_kv_splits(32704, 8, 8, 256, 8, mean_seq_len=32704) == 32
     assert auto_num_kv_splits(65472, 1, 8, 256, mean_seq_len=65472) == 256
