@@ -26,7 +26,8 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 4   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion */
+#define OMMX_ABI_VERSION 5   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
+                                5: decode without a workspace argument */
 
 /* step of the INT2 quantisers and the dtype of the k_scale / v_scale planes */
 #define OMMX_SCALE_POW2_INT8  0
@@ -199,6 +200,37 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
                         float* lse, int64_t lse_stride_b,
                         int B, int Hq, int Hkv, int D, int num_splits, int group_tokens,
                         float sm_scale, float logit_cap, void* stream);
+
+/*
+ * Whole decode step (split-KV stage, then the combine with the bf16 tail) for callers that
+ * cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference, whose launcher allocates the
+ * workspace `attn_logits` with torch when none is passed (paged_decode.py:3220-3222).
+ * Arguments are those of ommx_decode_splitkv and ommx_decode_combine without the workspace:
+ * the partial states of the splits are kept in a device array built into the library
+ * (2 Mi floats = 8 MiB, held by every GPU the library runs on until the process ends).
+ * Limit: B * Hq * (num_splits + 1) * (D + 1) <= 2097152 floats; larger calls return -1 with a
+ * message naming the limit.  Calls that overlap in time on one GPU share the array and race;
+ * calls on one stream (or otherwise ordered) are safe, and nothing needs clearing between
+ * them.  The call makes no hipMalloc / hipFree and nothing that allocates; its first use on a
+ * device looks the array's device address up (hipGetSymbolAddress), so make that first call
+ * outside stream capture.  seg_group_base is 0 (a segment has no tail to fold in).
+ */
+int ommx_decode_attention_noalloc(
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
+    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
+    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
+    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
+    int table_i64, const int32_t* b_seq_len,
+    const uint16_t* k_tail, const uint16_t* v_tail,
+    int64_t kt_stride_b, int64_t kt_stride_t, int64_t kt_stride_h,
+    int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
+    const int32_t* b_tail_len,
+    float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
+    int group_tokens, int group_channels, int v_bf16, int num_splits,
+    float sm_scale, float logit_cap, int packed_start_offset, void* stream);
 
 /*
  * bf16 residual ring, write side: one new K/V row per request.

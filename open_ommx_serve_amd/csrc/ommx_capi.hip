@@ -211,3 +211,89 @@ extern "C" int ommx_tail_gather(
     if (hipGetLastError() != hipSuccess) { set_error("ommx_tail_gather: launch failed"); return -2; }
     return 0;
 }
+
+// ---- decode without a workspace argument ------------------------------------------------------
+// The partial states of the splits live in a file-scope device array instead of a caller
+// workspace, so the call allocates nothing.  Every GPU the library runs on holds its own copy of
+// the array (at its own address) until the process ends; calls on one GPU share it, so two calls
+// that overlap on one GPU (different streams) race.  Stage 1 writes every (request, head, split)
+// state the combine reads, empty splits included, so nothing has to be cleared between calls.
+#define OMMX_NOALLOC_SCRATCH_FLOATS (2u * 1024u * 1024u)     /* 8 MiB */
+static __device__ __align__(256) float scratch[OMMX_NOALLOC_SCRATCH_FLOATS];
+
+namespace ommx {
+namespace {
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices];        // device address of `scratch` per device, 0 = not asked yet
+}  // namespace
+
+// Device address of this device's copy of `scratch` (the array's name is only a host-side
+// handle: kernels and copies need the address hipGetSymbolAddress returns).
+static float* scratch_on_current_device(const char** why) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        *why = "cannot tell the current device";
+        return nullptr;
+    }
+    float* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p) return p;
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) {
+        (void)hipGetLastError();
+        *why = "hipGetSymbolAddress failed for the scratch array";
+        return nullptr;
+    }
+    p = static_cast<float*>(sym);
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    return p;
+}
+}  // namespace ommx
+
+extern "C" int ommx_decode_attention_noalloc(
+    const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
+    const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
+    const uint16_t* k_ms, const uint16_t* k_mc, const uint8_t* k_index, const uint8_t* k_oval,
+    const uint8_t* v_main, const void* v_scale, const uint16_t* v_zp,
+    const void* req_to_token, int64_t rt_stride, const void* req_to_group, int64_t rg_stride,
+    int table_i64, const int32_t* b_seq_len,
+    const uint16_t* k_tail, const uint16_t* v_tail,
+    int64_t kt_stride_b, int64_t kt_stride_t, int64_t kt_stride_h,
+    int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
+    const int32_t* b_tail_len,
+    float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
+    int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
+    int group_tokens, int group_channels, int v_bf16, int num_splits,
+    float sm_scale, float logit_cap, int packed_start_offset, void* stream) {
+    using namespace ommx;
+    const char* where = "ommx_decode_attention_noalloc";
+    if (B <= 0 || Hq <= 0 || D <= 0 || num_splits < 1 || num_splits > 256) {
+        set_error2(where, "bad shape");
+        return -1;
+    }
+    const int64_t al_stride_s = D + 1, al_stride_h = (int64_t)(num_splits + 1) * al_stride_s,
+                  al_stride_b = (int64_t)Hq * al_stride_h;
+    const int64_t need = (int64_t)B * al_stride_b;
+    if (need > (int64_t)OMMX_NOALLOC_SCRATCH_FLOATS) {
+        g_error = std::string(where) + ": B*Hq*(num_splits+1)*(D+1) = " + std::to_string(need) +
+                  " floats of split states exceed the built-in scratch of " +
+                  std::to_string(OMMX_NOALLOC_SCRATCH_FLOATS) +
+                  " floats (8 MiB); use fewer splits or ommx_decode_splitkv + ommx_decode_combine "
+                  "with a caller workspace";
+        return -1;
+    }
+    const char* why = nullptr;
+    float* ws = scratch_on_current_device(&why);
+    if (!ws) { set_error2(where, why); return -3; }
+    int rc = ommx_decode_splitkv(q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_index,
+                                 k_oval, v_main, v_scale, v_zp, req_to_token, rt_stride, req_to_group,
+                                 rg_stride, table_i64, b_seq_len, ws, al_stride_b, al_stride_h,
+                                 al_stride_s, B, Hq, Hkv, D, page_size, k_outliers, index_repr,
+                                 scale_bf16, group_tokens, group_channels, v_bf16, num_splits,
+                                 sm_scale, logit_cap, packed_start_offset, 0, stream);
+    if (rc != 0) return rc;
+    return ommx_decode_combine(ws, al_stride_b, al_stride_h, al_stride_s, q, q_stride_b, q_stride_h,
+                               k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h, vt_stride_b,
+                               vt_stride_t, vt_stride_h, b_tail_len, b_seq_len, o, o_stride_b,
+                               o_stride_h, lse, lse_stride_b, B, Hq, Hkv, D, num_splits, group_tokens,
+                               sm_scale, logit_cap, stream);
+}
