@@ -22,6 +22,7 @@ SOURCES = {
     "ommx_store_generic.hip": ["-ffp-contract=off"],
     "ommx_decode_ref.hip": [],
     "ommx_decode.hip": [],
+    "ommx_decode_gqa4.hip": [],
     "ommx_combine.hip": [],
     "ommx_ring.hip": [],
     "ommx_merge.hip": [],

@@ -1,5 +1,6 @@
 // extern "C" entry points of libommx_hip.so for the decode side, argument checks and
 // kernel selection.  The store entry point lives beside its kernel in ommx_store.hip.
+#include <cstdlib>
 #include <string>
 
 #include "ommx_decode_args.h"
@@ -12,6 +13,7 @@ static thread_local std::string g_error;
 void set_error(const char* msg) { g_error = msg; }
 
 int launch_decode_fast(const DecodeArgs& a, int D, int R, hipStream_t st);
+int launch_decode_gqa4(const DecodeArgs& a, int D, int R, hipStream_t st);
 
 }  // namespace ommx
 
@@ -94,7 +96,9 @@ extern "C" int ommx_decode_splitkv(OMMX_DECODE_PARAMS) {
     if (const char* bad = check_decode(OMMX_DECODE_ARGS)) { set_error2("ommx_decode_splitkv", bad); return -1; }
     const DecodeArgs a = make_decode_args(OMMX_DECODE_ARGS);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = launch_decode_fast(a, D, Hq / Hkv, st);
+    static const bool use_old = getenv("OMMX_DECODE_OLD") != nullptr;      // TEMP: A/B switch while tuning
+    int rc = use_old ? 1 : launch_decode_gqa4(a, D, Hq / Hkv, st);
+    if (rc == 1) rc = launch_decode_fast(a, D, Hq / Hkv, st);
     if (rc == 1) rc = launch_decode_ref(a, D, Hq / Hkv, st);      // shapes the matrix-core kernel leaves out
     if (rc != 0) { set_error("ommx_decode_splitkv: no kernel for this shape"); return -1; }
     if (hipGetLastError() != hipSuccess) { set_error("ommx_decode_splitkv: launch failed"); return -2; }

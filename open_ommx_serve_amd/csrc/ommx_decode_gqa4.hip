@@ -1,0 +1,721 @@
+// Split-KV decode kernel for gfx950, serving shape: head_dim 128, 1, 2 or 4 q heads per kv head,
+// 6 outliers per K vector of 32 tokens (either index plane, either outlier map), INT2 V with
+// 32-channel vectors, int8 exponents.  Same operator as
+// ommx_gpu_serve/attention/paged_decode.py:1255-2284; the other shapes of the matrix-core path
+// (8 q heads per kv head, longer groups, no outliers) stay on the kernel in ommx_decode.hip.
+//
+// A wavefront owns one kv head (and its q heads) of one split and walks it 64 tokens at a time;
+// a workgroup is 4 waves = 4 neighbouring kv heads.  Measured on MI355X this operator is bound
+// by how many instructions one wave can issue (vector ALU first, LDS second), so the kernel is
+// built to keep THREE waves per SIMD resident: at most 168 vector registers and 13.5 KB of LDS
+// per wave.  What that takes, against the kernel in ommx_decode.hip:
+//   * P.V runs transposed (rows = V channels, columns = q heads), the V step 2^e sits in the
+//     exponent field of the V operand, and the four column replicas of the q heads each take
+//     every fourth channel block, so the output accumulator is 8 registers instead of 32;
+//   * the softmax denominator comes out of the same matrix instruction that sums p*2^e and
+//     p*zp (a row of ones), the running maximum is refreshed only when a logit exceeds it by
+//     more than 2^8 (any bound that keeps exp2 in range serves an online softmax);
+//   * the V staging area of LDS is the K staging area of the same step, reused once QK is done.
+// Arithmetic is that of ommx_decode.hip: exact 16-bit operands, fp32 accumulation.
+//   K base   B = (1 + code*2^(2k-7)) * 2^e as bf16 (code dropped into mantissa bits [2k+1:2k],
+//            k = 1 or 2 per channel pair), A = q * 2^(7-2k); the constant terms sum q*zp and
+//            sum A*2^e come from one small "bias" MFMA per 64 tokens.
+//   outliers a channel-major pass (one lane = two channels) overwrites the base code of every
+//            outlier position in the staged K rows by 0 or 3, whichever is nearer (ds_mskor_b32),
+//            and scatters (outlier - zp - code*2^e) as f16 into a [32 tokens][128 channels]
+//            tile that is the B operand of an f16 MFMA against A = q.  Deltas whose f16 rounding
+//            could show on a logit add their rounding residual times q through LDS float atomics.
+//   P.V      A = (1 + code/4 | 1 + code/16) * 2^e_v as f16 for 8 tokens of one channel, B = p (f16).
+#include <type_traits>
+
+#include "ommx_decode_util.h"
+
+namespace ommx {
+
+namespace {
+
+using namespace decode_util;
+
+#ifndef OMMX_Q_IN_REGS
+#define OMMX_Q_IN_REGS 1
+#endif
+#ifndef OMMX_LATE_FETCH
+#define OMMX_LATE_FETCH 0
+#endif
+#ifndef OMMX_GQA4_WAVES
+#define OMMX_GQA4_WAVES 3          // waves per SIMD the register budget is set for
+#endif
+constexpr int D = 128;
+// ---- per-wave LDS map (bytes) ------------------------------------------------------------
+constexpr int TILE_ROW = 272;                       // bytes per row of the outlier tile (256 used)
+constexpr int KT_ROW = 40;                          // bytes per staged K code row (32 used): 16 rows read as b64 spread over all banks
+constexpr int VT_COL = 68;                          // dwords per V dword column (64 used)
+constexpr int PT_ROW = 72;                          // halfwords per row of the f16 [row][64 tokens] arrays
+constexpr int OFF_TILE = 0;                         // [32 tokens][TILE_ROW] f16 outlier deltas of one group
+constexpr int OFF_KT = OFF_TILE + 32 * TILE_ROW;    // [64 tokens][KT_ROW] K code rows
+constexpr int OFF_MAG = OFF_KT + 64 * KT_ROW;       // [2 groups][128] f16 2^e, channels (p, p+8) adjacent
+constexpr int OFF_ZPP = OFF_MAG + 512;              // same order, f16 zero points over the A scale
+// after QK the same bytes hold what P.V needs
+constexpr int OFF_VT = OFF_KT;                      // [8 dword columns][VT_COL] V code dwords
+constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [4 heads][PT_ROW] f16 softmax weights
+constexpr int OFF_VZ = OFF_PT + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 V zero points
+constexpr int OFF_VS = OFF_VZ + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 2^e_v
+constexpr int OFF_STAGE_END = (OFF_VS + 4 * PT_ROW * 2 > OFF_ZPP + 512) ? OFF_VS + 4 * PT_ROW * 2 : OFF_ZPP + 512;
+constexpr int OFF_LC = OFF_STAGE_END;                 // [32 tokens][4 heads] f32 logit corrections of one group
+constexpr int OFF_ZERO = OFF_LC + 512;              // 128 B of zeros, never written again
+constexpr int OFF_ONES = OFF_ZERO + 128;            // 128 B of f16 1.0, never written again
+constexpr int LDS_WAVE = OFF_ONES + 128;            // 13568: three 4-wave workgroups fit a CU's 160 KB
+static_assert(OFF_KT % 16 == 0 && OFF_PT % 16 == 0 && OFF_VZ % 16 == 0 && OFF_LC % 16 == 0, "b128 alignment");
+static_assert(3 * 4 * LDS_WAVE <= 160 * 1024, "three workgroups per compute unit");
+
+// One f16 carries 11 bits: rounding an outlier delta d costs up to |d| * 2^-11, i.e. up to
+// |d| * max|q| * 2^-11 * sm_scale on a logit.  A delta with |d| * max|q| >= BIG_DELTA * 16
+// (at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its residual added exactly; smaller
+// ones stay below that and average a quarter of it.
+constexpr float BIG_DELTA = 2.0f;
+// the running maximum of the online softmax is refreshed when a logit (base 2) exceeds it by this
+constexpr float MAX_SLACK = 8.0f;
+
+// K pair p of a code dword: channels p (low half) and p+8 (high half) as f16 with the 2-bit
+// code at mantissa bits [2m+1:2m], m = k_pos(p) in 1..4, where the element reads
+// (1 + code * 2^(2m-10)) * 2^e; the A operand of that channel carries q * 2^(10-2m).  Four
+// positions, so that only pairs 0 (up two bits) and 5..7 (down six) need a shift.
+__host__ __device__ constexpr int k_pos(int p) { return p == 0 ? 1 : (p <= 4 ? p : p - 3); }
+template <int P>
+__device__ __forceinline__ uint32_t k_pair(uint32_t w, uint32_t w_up2, uint32_t w_dn6, uint32_t magic) {
+    const uint32_t sh = P == 0 ? w_up2 : (P <= 4 ? w : w_dn6);
+    return (sh & (0x00030003u << (2 * k_pos(P)))) | magic;
+}
+// V channel y of a merged dword (token a in the low 16 bits, token b in the high 16 bits) as
+// f16 (1 + c/16) * 2^e (even y, code at mantissa bits [7:6]) or (1 + c/4) * 2^e (odd y, bits
+// [9:8]); `step` holds the f16 2^e of the two tokens.
+template <int Y>
+__device__ __forceinline__ uint32_t v_pair(uint32_t m, uint32_t step) {
+    const uint32_t sh = Y <= 1 ? (m << 6) : Y <= 3 ? (m << 2) : Y <= 5 ? (m >> 2) : (m >> 6);
+    return (sh & ((Y & 1) ? 0x03000300u : 0x00C000C0u)) | step;
+}
+__device__ __forceinline__ uint32_t pk_u16(uint32_t lo, uint32_t hi) { return (lo & 0xFFFFu) | (hi << 16); }
+
+// IDX: 0 = outlier positions from 32-bit bitmaps, 1 = from 7-bit position streams.
+// OWN_MAP: outliers decode through their own (map_scale, centre) pair; false = through the
+// base scale and zero point.  PARTIAL: the kv head serves 1 or 2 q heads (spare head slots repeat
+// the last head and are not written).  ORDER: 0 one request, 1 up to 64 requests served longest
+// first, 2 up to 256 (radix select); see ommx_decode.hip.
+template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER>
+__global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // uniform: keeps the plane pointers scalar
+    uint8_t* const sm = smem_all + wave * LDS_WAVE;
+    const uint32_t sm_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint8_t*)sm));
+    const int j = lane & 15, kq = lane >> 4;
+    const int Hkv = a.Hkv;
+    const int waves = blockDim.x >> 6;
+    const int kvh = blockIdx.y * waves + wave;
+    const int heads = PARTIAL ? a.Hq / Hkv : 4;
+    const int qh0 = kvh * heads;
+    const int sp = blockIdx.x;
+    int b = blockIdx.z, L;
+    if (ORDER >= 1 && a.B > 1 && a.B <= 64) {
+        const int my_len = lane < a.B ? a.seq[lane] : 0;
+        const uint32_t key = (static_cast<uint32_t>(my_len) << 6) | (63u - lane);
+        int rank = 0;
+        for (int i = 0; i < a.B; ++i)
+            rank += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key), i)) > key;
+        b = __builtin_ctzll(__ballot(lane < a.B && rank == static_cast<int>(blockIdx.z)));
+        L = __builtin_amdgcn_readlane(my_len, b);
+    } else if (ORDER == 2 && a.B > 1 && a.B <= 256) {
+        uint32_t key[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = 64 * r + lane;
+            key[r] = idx < a.B ? (static_cast<uint32_t>(a.seq[idx] + 1) << 8) | (255u - idx) : 0u;
+        }
+        uint32_t want = 0;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = want | (1u << bit);
+            int reach = 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) reach += __popcll(__ballot(key[r] >= cand));
+            if (reach > static_cast<int>(blockIdx.z)) want = cand;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint64_t hit = __ballot(key[r] == want);
+            if (hit) b = 64 * r + __builtin_ctzll(hit);
+        }
+        L = static_cast<int>(want >> 8) - 1;
+    } else {
+        L = a.seq[b];
+    }
+    // q: this lane's 32 channels of head j % 4 (16 dwords, channel 2i in the low half of dword i)
+    // and channels 2*lane, 2*lane+1 of every head (for the channel pass)
+    uint32_t qw[16], qraw[4];      // qraw: channels 2*lane, 2*lane+1 of every head, for the thresholds below
+    {
+        const uint32_t* qh = reinterpret_cast<const uint32_t*>(
+            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & 3, heads - 1)) * a.q_sh + 32 * kq);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) qw[i] = qh[i];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            qraw[r] = *reinterpret_cast<const uint32_t*>(
+                a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
+    }
+    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
+    const int n_begin = per * sp;
+    const int n_end = min(n_begin + per, L);
+
+    if (n_begin >= n_end) {       // an empty split: the state of nothing attended
+        for (int r = 0; r < heads; ++r) {
+            float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
+            dst[lane] = 0.0f;
+            dst[64 + lane] = 0.0f;
+            if (lane == 0) dst[D] = -INFINITY;
+        }
+        return;
+    }
+
+    // ---- LDS that starts out constant: zero tile, zero corrections, the zero and one rows ----
+    {
+        u32x4* p = reinterpret_cast<u32x4*>(sm + OFF_TILE);
+        for (int i = lane; i < 32 * TILE_ROW / 16; i += 64) p[i] = u32x4{0, 0, 0, 0};
+        if (lane < 32) reinterpret_cast<u32x4*>(sm + OFF_LC)[lane] = u32x4{0, 0, 0, 0};
+        if (lane < 16) reinterpret_cast<u32x4*>(sm + OFF_ZERO)[lane] =
+            lane < 8 ? u32x4{0, 0, 0, 0} : u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+    }
+
+    f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    f32x4 accz = {0, 0, 0, 0};
+    float m_run[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
+
+    // ---- addressing ---------------------------------------------------------------------------
+    const uint32_t row_bytes = (uint32_t)Hkv * 32u;
+    const int last = n_end - 1;
+    const int ps_sh = __ffs(a.ps) - 1, ps_mask = a.ps - 1;
+    const int tsh = a.i64 ? 3 : 2;
+    const int tok_off = a.gbase * 32 + a.off;
+    const char* const rt_b = static_cast<const char*>(a.rt) + ((b * a.rt_s) << tsh);
+    const char* const rg_b = static_cast<const char*>(a.rg) + ((b * a.rg_s + a.gbase) << tsh);
+    const uint8_t* const kb_head = a.k_base + kvh * 32;
+    const uint8_t* const vb_head = a.v_main + kvh * 32;
+    const int8_t* const vs_head = a.v_scale + kvh * 4;
+    const uint16_t* const vz_head = a.v_zp + kvh * 4;
+
+    int pg1, ps1, gsl[2];
+    auto fetch_tables = [&](int n) {
+        const int p = min(n + lane, last) + tok_off;
+        pg1 = *reinterpret_cast<const int*>(rt_b + ((uint32_t)(p >> ps_sh) << tsh));
+        ps1 = p & ps_mask;
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const int gi = min((n + 32 * g) >> 5, last >> 5);
+            gsl[g] = *reinterpret_cast<const int*>(rg_b + ((uint32_t)gi << tsh));
+        }
+    };
+    u32x4 kr[2], vr[2];
+    u32x2 vzp;
+    uint32_t vsc, vrow;
+    auto fetch_k = [&]() {          // K code row of this lane's token; remembers the row for fetch_v
+        vrow = (uint32_t)((pg1 << ps_sh) + ps1);
+        const uint64_t ro = (uint64_t)vrow * row_bytes;
+        kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
+        kr[1] = *reinterpret_cast<const u32x4*>(kb_head + ro + 16);
+    };
+    auto fetch_v = [&]() {
+        const uint64_t ro = (uint64_t)vrow * row_bytes;
+        vr[0] = *reinterpret_cast<const u32x4*>(vb_head + ro);
+        vr[1] = *reinterpret_cast<const u32x4*>(vb_head + ro + 16);
+        vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)vrow * (uint32_t)(Hkv * 4));
+        vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)vrow * (uint32_t)(Hkv * 4));
+    };
+    // channel pair (2*lane, 2*lane+1) parameters of both groups
+    uint32_t g_sc[2], g_zp[2], g_ms[2] = {0, 0}, g_mc[2] = {0, 0};
+    u32x2 g_bm[2], g_ov[2];
+    uint32_t g_bx[2] = {0, 0};
+    const uint32_t kvh_s = __builtin_amdgcn_readfirstlane(kvh);
+    auto at = [](const void* base, uint32_t byte_off) { return static_cast<const char*>(base) + byte_off; };
+    auto fetch_params_g = [&](int g) {
+        // (the lane number goes through an opaque copy: otherwise plane pointer + lane offset is kept
+        // as a 64-bit register pair per plane across the loop, twelve registers the QK phase lacks;
+        // this way the loads take a scalar base and a 32-bit lane offset)
+        uint32_t lane_b = lane;
+        asm volatile("" : "+v"(lane_b));
+        const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);
+        const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + kvh_s) * D;
+        g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
+        g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
+        if (OWN_MAP) {
+            g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
+            g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
+        }
+        if constexpr (IDX == 0) {
+            g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
+        } else {
+            const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp + gidx * 6, 12 * lane_b));
+            g_bm[g] = u32x2{ixp[0], ixp[1]};
+            g_bx[g] = ixp[2];
+        }
+        const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
+        g_ov[g] = u32x2{ovp[0], ovp[1]};
+    };
+    fetch_tables(n_begin);
+    fetch_k();
+    fetch_v();
+    fetch_params_g(0);
+    fetch_params_g(1);
+    fetch_tables(n_begin + 64);
+
+    // ---- A operand of QK: q * 2^(10-2m) of head j % 4 for this lane's 32-channel quarter, f16, in
+    // pair order: k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2).  The base codes,
+    // the outlier tile and the bias columns all use this one operand (the tile and the zero points
+    // are stored divided by the channel's 2^(10-2m)).
+    u32x4 aq[4];
+    {
+        auto q_at = [&](int c) {
+            return __uint_as_float((c & 1) ? (qw[c >> 1] & 0xFFFF0000u) : (qw[c >> 1] << 16));
+        };
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
+                const float qs = static_cast<float>(1 << (10 - 2 * k_pos(4 * (ks & 1) + rr)));
+                aq[ks][rr] = pack_f16x2(qs * q_at(cl), qs * q_at(cl + 8));
+            }
+        }
+    }
+#if OMMX_Q_IN_REGS
+    auto q_of = [&](int u, int r) { return __uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16)); };
+#else
+    // q of head r, channel 2*lane + u: read again where it is needed (the residual walk, seldom taken)
+    auto q_of = [&](int u, int r) {
+        const uint32_t w = *reinterpret_cast<const uint32_t*>(
+            a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
+        return __uint_as_float(u ? (w & 0xFFFF0000u) : (w << 16));
+    };
+#endif
+    // ---- lane constants of the loop ------------------------------------------------------------
+    // channel pass: lane = channels c0 = 2*lane, c0 + 1
+    const uint32_t c0 = 2u * lane;
+    const uint32_t y0 = c0 & 15u;
+    // halfword slot of channel c0 in the pair-ordered arrays; channel c0 + 1 sits two slots on
+    const uint32_t hw0 = ((c0 >> 4) * 8u + (y0 & 7u)) * 2u + (y0 >> 3);
+    // 2^-(10-2m) of the two channels: what their zero points and tile entries are scaled by
+    const float cs0 = 1.0f / static_cast<float>(1 << (10 - 2 * k_pos(int(y0 & 7u))));
+    const float cs1 = 1.0f / static_cast<float>(1 << (10 - 2 * k_pos(int((y0 + 1u) & 7u))));
+    // per channel: the |tile entry| from which its f16 rounding matters (infinite for q = 0)
+    float big_thr[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        float qm = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
+        big_thr[u] = (BIG_DELTA * 16.0f) * (u ? cs1 : cs0) * __builtin_amdgcn_rcpf(qm);
+    }
+    const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
+    const uint32_t code_sh = 2u * (c0 & 3u);                      // bit of channel c0's code in that byte; c0 + 1 sits two on
+    const uint32_t nib_sh = 8u * ((6u * lane) & 3u);
+    const float c2 = a.sm_scale * 1.4426950408889634f;
+
+    for (int n0 = n_begin; n0 < n_end; n0 += 64) {
+        const bool more = n0 + 64 < n_end;
+        const bool g1_live = n0 + 32 < n_end;
+        {   // waves sharing a SIMD should finish together: the one with more work left goes first
+            const int left = (n_end - n0 + 63) >> 6;
+            if (left >= 4) __builtin_amdgcn_s_setprio(3);
+            else if (left == 3) __builtin_amdgcn_s_setprio(2);
+            else if (left == 2) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
+
+        // ------------------------------------------------------------------ stage K
+        {
+            u32x2* krow = reinterpret_cast<u32x2*>(sm + OFF_KT + lane * KT_ROW);
+            krow[0] = u32x2{kr[0][0], kr[0][1]};
+            krow[1] = u32x2{kr[0][2], kr[0][3]};
+            krow[2] = u32x2{kr[1][0], kr[1][1]};
+            krow[3] = u32x2{kr[1][2], kr[1][3]};
+            uint16_t* mg = reinterpret_cast<uint16_t*>(sm + OFF_MAG) + hw0;
+            uint16_t* zp = reinterpret_cast<uint16_t*>(sm + OFF_ZPP) + hw0;
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                // f16 2^e of both channels: (e + 15) << 10 per half, e a signed byte held at -15 or
+                // above (a step below 2^-14 is immaterial next to the f16 operands of the others)
+                const uint32_t e2 = __builtin_amdgcn_perm(0u, g_sc[g], 0x010C000Cu);       // (e1 << 8, e0 << 8)
+                typedef short s16x2 __attribute__((ext_vector_type(2)));
+                typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+                const s16x2 ec = __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256});
+                const uint32_t m2 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, ec) * u16x2{4, 4} + u16x2{0x3C00, 0x3C00});
+                mg[g * 128] = static_cast<uint16_t>(m2);
+                mg[g * 128 + 2] = static_cast<uint16_t>(m2 >> 16);
+                // zero points over the channel's A scale (exact: a power of two), f16
+                const uint32_t z2 = pack_f16x2(cs0 * __uint_as_float(g_zp[g] << 16),
+                                               cs1 * __uint_as_float(g_zp[g] & 0xFFFF0000u));
+                zp[g * 128] = static_cast<uint16_t>(z2);
+                zp[g * 128 + 2] = static_cast<uint16_t>(z2 >> 16);
+            }
+        }
+        lds_fence();
+#if !OMMX_LATE_FETCH
+        if (more) fetch_k();
+#endif
+
+        // ------------------------------------------------------------------ QK
+        f32x4 dsel = {0, 0, 0, 0};
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            if (g == 1 && !g1_live) break;
+            float dl_max[2] = {0.0f, 0.0f};
+            auto walk = [&](auto RES, auto U) {
+                constexpr int u = decltype(U)::value;
+                const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
+                const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
+                const float s = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                // everything below is in units of the channel's A scale: tile entry =
+                // (outlier - zp - code * 2^e) / 2^(10-2m) = level * a1 + b1 (less 3 * sc for code 3)
+                const float cs = u ? cs1 : cs0;
+                const float sc = s * cs;
+                float a1, b1;
+                if (OWN_MAP) {
+                    const float ms = __uint_as_float(u ? (g_ms[g] & 0xFFFF0000u) : (g_ms[g] << 16));
+                    const float mc = __uint_as_float(u ? (g_mc[g] & 0xFFFF0000u) : (g_mc[g] << 16));
+                    a1 = cs * __builtin_amdgcn_rcpf(ms);
+                    b1 = cs * (mc - zp);
+                } else {
+                    a1 = sc;
+                    b1 = 0.0f;
+                }
+                uint32_t bm = 0, ix_lo = 0, ix_hi = 0;
+                if constexpr (IDX == 0) {
+                    bm = g_bm[g][u];
+                } else {
+                    ix_lo = u ? __builtin_amdgcn_alignbit(g_bx[g], g_bm[g][1], 16) : g_bm[g][0];
+                    ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
+                }
+                const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
+                const uint32_t nib = static_cast<uint32_t>(ov64 >> (nib_sh + 24 * u)) & 0xFFFFFFu;
+                const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
+                const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
+                const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
+                // The base MFMA takes every position of the K rows as it is stored; the tile entry of an
+                // outlier is what is missing on top of its stored 2-bit code, which the lane looks up
+                // in the staged K rows (a byte read per outlier; the packer's code of an outlier is the
+                // clamped 0 or 3 nearly always, so the entry is small).
+                const uint8_t* kt = sm + kt_lane + g * 32 * KT_ROW;
+                float* lc = reinterpret_cast<float*>(sm + OFF_LC);
+                uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_TILE) + hw0 + 2 * u;      // pair order, like MAG
+                int pos[6];
+                uint32_t cb[6];
+#pragma unroll
+                for (int sidx = 0; sidx < 6; ++sidx) {
+                    if constexpr (IDX == 0) {
+                        pos[sidx] = __builtin_ctz(bm) & 31;
+                        if (sidx < 5) bm &= bm - 1;
+                    } else {
+                        pos[sidx] = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
+                                  : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
+                                              : ((ix_hi >> 3) & 31);
+                    }
+                    cb[sidx] = kt[pos[sidx] * KT_ROW];
+                }
+#pragma unroll
+                for (int sidx = 0; sidx < 6; ++sidx) {
+                    const float dl0 = fmaf(lv[sidx], a1, b1);
+                    const float code = static_cast<float>((cb[sidx] >> (code_sh + 2 * u)) & 3u);
+                    const float dl = fmaf(-code, sc, dl0);
+                    const _Float16 hi = static_cast<_Float16>(dl);
+                    if constexpr (!decltype(RES)::value) {
+                        dt[pos[sidx] * (TILE_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
+                        dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
+                    } else {
+                        if (fabsf(dl) >= big_thr[u]) {
+                            const float lo = (dl - static_cast<float>(hi)) * __builtin_amdgcn_rcpf(cs);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                __hip_atomic_fetch_add(lc + pos[sidx] * 4 + r, lo * q_of(u, r), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
+                        }
+                    }
+                }
+            };
+            walk(std::false_type{}, std::integral_constant<int, 0>{});
+            walk(std::false_type{}, std::integral_constant<int, 1>{});
+            const bool res0 = __any(dl_max[0] >= big_thr[0]), res1 = __any(dl_max[1] >= big_thr[1]);
+            if (res0) walk(std::true_type{}, std::integral_constant<int, 0>{});
+            if (res1) walk(std::true_type{}, std::integral_constant<int, 1>{});
+            lds_fence();
+#if !OMMX_LATE_FETCH
+            if (more) fetch_params_g(g);
+#endif
+            // both 16-token blocks of the group go through the eight k-steps together (two independent
+            // accumulation chains): tile rows (read, clear), then the base codes
+            f32x4 d[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+            u32x2 kw[2];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+                kw[t2] = *reinterpret_cast<const u32x2*>(sm + OFF_KT + (16 * (2 * g + t2) + j) * KT_ROW + 8 * kq);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2) {
+                    u32x4* row = reinterpret_cast<u32x4*>(sm + OFF_TILE + (16 * t2 + j) * TILE_ROW + 64 * kq);
+                    const u32x4 bt = row[ks];
+                    row[ks] = u32x4{0, 0, 0, 0};
+                    d[t2] = mfma_f16(aq[ks], bt, d[t2]);
+                }
+            }
+            const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAG + g * 256 + kq * 64);
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {          // code dword: channels 16*hf .. 16*hf+15 of the quarter
+                uint32_t w[2], wu[2], wd[2];
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2) { w[t2] = kw[t2][hf]; wu[t2] = w[t2] << 2; wd[t2] = w[t2] >> 6; }
+                const u32x4 ma = mg[2 * hf], mb = mg[2 * hf + 1];
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2)
+                    d[t2] = mfma_f16(aq[2 * hf], u32x4{k_pair<0>(w[t2], wu[t2], wd[t2], ma[0]), k_pair<1>(w[t2], wu[t2], wd[t2], ma[1]),
+                                                       k_pair<2>(w[t2], wu[t2], wd[t2], ma[2]), k_pair<3>(w[t2], wu[t2], wd[t2], ma[3])}, d[t2]);
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2)
+                    d[t2] = mfma_f16(aq[2 * hf + 1], u32x4{k_pair<4>(w[t2], wu[t2], wd[t2], mb[0]), k_pair<5>(w[t2], wu[t2], wd[t2], mb[1]),
+                                                           k_pair<6>(w[t2], wu[t2], wd[t2], mb[2]), k_pair<7>(w[t2], wu[t2], wd[t2], mb[3])}, d[t2]);
+            }
+            // rows 4kq..4kq+3 of every result hold the four heads: the lane keeps its own token block
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+                if (kq == 2 * g + t2) dsel = d[t2];
+            if (res0 || res1) {       // exact residuals of this group's large deltas, then zero again
+                const f32x4 corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * (lane & 31));
+                if ((kq >> 1) == g) dsel += corr;
+                lds_fence();
+                *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * (lane & 31)) = u32x4{0, 0, 0, 0};
+            }
+            lds_fence();
+        }
+        // bias columns: 0 zp(g0) 1 zp(g1) 2 2^e(g0) 3 2^e(g1); other columns repeat them
+        f32x4 dbias = {0, 0, 0, 0};
+        {
+            const int src = ((j & 2) ? OFF_MAG : OFF_ZPP) + (j & 1) * 256 + kq * 64;
+            const u32x4* bp = reinterpret_cast<const u32x4*>(sm + src);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) dbias = mfma_f16(aq[ks], bp[ks], dbias);
+        }
+#if OMMX_LATE_FETCH
+        if (more) { fetch_k(); fetch_params_g(0); fetch_params_g(1); }
+#endif
+        if (more) fetch_tables(n0 + 128);
+        lds_fence();
+
+        // ------------------------------------------------------------------ stage V (over the K staging)
+        {
+            uint32_t* vt = reinterpret_cast<uint32_t*>(sm + OFF_VT) + lane;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) vt[c * VT_COL] = vr[c >> 2][c & 3];
+            typedef short s16x2 __attribute__((ext_vector_type(2)));
+            typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+            uint16_t* vs16 = reinterpret_cast<uint16_t*>(sm + OFF_VS) + lane;
+            uint16_t* vz16 = reinterpret_cast<uint16_t*>(sm + OFF_VZ) + lane;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                // f16 2^e of two channel groups: (e + 15) << 10 per half; below 2^-15 the step is
+                // immaterial and is held there
+                const uint32_t e2 = __builtin_amdgcn_perm(0u, vsc, h2 ? 0x030C020Cu : 0x010C000Cu);   // (e << 8) pairs
+                const s16x2 ec = __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256});
+                const u16x2 st = __builtin_bit_cast(u16x2, ec) * u16x2{4, 4} + u16x2{0x3C00, 0x3C00};
+                const uint32_t s2 = __builtin_bit_cast(uint32_t, st);
+                vs16[(2 * h2) * PT_ROW] = static_cast<uint16_t>(s2);
+                vs16[(2 * h2 + 1) * PT_ROW] = static_cast<uint16_t>(s2 >> 16);
+                const uint32_t z2 = pack_f16x2(__uint_as_float(vzp[h2] << 16), __uint_as_float(vzp[h2] & 0xFFFF0000u));
+                vz16[(2 * h2) * PT_ROW] = static_cast<uint16_t>(z2);
+                vz16[(2 * h2 + 1) * PT_ROW] = static_cast<uint16_t>(z2 >> 16);
+            }
+        }
+        if (more) fetch_v();
+
+        // ------------------------------------------------------------------ softmax
+        // the lane owns token n0 + lane and the four heads; bias of (group, head) = sum q*zp - sum A*2^e
+        float x[4];
+        {
+            const int gsel = lane >> 5;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // lane 0 / 1 of every row: column 0 / 1 (zp) minus column 2 / 3 (2^e)
+                // (each row goes through a register of its own first: read straight out of the 4-register
+                // result, the four moves came out as one, all reading row 0)
+                float mine = dbias[r];
+                asm volatile("" : "+v"(mine));
+                const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                    0, __builtin_bit_cast(int, mine), 0x4E, 0xF, 0xF, true));     // quad_perm [2,3,0,1]
+                x[r] = dsel[r] + __shfl(mine - other, gsel);
+            }
+        }
+        float pe[4];          // base-2 logit minus the running maximum
+        if (a.cap > 0.0f) {
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int r = 0; r < 4; ++r) x[r] = apply_cap(x[r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pe[r] = x[r] - m_run[r];
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                x[r] *= c2;
+                pe[r] = x[r] - m_run[r];
+            }
+        }
+        const bool tok_ok = n0 + lane < n_end;
+        if (n0 + 64 > n_end) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (!tok_ok) { x[r] = -INFINITY; pe[r] = -INFINITY; }
+            }
+        }
+        if (__any(fmaxf(fmaxf(pe[0], pe[1]), fmaxf(pe[2], pe[3])) > MAX_SLACK)) {
+            // refresh the running maxima (always on the first step) and rescale what is summed so far
+            float mxs[4] = {x[0], x[1], x[2], x[3]};
+            wave_max4(mxs);
+            float alpha[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float m_new = fmaxf(m_run[r], mxs[r]);
+                alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                m_run[r] = m_new;
+                pe[r] = x[r] - m_new;
+            }
+            // accumulators hold column (x, head j % 4) in every register
+            const float al = (j & 3) == 0 ? alpha[0] : ((j & 3) == 1 ? alpha[1] : ((j & 3) == 2 ? alpha[2] : alpha[3]));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { acc[0][i] *= al; acc[1][i] *= al; accz[i] *= al; }
+        }
+        {
+            const uint32_t p01 = pack_f16x2(__builtin_amdgcn_exp2f(pe[0]), __builtin_amdgcn_exp2f(pe[1]));
+            const uint32_t p23 = pack_f16x2(__builtin_amdgcn_exp2f(pe[2]), __builtin_amdgcn_exp2f(pe[3]));
+            uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT) + lane;
+            pt[0] = static_cast<uint16_t>(p01);
+            pt[PT_ROW] = static_cast<uint16_t>(p01 >> 16);
+            pt[2 * PT_ROW] = static_cast<uint16_t>(p23);
+            pt[3 * PT_ROW] = static_cast<uint16_t>(p23 >> 16);
+        }
+        lds_fence();
+
+        // ------------------------------------------------------------------ P.V (transposed)
+        // Lane addresses of this phase, formed here from the lane number rather than carried through
+        // the QK phase, where registers are shortest (the copy below keeps them from being hoisted).
+        // Row i = j of the V operand is channel 16*(j & 7) + 8*(j >> 3) + Y; column j is (x = j >> 2, head j & 3).
+        int lane_pv = lane;
+        asm volatile("" : "+v"(lane_pv));
+        const int jp = lane_pv & 15, kqp = lane_pv >> 4;
+        const uint32_t vt_addr = OFF_VT + ((jp & 7) * VT_COL + 8 * kqp) * 4;
+        const uint32_t vs_addr = OFF_VS + (((jp & 7) >> 1) * PT_ROW + 8 * kqp) * 2;
+        const uint32_t pt_addr = OFF_PT + ((jp & 3) * PT_ROW + 8 * kqp) * 2;
+        // rows of the sums operand: 0-3 V zero points, 4-7 V steps, 8 ones, others zero
+        const uint32_t az_addr = jp < 8 ? OFF_VZ + (jp * PT_ROW + 8 * kqp) * 2 : (jp == 8 ? OFF_ONES : OFF_ZERO) + 16 * kqp;
+        const uint32_t vsel = (jp & 8) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            if (kb == 1 && !g1_live) break;
+            // sums: rows vz[cg], 2^e[cg], ones against the weights of column (x, head)
+            const u32x4 pw = *reinterpret_cast<const u32x4*>(sm + pt_addr + 64 * kb);
+            const u32x4 az = *reinterpret_cast<const u32x4*>(sm + az_addr + 64 * kb);
+            accz = mfma_f16(az, pw, accz);
+            const u32x4 sw = *reinterpret_cast<const u32x4*>(sm + vs_addr + 64 * kb);
+            const u32x4 va = *reinterpret_cast<const u32x4*>(sm + vt_addr + 128 * kb);
+            const u32x4 vb = *reinterpret_cast<const u32x4*>(sm + vt_addr + 128 * kb + 16);
+            const uint32_t mg0 = __builtin_amdgcn_perm(va[1], va[0], vsel);
+            const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], vsel);
+            const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], vsel);
+            const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], vsel);
+            // column replica x takes the channel blocks Y with Y % 4 == x: for the others the weights are zeroed
+#define OMMX_PVX(X)                                                                                   \
+            {                                                                                         \
+                const bool mine = (jp >> 2) == X;                                                     \
+                const u32x4 bx = {mine ? pw[0] : 0u, mine ? pw[1] : 0u, mine ? pw[2] : 0u, mine ? pw[3] : 0u}; \
+                acc[0] = mfma_f16(u32x4{v_pair<X>(mg0, sw[0]), v_pair<X>(mg1, sw[1]),                 \
+                                        v_pair<X>(mg2, sw[2]), v_pair<X>(mg3, sw[3])}, bx, acc[0]);   \
+                acc[1] = mfma_f16(u32x4{v_pair<4 + X>(mg0, sw[0]), v_pair<4 + X>(mg1, sw[1]),         \
+                                        v_pair<4 + X>(mg2, sw[2]), v_pair<4 + X>(mg3, sw[3])}, bx, acc[1]); \
+            }
+            OMMX_PVX(0) OMMX_PVX(1) OMMX_PVX(2) OMMX_PVX(3)
+#undef OMMX_PVX
+        }
+        lds_fence();
+    }
+
+    // ---- epilogue: o = (f*(acc - sum p*2^e) + sum p*zp) / l, f = 16 or 4; lse = m + ln l ----------
+    // sums live in the lanes of the same column j: rows 0-3 (kq 0) zero points, 4-7 (kq 1) steps, 8 (kq 2) ones
+    const int h = j & 3, x = j >> 2;
+    const float l_tot = __shfl(accz[0], 32 + j);
+    float z4[4], s4[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        z4[r] = __shfl(accz[r], j);
+        s4[r] = __shfl(accz[r], 16 + j);
+    }
+    const float inv = l_tot > 0.0f ? __builtin_amdgcn_rcpf(l_tot) : 0.0f;
+    if (h < heads) {
+        float* dst = a.al + b * a.al_b + (int64_t)(qh0 + h) * a.al_h + (int64_t)sp * a.al_s;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // row i = 4kq + r of block Y = 4*a2 + x: channel 16*(i & 7) + 8*(i >> 3) + Y, group (i & 7) / 2
+                const int cg_lo = 2 * (kq & 1);
+                const float pz = (r >> 1) ? ((kq & 1) ? z4[3] : z4[1]) : ((kq & 1) ? z4[2] : z4[0]);
+                const float psum = (r >> 1) ? ((kq & 1) ? s4[3] : s4[1]) : ((kq & 1) ? s4[2] : s4[0]);
+                (void)cg_lo;
+                const int ch = 64 * (kq & 1) + 16 * r + 8 * (kq >> 1) + 4 * a2 + x;
+                const float f = (x & 1) ? 4.0f : 16.0f;
+                dst[ch] = (f * (acc[a2][r] - psum) + pz) * inv;
+            }
+        }
+        if (x == 0 && kq == 0) {
+            const float mt = h == 0 ? m_run[0] : (h == 1 ? m_run[1] : (h == 2 ? m_run[2] : m_run[3]));
+            dst[D] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
+#ifdef OMMX_DBG
+            if (sp == 0) { float* dbg = dst + (int64_t)(a.S - sp) * a.al_s; dbg[0] = mt; dbg[1] = l_tot; dbg[2] = m_run[0]; dbg[3] = m_run[1]; dbg[4] = m_run[2]; dbg[5] = m_run[3]; }
+#endif
+        }
+    }
+}
+
+}  // namespace
+
+// Returns 0 when launched, 1 when the shape belongs to another kernel.
+int launch_decode_gqa4(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
+    if (Dh != 128 || !(R == 1 || R == 2 || R == 4)) return 1;
+    if (a.kout != 6 || a.scale_bf16 || a.v_bf16 || a.gt != 32 || a.gc != 32) return 1;
+    if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
+    const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
+    const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
+    const size_t shm = (size_t)waves * LDS_WAVE;
+    const bool own_map = a.k_ms != nullptr;
+    const int order = a.B == 1 ? 0 : (a.B > 64 && a.B <= 256 ? 2 : 1);
+#define OMMX_GO(IDX, MAP, PART, ORD) \
+    hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD>), grid, block, shm, st, a)
+#define OMMX_GO_ORD(IDX, MAP, PART)                                  \
+    do {                                                             \
+        if (order == 0) OMMX_GO(IDX, MAP, PART, 0);                  \
+        else if (order == 2) OMMX_GO(IDX, MAP, PART, 2);             \
+        else OMMX_GO(IDX, MAP, PART, 1);                             \
+    } while (0)
+    switch ((R < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
+        case 0: OMMX_GO_ORD(0, false, false); break;
+        case 1: OMMX_GO_ORD(0, true, false); break;
+        case 2: OMMX_GO_ORD(1, false, false); break;
+        case 3: OMMX_GO_ORD(1, true, false); break;
+        case 4: OMMX_GO(0, false, true, 1); break;
+        case 5: OMMX_GO(0, true, true, 1); break;
+        case 6: OMMX_GO(1, false, true, 1); break;
+        default: OMMX_GO(1, true, true, 1); break;
+    }
+#undef OMMX_GO
+#undef OMMX_GO_ORD
+    return 0;
+}
+
+}  // namespace ommx
