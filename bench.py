@@ -91,7 +91,7 @@ def _make_runner(case, splits=None):
     # serving caller would take from its own bookkeeping
     mean_len = sum(case.packed_lens) / len(case.packed_lens)
     S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu, Hq // case.kv_heads,
-                                     mean_seq_len=mean_len)
+                                     mean_seq_len=mean_len, resident=3 if Hq // case.kv_heads <= 4 else 2)
     ws = make_attn_logits(B, Hq, S, D, dev)
     o = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
     lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
@@ -116,7 +116,8 @@ def _make_runner(case, splits=None):
             1 if case.req_to_token.dtype == torch.int64 else 0, case.b_seq_len.data_ptr(),
             ws.data_ptr(), ws.stride(0), ws.stride(1), ws.stride(2),
             B, Hq, case.kv_heads, D, case.page_size, case.outliers_per_vector, _hip.INDEX_BITMAP, 0, 32, 32, 0, S,
-            float(case.sm_scale), 0.0, 0, 0, torch.cuda.current_stream(dev).cuda_stream)
+            float(case.sm_scale), 0.0, 0, 0, int(p["k_base"].shape[0]), int(p["k_scale"].shape[0]), None,
+            torch.cuda.current_stream(dev).cuda_stream)
         _hip.check(rc, "ommx_decode_splitkv")
 
     return step, stage1, o, lse, S
@@ -183,7 +184,8 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
     lse = torch.empty(B, q_heads, dtype=torch.float32, device="cuda")
     n_cu = torch.cuda.get_device_properties(0).multi_processor_count
     max_seq = win.packed_len(ctx + total)
-    S = splits or auto_num_kv_splits(max_seq, B, H, n_cu, q_heads // H, mean_seq_len=win.packed_len(ctx))
+    S = splits or auto_num_kv_splits(max_seq, B, H, n_cu, q_heads // H, mean_seq_len=win.packed_len(ctx),
+                                     resident=3 if q_heads // H <= 4 else 2)
     ws = make_attn_logits(B, q_heads, S, D, "cuda")
 
     def step():

@@ -26,8 +26,9 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 5   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
-                                5: decode without a workspace argument */
+#define OMMX_ABI_VERSION 6   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
+                                5: decode without a workspace argument; 6: plane extents + error flag on
+                                the decode entry points, up to 512 splits */
 
 /* step of the INT2 quantisers and the dtype of the k_scale / v_scale planes */
 #define OMMX_SCALE_POW2_INT8  0
@@ -52,6 +53,8 @@ extern "C" {
 #define OMMX_ERR_EXP_RANGE     8   /* scale exponent does not fit the int8 plane */
 /* error bit OR-ed into *err_flag by ommx_ring_write / ommx_tail_gather */
 #define OMMX_ERR_RING_RANGE   16   /* row outside the history (kv_store_ops.py:33-34,52-53) */
+/* error bit OR-ed into *err_flag by the decode entry points */
+#define OMMX_ERR_TABLE_RANGE  64   /* a page id or group slot outside the planes (kv_pool.py:526-550 guards these on the host) */
 /* error bit OR-ed into *err_flag by ommx_index_convert */
 #define OMMX_ERR_INDEX_PLANE  32   /* a vector that does not name exactly k positions below group_tokens
                                       (codec.py:173-178 raises ValueError there) */
@@ -130,9 +133,11 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *   attn_logits   f32 [B,Hq,>=num_splits,D+1] with strides al_stride_b/h/s: partial
  *                 o (normalised) in [0,D) and lse at D; an empty split writes o=0,
  *                 lse=-inf (paged_decode.py:2262-2284)
- * Split s covers tokens [s*per, min((s+1)*per, L)), per = ceil(ceil(L/S)/gt)*gt with
- * gt = group_tokens (paged_decode.py:1429-1432); ommx_decode_combine must be given the same gt.
- * Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64; num_splits <= 256; planes 8-byte aligned.
+ * How the tokens are dealt out to the splits is the kernel's own business (the reference rounds
+ * ceil(L/S) up to whole groups, paged_decode.py:1429-1432; the kernel for up to 4 q heads per kv
+ * head deals whole groups out evenly): every split writes its state, an empty one o = 0 and
+ * lse = -inf, and ommx_decode_combine weighs the states by their lse.
+ * Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64; num_splits <= 512; planes 8-byte aligned.
  *   group_tokens / group_channels   tokens per K group and channels per V vector: 16, 32, 64, 128
  *   scale_bf16 = 1   k_scale / v_scale hold the steps themselves as bf16, not int8 exponents
  *   v_bf16 = 1       v_main is bf16 [P,ps,H,D]; v_scale / v_zp are ignored
@@ -141,6 +146,12 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *   64- or 128-token groups with 32/64/128-channel V vectors and 6 outliers, relidx7 plane;
  *   128-token groups with 10 outliers, relidx7 plane (4 or 8 q heads per kv head).
  * Every other supported shape or recipe (k_outliers up to 16) runs on the plain fp32 kernel.
+ *   num_pages, num_group_slots   extents of the planes the tables index (k_base / v_main pages,
+ *                 k_scale group slots); the reference guards table entries on the host
+ *                 (kv_pool.py:526-550), here an entry outside its plane is clamped into it, so no
+ *                 access leaves the planes, and OMMX_ERR_TABLE_RANGE is OR-ed into *err_flag
+ *                 (NULL allowed; the caller zeroes it).  0 = extent not given, entries used as
+ *                 they are.  A negative b_seq_len counts as 0 and is reported the same way.
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
@@ -155,7 +166,15 @@ int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_
                         int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
                         int index_repr, int scale_bf16, int group_tokens, int group_channels,
                         int v_bf16, int num_splits, float sm_scale, float logit_cap,
-                        int packed_start_offset, int seg_group_base, void* stream);
+                        int packed_start_offset, int seg_group_base,
+                        int num_pages, int num_group_slots, int32_t* err_flag, void* stream);
+
+/*
+ * The clamp the decode kernels apply to a page id / group slot read from a table, evaluated on the
+ * host: returns the id held inside [0, extent) (unchanged when extent is 0 = not given) and sets
+ * *out_of_range (may be NULL) to whether it had to be moved.  For tests of the arithmetic.
+ */
+int ommx_clamp_table_id(int id, int extent, int* out_of_range);
 
 /*
  * The same operator through the plain fp32 kernel only; identical arguments.  It has no
@@ -174,20 +193,22 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
                             int64_t al_stride_s,
                             int B, int Hq, int Hkv, int D, int page_size, int k_outliers,
                             int index_repr, int scale_bf16, int group_tokens, int group_channels,
-                        int v_bf16, int num_splits, float sm_scale, float logit_cap,
-                            int packed_start_offset, int seg_group_base, void* stream);
+                            int v_bf16, int num_splits, float sm_scale, float logit_cap,
+                            int packed_start_offset, int seg_group_base,
+                            int num_pages, int num_group_slots, int32_t* err_flag, void* stream);
 
 /*
  * Split combine with the bf16 sink/recent tail folded in (stage 2).
  *   k_tail,v_tail bf16 [B,Tmax,Hkv,D] with strides t_stride_b/t/h (K and V alike)
  *   b_tail_len    int32[B] valid tail rows (0 allowed)
  *   o             f32 [B,Hq,D] strides o_stride_b/h;  lse f32 [B,Hq] stride lse_stride_b
- * Valid splits are recomputed from b_seq_len with the stage-1 rounding
- * (paged_decode.py:2407-2410); nothing attended gives o = 0, lse = -inf.
+ * A split with lse = -inf weighs nothing (the reference recomputes which splits are empty from
+ * b_seq_len, paged_decode.py:2407-2410; here stage 1 marks them); nothing attended gives o = 0,
+ * lse = -inf.
  * b_tail_len == NULL (then k_tail, v_tail, q may be NULL too) combines the splits alone:
  * the un-merged state of a group-range segment (paged_decode.py:2892-2902).
  * k_tail rows must be 16-byte aligned (base pointer and strides multiples of 8 elements);
- * num_splits <= 256.
+ * num_splits <= 512.
  */
 int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,
@@ -209,6 +230,7 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
  * Arguments are those of ommx_decode_splitkv and ommx_decode_combine without the workspace:
  * the partial states of the splits are kept in a device array built into the library
  * (2 Mi floats = 8 MiB, held by every GPU the library runs on until the process ends).
+ * num_pages / num_group_slots / err_flag as for ommx_decode_splitkv.
  * Limit: B * Hq * (num_splits + 1) * (D + 1) <= 2097152 floats; larger calls return -1 with a
  * message naming the limit.  Calls that overlap in time on one GPU share the array and race;
  * calls on one stream (or otherwise ordered) are safe, and nothing needs clearing between
@@ -230,7 +252,8 @@ int ommx_decode_attention_noalloc(
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
     int group_tokens, int group_channels, int v_bf16, int num_splits,
-    float sm_scale, float logit_cap, int packed_start_offset, void* stream);
+    float sm_scale, float logit_cap, int packed_start_offset,
+    int num_pages, int num_group_slots, int32_t* err_flag, void* stream);
 
 /*
  * bf16 residual ring, write side: one new K/V row per request.

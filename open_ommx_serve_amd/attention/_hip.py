@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
-ABI_VERSION = 5
+ABI_VERSION = 6
 INDEX_BITMAP, INDEX_RELIDX7, INDEX_COMBINADIC = 0, 1, 2
 SCALE_POW2_INT8, SCALE_POW2_BF16, SCALE_BF16 = 0, 1, 2
 
@@ -29,6 +29,7 @@ def scale_mode(use_pow2: bool, kv_int8_scale: bool) -> int:
     return SCALE_POW2_INT8 if kv_int8_scale else SCALE_POW2_BF16
 ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
 ERR_INDEX_PLANE = 32
+ERR_TABLE_RANGE = 64
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -41,7 +42,8 @@ _DECODE_ARGS = [
     _P, _L, _L, _L,                   # attn_logits, strides
     _I, _I, _I, _I, _I, _I, _I, _I,       # B Hq Hkv D ps kout index_repr scale_bf16
     _I, _I, _I, _I,                       # group_tokens group_channels v_bf16 S
-    _F, _F, _I, _I, _P,               # sm_scale cap off gbase stream
+    _F, _F, _I, _I,                   # sm_scale cap off gbase
+    _I, _I, _P, _P,                   # num_pages num_group_slots err_flag stream
 ]
 
 _SIGNATURES = {
@@ -52,6 +54,7 @@ _SIGNATURES = {
                              _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ommx_decode_splitkv": (_I, _DECODE_ARGS),
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),
+    "ommx_clamp_table_id": (_I, [_I, _I, _P]),
     "ommx_decode_combine": (_I, [_P, _L, _L, _L, _P, _L, _L, _P, _P, _L, _L, _L, _L, _L, _L,
                                  _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _I, _F, _F, _P]),
     "ommx_decode_attention_noalloc": (_I, [
@@ -60,7 +63,7 @@ _SIGNATURES = {
         _P, _P, _L, _L, _L, _L, _L, _L, _P,                      # tail rows, strides, b_tail_len
         _P, _L, _L, _P, _L,                                      # o, lse
         _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,          # B Hq Hkv D ps kout repr scale_bf16 gt gc v_bf16 S
-        _F, _F, _I, _P]),                                        # sm_scale cap off stream
+        _F, _F, _I, _I, _I, _P, _P]),                            # sm_scale cap off num_pages num_group_slots err stream
     "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
                              _I, _I, _I, _I, _I, _P, _P]),
     "ommx_merge_states": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P]),

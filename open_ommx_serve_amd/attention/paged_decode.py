@@ -30,40 +30,54 @@ def _cu_count(device: torch.device) -> int:
     return _CU_COUNT[key]
 
 
+MAX_KV_SPLITS = 512
+
+
 def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 256,
                        q_per_kv: int = 4, group_tokens: int = 32,
-                       mean_seq_len: Optional[float] = None) -> int:
-    """Split count that gives every compute unit four workgroups, two resident and two queued
-    behind them so that requests of different length even out (a workgroup is four waves of
-    one split; a wave covers one kv head and all of its q heads, so ``q_per_kv`` does not
-    enter) -- or only the two resident ones when ``mean_seq_len`` says that the requests are
-    about equally long (at least 0.9 of the longest): little is left to even out then, and a
-    second round of workgroups mostly pays the start-up of a workgroup (about one step) again,
-    10 % of the whole on short splits and still 6 % at 16 steps per split (2 x 64K tokens, 8 x 32K
-    with 8 q heads per kv head; 8 x 64K, 16 x 32K and 32 x 16K measure the same either way); and
-    eight per unit when the requests differ in length and a
-    workgroup would otherwise run for more than sixteen steps -- but never less than one
-    64-token step per split (one 32-token group when even that leaves units idle): a wave's time
-    is a fixed part plus ~5 us per step, so while compute units are idle more splits are faster;
-    and the steps are dealt out evenly (the split length
-    is rounded up to whole groups by the kernel, so a careless count leaves splits empty and
-    others a step longer).  At most 256, the number of partial states the combine kernel keeps
-    on chip.  Splits are whole K groups (``group_tokens``), so longer groups mean coarser steps."""
+                       mean_seq_len: Optional[float] = None, resident: int = 2) -> int:
+    """Split count for one decode call.  A workgroup is four waves of one split (a wave covers one
+    kv head and all of its q heads, so ``q_per_kv`` does not enter); ``resident`` workgroups fit a
+    compute unit at a time (3 for the kernel that serves up to 4 q heads per kv head, 2 for the
+    others).  Requests about equally long (``mean_seq_len`` at least 0.9 of the longest) get one
+    round of workgroups: little is left to even out, and a second round mostly pays the start-up of
+    a workgroup (about one step) again.  Requests of different length get two rounds, so that they
+    even out, and four when a workgroup would otherwise run for more than sixteen steps.  Never
+    less than one 64-token step per split (one 32-token group when even that leaves units idle): a
+    wave's time is a fixed part plus a few microseconds per step, so while compute units are idle
+    more splits are faster.  The kernel with ``resident`` 3 deals whole groups out evenly by itself;
+    for the others the count is chosen so that their rounding leaves no split empty.  At most 512,
+    the number of partial states the combine kernel keeps on chip.  Splits are whole K groups
+    (``group_tokens``), so longer groups mean coarser steps."""
     wgs_per_split = max(1, int(batch) * max(1, int(kv_heads) // 4))
-    want = max(1, min(256, (4 * int(n_cu)) // wgs_per_split))
     gt = max(32, int(group_tokens))
     step_tokens = max(64, gt)
     steps = max(1, (int(max_seq_len) + step_tokens - 1) // step_tokens)
-    equal = mean_seq_len is not None and float(mean_seq_len) >= 0.9 * float(max_seq_len)
-    steps_per_split = (steps + min(want, steps) - 1) // min(want, steps)
-    if equal:
-        want = max(1, min(256, (2 * int(n_cu)) // wgs_per_split))
-    elif not equal and int(batch) > 1 and steps_per_split > 16:
-        # long splits of requests of different length: eight per unit even out better (3-6 %
-        # on 96-128 requests of 1K..16K tokens), the start-up they add is small against 16 steps
-        want = max(1, min(256, (8 * int(n_cu)) // wgs_per_split))
+    groups = max(1, (int(max_seq_len) + gt - 1) // gt)
+    equal = int(batch) == 1 or (mean_seq_len is not None and float(mean_seq_len) >= 0.9 * float(max_seq_len))
+    rounds = 1 if equal else 2
+
+    def count(res: int) -> int:
+        want = max(1, min(MAX_KV_SPLITS, (rounds * res * int(n_cu)) // wgs_per_split))
+        if not equal and int(batch) > 1 and (steps + min(want, steps) - 1) // min(want, steps) > 16:
+            # long splits of requests of different length: four rounds even out better (3-6 % on
+            # 96-128 requests of 1K..16K tokens), the start-up they add is small against 16 steps
+            want = max(1, min(MAX_KV_SPLITS, (4 * res * int(n_cu)) // wgs_per_split))
+        return want
+
+    res = max(1, int(resident))
+    want = count(res)
+    if res >= 3 and steps < 4 * want:
+        # a third resident workgroup pays only while every wave keeps four steps or more: below that
+        # the start-up of the extra waves costs more than their overlap returns (one request of 64K
+        # tokens: 27.7 us with 256 splits of four steps, 28.9 us with 384 of fewer than three)
+        res = 2
+        want = count(res)
     if want >= 2 * steps:          # plenty of idle units: splits of one K group
-        return int(min(want, max(1, (int(max_seq_len) + gt - 1) // gt)))
+        return int(min(want, groups))
+    if res >= 3:
+        # the kernel deals the groups out evenly whatever the count: fill the chip
+        return int(max(1, min(want, groups)))
     target = max(1, min(want, steps))
     # equal whole steps per split, no empty split: the slowest wave sets the kernel's time
     steps_per_split = (steps + target - 1) // target
@@ -108,6 +122,7 @@ def ommx_paged_decode_attention_canonical(
     seg_group_base: int = 0,
     _force_reference_kernel: bool = False,
     mean_seq_len: Optional[float] = None,
+    err_flag: Any = None,
 ) -> None:
     """Canonical-KV paged decode attention.  Writes ``o [B,Hq,D]`` / ``lse [B,Hq]`` in place.
 
@@ -117,7 +132,10 @@ def ommx_paged_decode_attention_canonical(
 
     ``mean_seq_len`` (not in the reference's signature) is a hint for the automatic split count
     only: a caller that passes ``max_seq_len`` to avoid the host sync may also say how long the
-    requests are on average, see :func:`auto_num_kv_splits`.
+    requests are on average, see :func:`auto_num_kv_splits`.  ``err_flag`` (not in the reference's
+    signature either): an int32 device tensor that receives ``_hip.ERR_TABLE_RANGE`` when a page id
+    or group slot of the tables lies outside the planes (the kernels clamp such an entry, so nothing
+    is read out of bounds; the reference leaves these checks to the pools, ``kv_pool.py:526-550``).
     """
     pages, ngroups = int(k_base.shape[0]), int(k_scale.shape[0])
     ps = int(page_size)
@@ -244,9 +262,13 @@ def ommx_paged_decode_attention_canonical(
             mean_seq_len = sum(lens) / len(lens)
     else:
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
+    # the kernel for up to 4 q heads per kv head (serving recipe shapes) keeps three workgroups per
+    # compute unit resident, the others two; it also serves the call in one launch
+    lean = (D == 128 and Hq // Hkv <= 4 and k == 6 and group_tokens == 32 and group_channels == 32
+            and not scale_bf16 and not v_bf16 and not _force_reference_kernel)
     if num_kv_splits is None:
         num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv, group_tokens,
-                                           mean_seq_len)
+                                           mean_seq_len, resident=3 if lean else 2)
     S = max(1, int(num_kv_splits))
     if attn_logits is None:
         attn_logits = make_attn_logits(B, Hq, S, D, q.device)
@@ -264,32 +286,32 @@ def ommx_paged_decode_attention_canonical(
                 or k_tail.stride(-1) != 1 or v_tail.stride(-1) != 1:
             raise ValueError("k_tail / v_tail must be bf16 [B, T, Hkv, D] with unit inner stride")
 
+    if err_flag is not None and (err_flag.dtype != torch.int32 or err_flag.device != q.device):
+        raise ValueError("err_flag must be an int32 tensor on the device of q")
     lib = _hip.load()
     stream = _hip.current_stream_ptr(q.device)
     splitkv = lib.ommx_decode_splitkv_ref if _force_reference_kernel else lib.ommx_decode_splitkv
+    tail_args = ((k_tail.data_ptr(), v_tail.data_ptr(), k_tail.stride(0), k_tail.stride(1), k_tail.stride(2),
+                  v_tail.stride(0), v_tail.stride(1), v_tail.stride(2), b_tail_len.data_ptr())
+                 if has_tail else (None, None, 0, 0, 0, 0, 0, 0, None))
+    planes = (k_base.data_ptr(), k_scale.data_ptr(), k_zp.data_ptr(),
+              _hip.ptr(k_fp4_mapscale) if use_map else None, _hip.ptr(k_fp4_mapcenter) if use_map else None,
+              _hip.ptr(k_index) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
+              v_main.data_ptr(), v_scale.data_ptr(), v_zp.data_ptr(),
+              req_to_token.data_ptr(), req_to_token.stride(0),
+              req_to_group.data_ptr(), req_to_group.stride(0),
+              1 if req_to_token.dtype == torch.int64 else 0,
+              b_seq_len.data_ptr(),
+              attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2))
+    shape = (B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, group_tokens, group_channels,
+             1 if v_bf16 else 0, S, float(sm_scale), float(logit_cap), off, gbase,
+             pages, ngroups, _hip.ptr(err_flag), stream)
     with torch.cuda.device(q.device):
-        rc = splitkv(
-            q.data_ptr(), q.stride(0), q.stride(1),
-            k_base.data_ptr(), k_scale.data_ptr(), k_zp.data_ptr(),
-            _hip.ptr(k_fp4_mapscale) if use_map else None, _hip.ptr(k_fp4_mapcenter) if use_map else None,
-            _hip.ptr(k_index) if k > 0 else None, _hip.ptr(k_oval) if k > 0 else None,
-            v_main.data_ptr(), v_scale.data_ptr(), v_zp.data_ptr(),
-            req_to_token.data_ptr(), req_to_token.stride(0),
-            req_to_group.data_ptr(), req_to_group.stride(0),
-            1 if req_to_token.dtype == torch.int64 else 0,
-            b_seq_len.data_ptr(),
-            attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            B, Hq, Hkv, D, ps, k, index_repr, 1 if scale_bf16 else 0, group_tokens, group_channels,
-            1 if v_bf16 else 0, S,
-            float(sm_scale), float(logit_cap), off, gbase, stream)
+        rc = splitkv(q.data_ptr(), q.stride(0), q.stride(1), *planes, *shape)
         _hip.check(rc, "ommx_decode_splitkv")
         rc = lib.ommx_decode_combine(
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
-            q.data_ptr(), q.stride(0), q.stride(1),
-            k_tail.data_ptr() if has_tail else None, v_tail.data_ptr() if has_tail else None,
-            *( (k_tail.stride(0), k_tail.stride(1), k_tail.stride(2),
-                v_tail.stride(0), v_tail.stride(1), v_tail.stride(2)) if has_tail else (0,) * 6),
-            b_tail_len.data_ptr() if has_tail else None, b_seq_len.data_ptr(),
+            q.data_ptr(), q.stride(0), q.stride(1), *tail_args[:8], tail_args[8], b_seq_len.data_ptr(),
             o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(0),
             B, Hq, Hkv, D, S, group_tokens, float(sm_scale), float(logit_cap), stream)
         _hip.check(rc, "ommx_decode_combine")

@@ -1,6 +1,5 @@
 // extern "C" entry points of libommx_hip.so for the decode side, argument checks and
 // kernel selection.  The store entry point lives beside its kernel in ommx_store.hip.
-#include <cstdlib>
 #include <string>
 
 #include "ommx_decode_args.h"
@@ -21,6 +20,15 @@ extern "C" int ommx_abi_version(void) { return OMMX_ABI_VERSION; }
 
 extern "C" const char* ommx_last_error(void) { return ommx::g_error.c_str(); }
 
+// The clamp the decode kernels apply to every page id / group slot they read from a table, on the
+// host (for tests of the arithmetic: no kernel has to be given a bad table to check it).
+extern "C" int ommx_clamp_table_id(int id, int extent, int* out_of_range) {
+    bool bad = false;
+    const int r = ommx::clamp_id(id, extent, bad);
+    if (out_of_range) *out_of_range = bad ? 1 : 0;
+    return r;
+}
+
 // The two split-KV entry points take the same arguments and refuse the same ones.
 #define OMMX_DECODE_PARAMS                                                                          \
     const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,                                      \
@@ -32,13 +40,14 @@ extern "C" const char* ommx_last_error(void) { return ommx::g_error.c_str(); }
     float* attn_logits, int64_t al_stride_b, int64_t al_stride_h, int64_t al_stride_s,              \
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,   \
     int group_tokens, int group_channels, int v_bf16, int num_splits,                               \
-    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base, void* stream
+    float sm_scale, float logit_cap, int packed_start_offset, int seg_group_base,                   \
+    int num_pages, int num_group_slots, int32_t* err_flag, void* stream
 #define OMMX_DECODE_ARGS                                                                            \
     q, q_stride_b, q_stride_h, k_base, k_scale, k_zp, k_ms, k_mc, k_index, k_oval, v_main, v_scale, \
     v_zp, req_to_token, rt_stride, req_to_group, rg_stride, table_i64, b_seq_len, attn_logits,      \
     al_stride_b, al_stride_h, al_stride_s, B, Hq, Hkv, D, page_size, k_outliers, index_repr,        \
     scale_bf16, group_tokens, group_channels, v_bf16, num_splits, sm_scale, logit_cap,              \
-    packed_start_offset, seg_group_base, stream
+    packed_start_offset, seg_group_base, num_pages, num_group_slots, err_flag, stream
 
 namespace ommx {
 
@@ -51,7 +60,8 @@ static const char* check_decode(OMMX_DECODE_PARAMS) {
     (void)q_stride_b; (void)q_stride_h; (void)rt_stride; (void)rg_stride; (void)table_i64;
     (void)al_stride_b; (void)al_stride_h; (void)al_stride_s; (void)scale_bf16; (void)v_bf16;
     (void)k_scale; (void)v_scale;
-    (void)sm_scale; (void)logit_cap; (void)stream;
+    (void)sm_scale; (void)logit_cap; (void)stream; (void)err_flag;
+    if (num_pages < 0 || num_group_slots < 0) return "num_pages / num_group_slots must be >= 0 (0 = not given)";
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv)
         return "q heads must be a positive multiple of kv heads";
     const int R = Hq / Hkv;
@@ -63,8 +73,8 @@ static const char* check_decode(OMMX_DECODE_PARAMS) {
     if (packed_start_offset < 0 || packed_start_offset >= page_size || seg_group_base < 0)
         return "packed_start_offset must be in [0,page_size), seg_group_base >= 0";
     if (k_outliers < 0 || k_outliers > 16 || k_outliers > group_tokens || num_splits < 1 ||
-        num_splits > 256 || (index_repr != 0 && index_repr != 1))
-        return "k_outliers in [0,min(16,group_tokens)], num_splits in [1,256], index_repr 0|1";
+        num_splits > 512 || (index_repr != 0 && index_repr != 1))
+        return "k_outliers in [0,min(16,group_tokens)], num_splits in [1,512], index_repr 0|1";
     if ((reinterpret_cast<uintptr_t>(k_base) | reinterpret_cast<uintptr_t>(v_main) |
          reinterpret_cast<uintptr_t>(v_zp) | reinterpret_cast<uintptr_t>(k_index) |
          reinterpret_cast<uintptr_t>(k_oval) | reinterpret_cast<uintptr_t>(k_zp) |
@@ -84,7 +94,7 @@ static DecodeArgs make_decode_args(OMMX_DECODE_PARAMS) {
                       req_to_group, rg_stride, table_i64, b_seq_len, attn_logits, al_stride_b, al_stride_h,
                       al_stride_s, B, Hq, Hkv, page_size, k_outliers, num_splits, sm_scale, logit_cap,
                       packed_start_offset, seg_group_base, index_repr, scale_bf16 ? 1 : 0,
-                      group_tokens, group_channels, v_bf16 ? 1 : 0};
+                      group_tokens, group_channels, v_bf16 ? 1 : 0, num_pages, num_group_slots, err_flag};
 }
 
 static void set_error2(const char* where, const char* what) { g_error = std::string(where) + ": " + what; }
@@ -96,8 +106,7 @@ extern "C" int ommx_decode_splitkv(OMMX_DECODE_PARAMS) {
     if (const char* bad = check_decode(OMMX_DECODE_ARGS)) { set_error2("ommx_decode_splitkv", bad); return -1; }
     const DecodeArgs a = make_decode_args(OMMX_DECODE_ARGS);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    static const bool use_old = getenv("OMMX_DECODE_OLD") != nullptr;      // TEMP: A/B switch while tuning
-    int rc = use_old ? 1 : launch_decode_gqa4(a, D, Hq / Hkv, st);
+    int rc = launch_decode_gqa4(a, D, Hq / Hkv, st);
     if (rc == 1) rc = launch_decode_fast(a, D, Hq / Hkv, st);
     if (rc == 1) rc = launch_decode_ref(a, D, Hq / Hkv, st);      // shapes the matrix-core kernel leaves out
     if (rc != 0) { set_error("ommx_decode_splitkv: no kernel for this shape"); return -1; }
@@ -144,8 +153,8 @@ extern "C" int ommx_decode_combine(
         set_error("ommx_decode_combine: k_tail rows must be 16-byte aligned (strides multiples of 8)");
         return -1;
     }
-    if (num_splits > 256) {
-        set_error("ommx_decode_combine: at most 256 KV splits");
+    if (num_splits > 512) {
+        set_error("ommx_decode_combine: at most 512 KV splits");
         return -1;
     }
     CombineArgs a{attn_logits, al_stride_b, al_stride_h, al_stride_s, q, q_stride_b, q_stride_h,
@@ -267,10 +276,11 @@ extern "C" int ommx_decode_attention_noalloc(
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
     int group_tokens, int group_channels, int v_bf16, int num_splits,
-    float sm_scale, float logit_cap, int packed_start_offset, void* stream) {
+    float sm_scale, float logit_cap, int packed_start_offset,
+    int num_pages, int num_group_slots, int32_t* err_flag, void* stream) {
     using namespace ommx;
     const char* where = "ommx_decode_attention_noalloc";
-    if (B <= 0 || Hq <= 0 || D <= 0 || num_splits < 1 || num_splits > 256) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || num_splits < 1 || num_splits > 512) {
         set_error2(where, "bad shape");
         return -1;
     }
@@ -293,7 +303,8 @@ extern "C" int ommx_decode_attention_noalloc(
                                  rg_stride, table_i64, b_seq_len, ws, al_stride_b, al_stride_h,
                                  al_stride_s, B, Hq, Hkv, D, page_size, k_outliers, index_repr,
                                  scale_bf16, group_tokens, group_channels, v_bf16, num_splits,
-                                 sm_scale, logit_cap, packed_start_offset, 0, stream);
+                                 sm_scale, logit_cap, packed_start_offset, 0, num_pages, num_group_slots,
+                                 err_flag, stream);
     if (rc != 0) return rc;
     return ommx_decode_combine(ws, al_stride_b, al_stride_h, al_stride_s, q, q_stride_b, q_stride_h,
                                k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h, vt_stride_b,

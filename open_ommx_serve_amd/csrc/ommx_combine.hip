@@ -62,12 +62,12 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
         }
     }
     const uint32_t q_raw = (a.q && tid < D) ? a.q[b * a.q_sb + (int64_t)h * a.q_sh + tid] : 0u;
-    const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:2407
+    // Every split wrote its state, an empty one with lse = -inf (paged_decode.py:2262-2284), so the
+    // weights follow from the lse column alone, whatever rule dealt the tokens out to the splits
+    // (the reference recomputes its rounding here, paged_decode.py:2407-2410).
     float my_lse = -INFINITY;
-    if (tid < MAXS) {
-        const bool valid = tid < a.S && min(per * tid + per, L) > per * tid;
-        if (valid) my_lse = base[(int64_t)tid * a.al_s + D];
-    }
+    if (tid < MAXS && tid < a.S) my_lse = base[(int64_t)tid * a.al_s + D];
+    (void)L;
 
     if (tid < D) s_q[tid] = __uint_as_float(q_raw << 16);
     if (tid < MAXS) {
@@ -223,9 +223,9 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
             s_q[r][2 * c2 + 1] = __uint_as_float(w & 0xFFFF0000u);
         }
     }
-    const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:2407
+    (void)L;
     if (wave < R) {
-        const bool valid = lane < a.S && min(per * lane + per, L) > per * lane;
+        const bool valid = lane < a.S;          // an empty split's lse is -inf
         const float my_lse = valid ? base[(int64_t)wave * a.al_h + (int64_t)lane * a.al_s + D] : -INFINITY;
         const float g_max = wave_max_f32(my_lse);
         const float g_safe = (g_max == -INFINITY) ? 0.0f : g_max;
@@ -381,7 +381,7 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
 }
 
 int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
-    if (a.S > 256) return -1;
+    if (a.S > 512) return -1;
     // Pieces per head.  At batch 1 the kernel is latency bound and 2 pieces measured best (1.4 us
     // per step at 64K less than one, the same as four, 0.5 us less than eight); with many
     // (request, head) pairs the grid fills the chip by itself and one piece repeats no work.
@@ -397,6 +397,15 @@ int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
         else if (D == 128) hipLaunchKernelGGL((combine_grouped_kernel<128, 8>), g2, dim3(512), 0, st, a);
         else if (D == 64 && R == 4) hipLaunchKernelGGL((combine_grouped_kernel<64, 4>), g2, dim3(512), 0, st, a);
         else if (D == 64) hipLaunchKernelGGL((combine_grouped_kernel<64, 8>), g2, dim3(512), 0, st, a);
+        else return -1;
+        return 0;
+    }
+    if (a.S > 256) {        // 257..512 splits: the same kernel with twice the split slots per thread
+        const dim3 g1(a.B, a.Hq, split2 ? 2 : 1);
+        if (D == 128 && split2) hipLaunchKernelGGL((combine_kernel<128, 2, 1024, 512>), g1, dim3(1024), 0, st, a);
+        else if (D == 128) hipLaunchKernelGGL((combine_kernel<128, 1, 1024, 512>), g1, dim3(1024), 0, st, a);
+        else if (D == 64 && split2) hipLaunchKernelGGL((combine_kernel<64, 2, 1024, 512>), g1, dim3(1024), 0, st, a);
+        else if (D == 64) hipLaunchKernelGGL((combine_kernel<64, 1, 1024, 512>), g1, dim3(1024), 0, st, a);
         else return -1;
         return 0;
     }

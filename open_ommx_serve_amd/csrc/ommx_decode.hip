@@ -188,6 +188,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     constexpr int GT = 32 << GTS;
     static_assert(GTS == 0 || IDX == 1, "longer groups are read through position streams");
     static_assert(KO == 6 || (KO == 10 && IDX == 1), "10 outliers: position streams only");
+    if (L < 0) { L = 0; report_table_range(a.err, true); }      // a negative length: nothing packed, reported
     const int per = ((((L + a.S - 1) / a.S) + GT - 1) / GT) * GT;
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
@@ -246,7 +247,9 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     u32x4 kr[2], vr[2];
     u32x2 vzp;
     uint32_t vsc;
+    bool bad_id = false;            // a table entry outside the planes was seen (and clamped)
     auto fetch_kv = [&]() {
+        pg1 = clamp_id(pg1, a.n_pages, bad_id);
         const int row1 = (pg1 << ps_sh) + ps1;              // physical row of this lane's token
         const uint64_t ro = (uint64_t)(uint32_t)row1 * row_bytes;
         kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
@@ -286,7 +289,7 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
     };
     auto fetch_params_g = [&](int g) {
         {
-            const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);   // same for every lane
+            const uint32_t gs = __builtin_amdgcn_readfirstlane(clamp_id(gsl[g], a.n_gslots, bad_id));   // same for every lane
             const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + kvh_s) * D;
             g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
             g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
@@ -768,6 +771,8 @@ __global__ void __launch_bounds__(256, 2) decode_splitkv_mfma_kernel(DecodeArgs 
         }
         lds_fence();
     }
+
+    report_table_range(a.err, bad_id);
 
     // ---- epilogue: o = (f*(acc - PVS) + PVZ) / l with f = 4 or 16, lse = m + ln l ----------
     float l_tot[4] = {l_run[0], l_run[1], l_run[2], l_run[3]};

@@ -21,6 +21,11 @@ struct DecodeArgs {
     int scale_bf16;                  // k_scale / v_scale hold bf16 steps instead of int8 exponents
     int gt, gc;                      // tokens per K group, channels per V vector (16, 32, 64 or 128)
     int v_bf16;                      // v_main holds bf16 rows [P,ps,H,D] instead of INT2 codes
+    // Extents of the planes the tables index: a page id outside [0, n_pages) or a group slot outside
+    // [0, n_gslots) is clamped into range (no access leaves the planes) and OMMX_ERR_TABLE_RANGE is
+    // OR-ed into *err (may be NULL).  0 = extent not given: ids are used as they are.
+    int n_pages, n_gslots;
+    int32_t* err;
 };
 
 // 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)
@@ -28,6 +33,19 @@ __host__ __device__ constexpr int relidx7_bytes(int k) { return (7 * k + 7) / 8;
 
 __device__ __forceinline__ int64_t table_at(const void* t, int64_t i, int i64) {
     return i64 ? static_cast<const int64_t*>(t)[i] : static_cast<const int32_t*>(t)[i];
+}
+
+// Page id / group slot as read from a table, held inside the plane; `bad` collects whether any was not.
+__host__ __device__ __forceinline__ int clamp_id(int id, int n, bool& bad) {
+    if (n > 0) {
+        const uint32_t u = static_cast<uint32_t>(id), top = static_cast<uint32_t>(n - 1);
+        bad |= u > top;                       // negative ids are huge as unsigned: one comparison
+        id = static_cast<int>(u < top ? u : top);
+    }
+    return id;
+}
+__device__ __forceinline__ void report_table_range(int32_t* err, bool bad) {
+    if (__any(bad) && err && (threadIdx.x & 63) == 0) atomicOr(err, OMMX_ERR_TABLE_RANGE);
 }
 
 __device__ __forceinline__ float apply_cap(float x, float cap) {

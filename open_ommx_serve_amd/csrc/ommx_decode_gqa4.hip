@@ -162,9 +162,13 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
             qraw[r] = *reinterpret_cast<const uint32_t*>(
                 a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
     }
-    const int per = ((((L + a.S - 1) / a.S) + 31) / 32) * 32;
-    const int n_begin = per * sp;
-    const int n_end = min(n_begin + per, L);
+    // The 32-token groups are dealt out evenly: split s takes groups [s*G/S, (s+1)*G/S), so no two
+    // splits differ by more than one group and none is empty while G >= S.  (The combine weighs the
+    // states by their lse, -inf for an empty split, so it need not know this rule.)
+    if (L < 0) { L = 0; report_table_range(a.err, true); }      // a negative length: nothing packed, reported
+    const int G = (L + 31) >> 5;
+    const int n_begin = static_cast<int>((static_cast<int64_t>(sp) * G) / a.S) << 5;
+    const int n_end = min(static_cast<int>((static_cast<int64_t>(sp + 1) * G) / a.S) << 5, L);
 
     if (n_begin >= n_end) {       // an empty split: the state of nothing attended
         for (int r = 0; r < heads; ++r) {
@@ -215,10 +219,12 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
             gsl[g] = *reinterpret_cast<const int*>(rg_b + ((uint32_t)gi << tsh));
         }
     };
+    bool bad_id = false;            // a table entry outside the planes was seen (and clamped)
     u32x4 kr[2], vr[2];
     u32x2 vzp;
     uint32_t vsc, vrow;
     auto fetch_k = [&]() {          // K code row of this lane's token; remembers the row for fetch_v
+        pg1 = clamp_id(pg1, a.n_pages, bad_id);
         vrow = (uint32_t)((pg1 << ps_sh) + ps1);
         const uint64_t ro = (uint64_t)vrow * row_bytes;
         kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
@@ -243,7 +249,7 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         // this way the loads take a scalar base and a 32-bit lane offset)
         uint32_t lane_b = lane;
         asm volatile("" : "+v"(lane_b));
-        const uint32_t gs = __builtin_amdgcn_readfirstlane(gsl[g]);
+        const uint32_t gs = __builtin_amdgcn_readfirstlane(clamp_id(gsl[g], a.n_gslots, bad_id));
         const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + kvh_s) * D;
         g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
         g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
@@ -646,6 +652,8 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         lds_fence();
     }
 
+    report_table_range(a.err, bad_id);
+
     // ---- epilogue: o = (f*(acc - sum p*2^e) + sum p*zp) / l, f = 16 or 4; lse = m + ln l ----------
     // sums live in the lanes of the same column j: rows 0-3 (kq 0) zero points, 4-7 (kq 1) steps, 8 (kq 2) ones
     const int h = j & 3, x = j >> 2;
@@ -676,9 +684,6 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         if (x == 0 && kq == 0) {
             const float mt = h == 0 ? m_run[0] : (h == 1 ? m_run[1] : (h == 2 ? m_run[2] : m_run[3]));
             dst[D] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
-#ifdef OMMX_DBG
-            if (sp == 0) { float* dbg = dst + (int64_t)(a.S - sp) * a.al_s; dbg[0] = mt; dbg[1] = l_tot; dbg[2] = m_run[0]; dbg[3] = m_run[1]; dbg[4] = m_run[2]; dbg[5] = m_run[3]; }
-#endif
         }
     }
 }

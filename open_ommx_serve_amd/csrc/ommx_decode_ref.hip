@@ -26,7 +26,8 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
     int64_t* s_row = reinterpret_cast<int64_t*>(s_al + 8);   // [32]
 
     const int b = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z, tid = threadIdx.x;
-    const int L = a.seq[b];
+    const int L = max(a.seq[b], 0);      // a negative length: nothing packed, reported
+    if (a.seq[b] < 0 && a.err && tid == 0) atomicOr(a.err, OMMX_ERR_TABLE_RANGE);
     const int per = ((((L + a.S - 1) / a.S) + a.gt - 1) / a.gt) * a.gt;      // paged_decode.py:1429-1430
     const int n_begin = per * sp;
     const int n_end = min(n_begin + per, L);
@@ -53,7 +54,11 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
         int64_t gidx_u[2] = {0, 0};
         for (int u = 0; u < nsub; ++u) {
             const int gi = min(g_first + u, (n_end - 1) / gt);
-            const int64_t gslot = table_at(a.rg, b * a.rg_s + a.gbase + gi, a.i64);
+            int64_t gslot = table_at(a.rg, b * a.rg_s + a.gbase + gi, a.i64);
+            if (a.n_gslots > 0 && (gslot < 0 || gslot >= a.n_gslots)) {      // held inside the plane, reported
+                gslot = gslot < 0 ? 0 : a.n_gslots - 1;
+                if (a.err && tid == 0) atomicOr(a.err, OMMX_ERR_TABLE_RANGE);
+            }
             gidx_u[u] = (gslot * a.Hkv + kvh) * D;
         }
         for (int i = tid; i < nsub * D; i += 256) {
@@ -68,7 +73,12 @@ __global__ void __launch_bounds__(256) decode_splitkv_ref_kernel(DecodeArgs a) {
             int64_t prow = 0;
             if (n < n_end) {
                 const int64_t p = (int64_t)n + (int64_t)a.gbase * gt + a.off;
-                prow = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64) * a.ps + p % a.ps;
+                int64_t page = table_at(a.rt, b * a.rt_s + p / a.ps, a.i64);
+                if (a.n_pages > 0 && (page < 0 || page >= a.n_pages)) {
+                    page = page < 0 ? 0 : a.n_pages - 1;
+                    if (a.err) atomicOr(a.err, OMMX_ERR_TABLE_RANGE);
+                }
+                prow = page * a.ps + p % a.ps;
             }
             s_row[tid] = prow;
         }

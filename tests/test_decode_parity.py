@@ -103,20 +103,21 @@ def test_long_context_64k_permuted_all_split_counts():
     assert case.b_seq_len.tolist() == [65472]
     assert case.algorithmic_bytes() == 65472 * 8 * 132 + 64 * 8 * 128 * 4
     want = _oracle(case)
-    for S in (1, 8, 32, 64, None):
+    for S in (1, 8, 32, 64, 384, None):
         _check(_run(case, num_kv_splits=S), want, f"S{S}")
     _check(_run(case, num_kv_splits=64, ref_kernel=True), want, "ref S64")
 
 
 def test_long_context_128k_int64_tables_and_the_split_limit():
-    """ctx 131072 (the longest the reference serves), int64 tables, 256 splits (the limit) and
+    """ctx 131072 (the longest the reference serves), int64 tables, 512 splits (the limit) and
     odd split counts that leave the last splits short or empty."""
     case = build_decode_case([131072], seed=43, permute_tables=True, sparse_frac=0.005,
                              table_dtype=torch.int64)
     assert case.b_seq_len.tolist() == [131008]
     want = _oracle(case, dtype=torch.float32)
-    for S in (None, 256, 255, 100, 3):
+    for S in (None, 512, 256, 255, 100, 3):
         _check(_run(case, num_kv_splits=S), want, f"S{S}")
+    _check(_run(case, num_kv_splits=300, ref_kernel=True), want, "ref S300")
 
 
 @pytest.mark.parametrize("ref_kernel", [False, True])
@@ -510,3 +511,30 @@ def test_randomised_shapes_two_kernels_and_the_oracle():
             f2 = torch.isfinite(wl)
             if f2.any():
                 assert ((fast[1].double()[f2] - wl[f2]).abs() - 1e-5 * wl[f2].abs()).max().item() <= 2e-3, what
+
+
+def test_plane_extents_are_passed_and_in_range_tables_raise_no_flag():
+    """The launcher hands the plane extents to the kernels, which clamp every table entry into them
+    and report one that was outside.  With tables in range nothing is reported (both kernels);
+    a negative packed length counts as nothing packed and is reported."""
+    from open_ommx_serve_amd.attention import _hip
+    case = build_decode_case([2048 + 40, 777], seed=9, permute_tables=True, sparse_frac=0.005)
+    want = _oracle(case)
+    for ref in (False, True):
+        err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+        _check(_run(case, ref_kernel=ref, err_flag=err), want, f"ref={ref}")
+        assert int(err.item()) == 0
+    neg = case.b_seq_len.clone()
+    neg[1] = -5
+    err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+    B, Hq, D = case.q.shape
+    o = torch.full((B, Hq, D), float("nan"), dtype=torch.float32, device=case.q.device)
+    lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=case.q.device)
+    args = list(case.decode_args(o, lse))
+    args[-1] = neg
+    ommx_paged_decode_attention_canonical(*args, err_flag=err, **case.decode_kwargs())
+    torch.cuda.synchronize()
+    assert int(err.item()) & _hip.ERR_TABLE_RANGE
+    assert torch.isfinite(o).all()
+    # request 1 attends its tail rows only; request 0 is untouched
+    assert (o[0].cpu().double() - want[0][0]).abs().max().item() <= MAX_ABS

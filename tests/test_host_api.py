@@ -33,7 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     for n in names:
         assert getattr(raw, n) is not None, n
     assert set(_hip.exported_symbols()) == set(names)
-    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 5
+    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 6
 
 
 def test_default_decision_table_is_the_exact_arithmetic_one():
@@ -95,6 +95,12 @@ def test_split_heuristic_bounds():
     assert auto_num_kv_splits(32704, 8, 8, 256, 8, mean_seq_len=32704) == 32
     assert auto_num_kv_splits(65472, 1, 8, 256, mean_seq_len=65472) == 256
     assert 1 <= auto_num_kv_splits(1, 1, 1, 256) <= 256
+    # the kernel that keeps three workgroups per compute unit deals groups out evenly: fill the chip
+    assert auto_num_kv_splits(65472, 1, 8, 256, resident=3) == 256          # fewer than four steps per wave at 384
+    assert auto_num_kv_splits(960, 1, 8, 256, resident=3) == 30
+    assert auto_num_kv_splits(65472, 2, 8, 256, mean_seq_len=65472, resident=3) == 192
+    assert auto_num_kv_splits(10 ** 6, 1, 8, 1024, resident=3) <= 512
+    assert auto_num_kv_splits(131008, 1, 8, 256, resident=3) == 384         # 128K tokens: 5.3 steps per wave
 
 
 def test_pack_argument_errors_match_the_reference():
@@ -250,3 +256,17 @@ def test_ring_ops_validate_before_touching_the_device():
         write_tokens(kh.float(), kh.float(), torch.zeros(1, dtype=torch.int64), kh[0, :1], kh[0, :1], 0, 0)
     with pytest.raises(ValueError, match="num_slots"):
         gather_tails(kh[0], kh[0], kh, kh, 0, 0, seq=torch.zeros(1, dtype=torch.int64))
+
+
+def test_table_id_clamp_arithmetic():
+    """The clamp every decode kernel applies to the page ids and group slots it reads: ids inside
+    the plane pass, anything else (negative ids included) lands on the nearest valid id and is
+    reported; an extent of 0 means not given."""
+    lib = _hip.load()
+    flag = ctypes.c_int(0)
+    for ident, extent, want, bad in [(0, 10, 0, 0), (9, 10, 9, 0), (10, 10, 9, 1), (10 ** 9, 10, 9, 1),
+                                     (-1, 10, 9, 1), (-2 ** 31, 10, 9, 1), (5, 1, 0, 1), (0, 1, 0, 0),
+                                     (123456, 0, 123456, 0), (-7, 0, -7, 0), (2 ** 31 - 1, 2 ** 31 - 1, 2 ** 31 - 2, 1)]:
+        got = lib.ommx_clamp_table_id(ident, extent, ctypes.byref(flag))
+        assert (got, flag.value) == (want, bad), (ident, extent, got, flag.value)
+        assert extent == 0 or 0 <= got < extent
