@@ -7,9 +7,11 @@ checks and exception types (``:2916-3064``, ``:3323-3325``), the workspace shape
 writes ``o`` and ``lse`` in place on the current stream, allocates nothing when
 ``attn_logits`` is passed, and never synchronises when ``max_seq_len`` is passed.
 
-Implemented on the device: the serving recipe (INT2 base, bitmap-indexed FP4 outliers with
-the dedicated map, int8 exponent scales, 32-token / 32-channel vectors).  The reference's
-environment knobs are not read; ``num_stages`` / ``num_warps`` / ``qzp_buf`` are accepted
+Implemented on the device: INT2 base with 0..16 FP4 outliers per vector behind any of the three
+index planes (bitmap, 7-bit position stream, combinadic rank), dedicated or base-shared outlier
+map, int8 exponent or bf16 step planes, 16/32/64/128-element vectors, INT2 or bf16 V.  The
+serving recipe (bitmap, 6 outliers, dedicated map, int8 exponents, 32/32 vectors, INT2 V) takes
+the fastest kernel; the library picks per call.  The reference's environment knobs are not read; ``num_stages`` / ``num_warps`` / ``qzp_buf`` are accepted
 and ignored (they tune Triton, not this kernel).
 """
 from __future__ import annotations
@@ -212,7 +214,7 @@ def ommx_paged_decode_attention_canonical(
         unsupported.append("q that is not bf16 with unit inner stride")
     if unsupported:
         raise NotImplementedError(
-            "the HIP decode kernel implements the serving recipe only; not: " + ", ".join(unsupported))
+            "not covered by the HIP decode kernels: " + ", ".join(unsupported))
     if combinadic_read and k > 0:
         # The kernels read positions, not ranks: the rank plane is unranked into a position plane
         # by one launch ahead of the decode (paged_decode.py:969-1010 unranks inside the tile loop

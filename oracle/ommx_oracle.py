@@ -13,22 +13,28 @@ checkout, ``ommx_gpu_serve/attention/``).
 Parity status of each function (what pins it, besides reading):
 
   fp4_encode / fp4_decode      closed form + the 16 fixed points + brute-force
-                               nearest-in-log check            (tests/test_oracle_codec.py)
+                               nearest-in-log check            (tests/test_oracle_pins.py)
   pack_int2 / unpack_int2      closed form, round trip
   bitmap_pack / bitmap_unpack  closed form, popcount / rank-rule invariants
   relidx7_pack / relidx7_unpack  closed form (7-bit LSB-first stream) against big-integer
                                arithmetic and hand-computed bytes; positions equal the
-                               bitmap's for the same input     (tests/test_oracle_codec.py)
+                               bitmap's for the same input; planes the reference packer
+                               wrote (tests/golden/variant_relidx7.npz, ..._k16_relidx7)
   combinadic_pack / _unpack    the combinatorial number system: every k-subset of a small set
                                enumerated in colexicographic order takes the ranks 0, 1, 2 ...
                                in turn; first / last subset, a hand-computed rank, field widths
-                               of the reference's recipes      (tests/test_oracle_pins.py)
+                               of the reference's recipes; a plane the reference packer
+                               wrote (tests/golden/variant_combinadic.npz)
   pow2_exponent                rule 2^rint(log2(x)) incl. exact-tie vectors
   select_outliers_signed       brute-force rank counting on small vectors with ties
   select_outliers_abs          the same, on magnitudes
-  pack_kv                      golden planes written by the reference packer itself
-                               (tests/golden/*.npz), plus all of the above
-  dequant_kv                   golden dequant of the same planes; encode/decode identity
+  pack_kv                      golden planes written by the reference packer itself: five
+                               blocks of the serving recipe (tests/golden/pack_*.npz) and one
+                               block per variant branch -- index planes, base-shared outliers,
+                               magnitude selector, free / bf16 steps, 16/64/128-element
+                               vectors with 0..16 outliers, bf16 V (tests/golden/variant_*.npz)
+  dequant_kv                   the reference's dequant of every one of those plane sets;
+                               encode/decode identity
   attend / decode_reference    softmax closed forms, fp64 cross-check, split-merge
                                associativity
   WindowSpec arithmetic        closed forms + the invariant recent <= seq-boundary < recent+gt

@@ -1,4 +1,5 @@
 """Shared fixtures.  Tests marked ``gpu`` need one ROCm GPU; the rest run on the CPU."""
+import json
 import os
 import sys
 
@@ -75,3 +76,45 @@ def assert_planes_equal(got, want_bits, what="", zero_sign_free=False):
             w = np.where(w == 0x8000, 0, w)
         bad = int((g != w).sum())
         assert bad == 0, f"{what} {name}: {bad} of {g.size} elements differ"
+
+
+# ---- one reference-written block per format variant (tests/golden/variant_*.npz) --------
+
+with open(os.path.join(GOLDEN_DIR, "variant_index.json")) as _f:
+    VARIANT_INDEX = json.load(_f)
+VARIANT_CASES = tuple(VARIANT_INDEX)
+ALL_PLANE_NAMES = PLANE_NAMES + ("k_oidx", "k_crank")
+
+
+def load_variant(name: str):
+    """``(arrays, recipe)`` of a variant fixture: raw plane bits plus the keyword arguments
+    the reference packer was called with."""
+    z = np.load(os.path.join(GOLDEN_DIR, f"variant_{name}.npz"))
+    return {k: z[k] for k in z.files}, dict(VARIANT_INDEX[name]["recipe"])
+
+
+def variant_planes(z, recipe):
+    """Plane dict (tensors + the metadata keys a dequant needs) of a variant fixture."""
+    planes = {p: (tensor_from_bits(z[p]) if p in z else None) for p in ALL_PLANE_NAMES}
+    planes.update(outliers_per_vector=recipe["outliers_per_vector"],
+                  group_tokens=recipe["group_tokens"], group_channels=recipe["group_channels"],
+                  outlier_repr=recipe["outlier_repr"], page_size=recipe["page_size"])
+    return planes
+
+
+def assert_variant_planes_equal(got, z, what=""):
+    """Every plane the reference wrote is matched bit for bit (dtype included); every plane it
+    left out must be absent from ``got`` as well."""
+    for name in ALL_PLANE_NAMES:
+        g = got.get(name)
+        if name not in z:
+            assert g is None, f"{what} {name}: reference wrote no such plane"
+            continue
+        assert g is not None, f"{what} {name}: plane missing"
+        want_dtype = VARIANT_INDEX[what]["planes"][name][0] if what in VARIANT_INDEX else None
+        if want_dtype:
+            assert str(g.dtype).replace("torch.", "") == want_dtype, f"{what} {name}: dtype {g.dtype}"
+        gb, w = bits_of(g), z[name]
+        assert gb.shape == w.shape, f"{what} {name}: shape {gb.shape} != {w.shape}"
+        bad = int((gb != w).sum())
+        assert bad == 0, f"{what} {name}: {bad} of {gb.size} elements differ"

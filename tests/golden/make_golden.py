@@ -10,6 +10,11 @@ invariant fixes, so it is recorded here as data: the inputs (bf16 bit patterns) 
 plane the reference writes for them, plus ``dequant_kv_canonical`` of those planes.  The
 fixtures are small ``.npz`` files; tests only read them.  Nothing from the reference's
 source text is stored.
+
+Besides the serving recipe (``pack_<case>.npz``) one small block per format variant is
+written (``variant_<name>.npz``): the other two index planes, base-shared outliers, the
+magnitude selector, steps that are not powers of two, bf16 step planes, 16/64/128-element
+vectors with up to 10 outliers, and bf16 V.  Each holds the recipe it was packed with.
 """
 from __future__ import annotations
 
@@ -29,6 +34,35 @@ SEEDS = {"tiny_ties": 101, "small_gauss": 202, "layer_outliers": 303, "wide_rang
 RECIPE = dict(outliers_per_vector=6, outlier_select="signed", outlier_repr="bitmap",
               k_format="i2f4", use_pow2=True, kv_outlier_map=True, kv_int8_scale=True,
               group_tokens=32, group_channels=32, page_size=16, v_format="i2")
+
+
+# name -> (recipe overrides, (T, H, D), seed)
+VARIANTS = {
+    "relidx7": (dict(outlier_repr="relidx7"), (128, 2, 64), 611),
+    "combinadic": (dict(outlier_repr="combinadic"), (128, 2, 64), 612),
+    "base_shared": (dict(kv_outlier_map=False), (128, 2, 64), 613),
+    "abs_select": (dict(outlier_select="abs"), (128, 2, 64), 614),
+    "abs_relidx7_k3": (dict(outlier_select="abs", outlier_repr="relidx7", outliers_per_vector=3),
+                       (64, 1, 64), 615),
+    "free_steps": (dict(use_pow2=False), (128, 2, 64), 616),
+    "bf16_steps": (dict(kv_int8_scale=False), (128, 2, 64), 617),
+    "gt64_gc64_k10": (dict(group_tokens=64, group_channels=64, outliers_per_vector=10,
+                           kv_outlier_map=False), (128, 1, 128), 618),
+    "gt64_gc64_k10_map": (dict(group_tokens=64, group_channels=64, outliers_per_vector=10),
+                          (128, 1, 64), 619),
+    "gt128_gc128_k10": (dict(group_tokens=128, group_channels=128, outliers_per_vector=10,
+                             kv_outlier_map=False), (256, 1, 128), 620),
+    "gt128_gc32_k16_relidx7": (dict(group_tokens=128, outliers_per_vector=16,
+                                    outlier_repr="relidx7"), (128, 1, 64), 621),
+    "gt16_k3": (dict(group_tokens=16, outliers_per_vector=3), (64, 2, 64), 622),
+    "gt16_gc16_k2": (dict(group_tokens=16, group_channels=16, outliers_per_vector=2),
+                     (64, 1, 64), 623),
+    "k0": (dict(outliers_per_vector=0), (64, 2, 64), 624),
+    "k1": (dict(outliers_per_vector=1), (64, 2, 64), 625),
+    "v_bf16": (dict(v_format="bf16"), (64, 2, 64), 626),
+    "v_bf16_bf16_steps": (dict(v_format="bf16", kv_int8_scale=False), (64, 1, 64), 627),
+}
+INDEX_PLANES = ("k_oidx", "k_crank")
 
 
 def _bits(t: torch.Tensor) -> np.ndarray:
@@ -60,6 +94,39 @@ def main(ref_root: str) -> None:
         print(name, {p: tuple(planes[p].shape) for p in PLANES})
     with open(os.path.join(HERE, "pack_index.json"), "w") as f:
         json.dump({"recipe": RECIPE, "torch": torch.__version__, "sha256": index}, f, indent=1)
+
+    vindex = {}
+    for name, (over, shape, seed) in VARIANTS.items():
+        g = torch.Generator().manual_seed(seed)
+        K, V = _variant_inputs(shape, g)
+        recipe = dict(RECIPE, **over)
+        planes = ommx_pack_kv_canonical_block(K, V, **recipe)
+        Kd, Vd = dequant_kv_canonical(planes)
+        out = {"K_bits": _bits(K), "V_bits": _bits(V),
+               "K_dq_bits": _bits(Kd), "V_dq_bits": _bits(Vd)}
+        held = []
+        for p in PLANES + INDEX_PLANES:
+            if torch.is_tensor(planes.get(p)):
+                out[p] = _bits(planes[p])
+                held.append(p)
+        np.savez_compressed(os.path.join(HERE, f"variant_{name}.npz"), **out)
+        vindex[name] = {"recipe": recipe, "shape": list(shape), "planes": {
+            p: [str(planes[p].dtype).replace("torch.", ""), list(planes[p].shape)] for p in held}}
+        print(name, vindex[name]["planes"])
+    with open(os.path.join(HERE, "variant_index.json"), "w") as f:
+        json.dump(vindex, f, indent=1)
+
+
+def _variant_inputs(shape, g: torch.Generator):
+    """Gaussian rows with a few heavy channels, some exact ties and a constant vector."""
+    T, H, D = shape
+    K = torch.randn(T, H, D, generator=g)
+    V = torch.randn(T, H, D, generator=g) * 2.0
+    K[:, :, [3, 17, 40]] *= 9.0
+    K[:, 0, 5] = torch.randint(-3, 4, (T,), generator=g).float() * 0.5      # many ties
+    K[:, 0, 6] = 0.25                                                        # constant
+    V[1, 0, :16] = 1.0
+    return K.to(torch.bfloat16), V.to(torch.bfloat16)
 
 
 def _case_inputs(name: str, g: torch.Generator):

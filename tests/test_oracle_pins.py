@@ -8,8 +8,9 @@ import pytest
 import torch
 
 import oracle.ommx_oracle as O
-from conftest import (GOLDEN_CASES, assert_planes_equal, bits_of, load_golden,
-                      tensor_from_bits)
+from conftest import (GOLDEN_CASES, VARIANT_CASES, assert_planes_equal,
+                      assert_variant_planes_equal, bits_of, load_golden, load_variant,
+                      tensor_from_bits, variant_planes)
 
 
 # ---- the composed packer against the reference's own output ---------------------------
@@ -28,6 +29,30 @@ def test_dequant_matches_reference_golden(name):
     planes = {k: tensor_from_bits(z[k]) for k in z if not k.endswith("_bits")}
     planes["outliers_per_vector"] = 6
     Kd, Vd = O.dequant_kv(planes)
+    assert np.array_equal(bits_of(Kd), z["K_dq_bits"])
+    assert np.array_equal(bits_of(Vd), z["V_dq_bits"])
+
+
+def _oracle_kwargs(recipe):
+    kw = dict(recipe)
+    assert kw.pop("k_format") == "i2f4"
+    return kw
+
+
+@pytest.mark.parametrize("name", VARIANT_CASES)
+def test_pack_variant_matches_reference_golden_planes(name):
+    """Each format variant's branch of the packer, against planes the reference packer wrote
+    for the same block with the same keyword arguments."""
+    z, recipe = load_variant(name)
+    K, V = tensor_from_bits(z["K_bits"]), tensor_from_bits(z["V_bits"])
+    planes = O.pack_kv(K, V, **_oracle_kwargs(recipe))
+    assert_variant_planes_equal(planes, z, what=name)
+
+
+@pytest.mark.parametrize("name", VARIANT_CASES)
+def test_dequant_variant_matches_reference_golden(name):
+    z, recipe = load_variant(name)
+    Kd, Vd = O.dequant_kv(variant_planes(z, recipe))
     assert np.array_equal(bits_of(Kd), z["K_dq_bits"])
     assert np.array_equal(bits_of(Vd), z["V_dq_bits"])
 

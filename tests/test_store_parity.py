@@ -5,7 +5,8 @@ import pytest
 import torch
 
 import oracle.ommx_oracle as O
-from conftest import (GOLDEN_CASES, PLANE_NAMES, assert_planes_equal, bits_of, load_golden,
+from conftest import (GOLDEN_CASES, PLANE_NAMES, VARIANT_CASES, assert_planes_equal,
+                      assert_variant_planes_equal, bits_of, load_golden, load_variant,
                       tensor_from_bits)
 from open_ommx_serve_amd.attention import pack as hip_pack
 from open_ommx_serve_amd.attention.pack import (alloc_planes, ommx_pack_kv_canonical_block,
@@ -37,6 +38,19 @@ def test_store_matches_reference_golden_planes(name):
                 "req_to_token", "req_to_group", "k_oidx", "k_crank"):
         assert key in planes
     assert planes["k_field_bytes"] == 4 and planes["k_oidx"] is None
+
+
+@pytest.mark.parametrize("name", VARIANT_CASES)
+def test_store_variant_matches_reference_golden_planes(name):
+    """One block per format variant (index planes, base-shared outliers, magnitude selector,
+    free and bf16 steps, 16/64/128-element vectors, bf16 V): every plane the reference packer
+    wrote for it, bit for bit, and no plane it did not write."""
+    z, recipe = load_variant(name)
+    K, V = tensor_from_bits(z["K_bits"]), tensor_from_bits(z["V_bits"])
+    planes = ommx_pack_kv_canonical_block(K.cuda(), V.cuda(), **recipe)
+    assert_variant_planes_equal(planes, z, what=name)
+    assert planes["outlier_repr"] == recipe["outlier_repr"]
+    assert planes["group_tokens"] == recipe["group_tokens"]
 
 
 @pytest.mark.parametrize("seed,T,H,D", [(1, 32, 1, 32), (2, 96, 3, 64), (3, 256, 8, 128),
