@@ -8,17 +8,23 @@ operator (split-KV kernel + combine kernel) on one MI355X, Llama-3.1-8B attentio
 One step = one decode call over one batch: the split-KV launch followed by the combine
 launch, operands resident in HBM, workspace preallocated.  Steps are replayed from HIP
 graphs of 32 consecutive steps (the 32 layers of one model forward; eager launches if
-capture fails), so K is rounded up to a multiple of 32.  Prints ONE JSON line.  ``value`` is the p50 over the K timed
-steps at the headline context; ``roofline`` is the split-KV kernel alone (algorithmic bytes
-of the packed planes it must read over its average duration, against 8 TB/s);
-``store`` is the quantize-on-store kernel over the same cache (its own roofline figures);
-``cpu_baseline`` is the CPU checker (dequantise-then-attend, torch on the host cores) on
-the same workload, a bounded number of runs, used here also for the post-timing parity
-check.
+capture fails), so K is rounded up to a multiple of 32 (``steps_requested`` /
+``warmup_requested`` keep what was asked for).  Every one of the 32 layers reads its own
+copy of the cache, query, tail and workspace, at its own addresses, as the layers of a model
+do: 32 x 69 MB at the headline context, far beyond the 256 MB last-level cache, so every
+step reads its planes from HBM.  Before anything is timed the outputs are filled with NaN,
+every layer is run once and compared with the CPU checker (``parity_before_timing``); a
+mismatch ends the run.  Prints ONE JSON line.  ``value`` is the p50 over the K timed steps
+at the headline context; ``roofline`` is the split-KV kernel alone (algorithmic bytes of the
+packed planes it must read over its average duration, against 8 TB/s); ``store`` is the
+quantize-on-store kernel over the same cache (its own roofline figures); ``cpu_baseline``
+is the CPU checker (dequantise-then-attend, torch on the host cores) timed on the same
+workload for a bounded number of runs, and on the 1024-token configuration.
 """
 from __future__ import annotations
 
 import argparse
+import dataclasses
 import json
 import os
 import statistics
@@ -77,9 +83,26 @@ def _time_steps(fn, calls, warmup, per_call=1):
     return wall_ms, [a.elapsed_time(b) * 1e3 / per_call for a, b in ev]
 
 
-def _make_runner(case, splits=None):
-    """Closures launching (full step, split-KV kernel only) with fixed buffers."""
+def _layer_copies(case, n):
+    """``n`` cases with the same contents at different addresses: the caches of n layers."""
     import torch
+
+    def dup(v):
+        return v.clone() if torch.is_tensor(v) else v
+    out = [case]
+    for _ in range(n - 1):
+        out.append(dataclasses.replace(
+            case, planes={k: dup(v) for k, v in case.planes.items()}, q=case.q.clone(),
+            k_tail=case.k_tail.clone(), v_tail=case.v_tail.clone(),
+            req_to_token=case.req_to_token.clone(), req_to_group=case.req_to_group.clone()))
+    return out
+
+
+def _make_runner(cases, splits=None):
+    """Closures ``step(i)`` / ``stage1(i)`` launching the full step / the split-KV kernel alone
+    on layer ``i`` with fixed buffers; ``outs[i] = (o, lse)`` of that layer."""
+    import torch
+    case = cases[0]
     from open_ommx_serve_amd.attention import _hip
     from open_ommx_serve_amd.attention.paged_decode import (auto_num_kv_splits, make_attn_logits,
                                                             ommx_paged_decode_attention_canonical)
@@ -92,19 +115,19 @@ def _make_runner(case, splits=None):
     mean_len = sum(case.packed_lens) / len(case.packed_lens)
     S = splits or auto_num_kv_splits(kw["max_seq_len"], B, case.kv_heads, n_cu, Hq // case.kv_heads,
                                      mean_seq_len=mean_len, resident=3 if Hq // case.kv_heads <= 4 else 2)
-    ws = make_attn_logits(B, Hq, S, D, dev)
-    o = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
-    lse = torch.empty(B, Hq, dtype=torch.float32, device=dev)
-    args = case.decode_args(o, lse)
+    wss = [make_attn_logits(B, Hq, S, D, dev) for _ in cases]
+    outs = [(torch.empty(B, Hq, D, dtype=torch.float32, device=dev),
+             torch.empty(B, Hq, dtype=torch.float32, device=dev)) for _ in cases]
+    argss = [c.decode_args(*ol) for c, ol in zip(cases, outs)]
+    kws = [c.decode_kwargs() for c in cases]
 
-    def step():
-        ommx_paged_decode_attention_canonical(*args, num_kv_splits=S, attn_logits=ws, **kw)
+    def step(i=0):
+        ommx_paged_decode_attention_canonical(*argss[i], num_kv_splits=S, attn_logits=wss[i], **kws[i])
 
     lib = _hip.load()
-    p = case.planes
-    stream = torch.cuda.current_stream(dev)
 
-    def stage1():
+    def stage1(i=0):
+        case, ws, p = cases[i], wss[i], cases[i].planes
         rc = lib.ommx_decode_splitkv(
             case.q.data_ptr(), case.q.stride(0), case.q.stride(1),
             p["k_base"].data_ptr(), p["k_scale"].data_ptr(), p["k_zp"].data_ptr(),
@@ -120,7 +143,32 @@ def _make_runner(case, splits=None):
             torch.cuda.current_stream(dev).cuda_stream)
         _hip.check(rc, "ommx_decode_splitkv")
 
-    return step, stage1, o, lse, S
+    return step, stage1, outs, S
+
+
+def _parity_gate(case, outs, run_layer, want=None):
+    """NaN-fill the outputs, run every layer once, compare each with the CPU checker's result for
+    the (shared) inputs.  Returns ``(figures, want)``; raises on a mismatch."""
+    import torch
+    for o, lse in outs:
+        o.fill_(float("nan"))
+        lse.fill_(float("nan"))
+    for i in range(len(outs)):
+        run_layer(i)
+    torch.cuda.synchronize()
+    if want is None:
+        want = _cpu_reference(case, 1)[1]
+    wo, wl = want[0].double(), want[1].double()
+    worst = {"max_abs": 0.0, "mean_abs": 0.0, "lse_max_abs": 0.0}
+    for i, (o, lse) in enumerate(outs):
+        err = (o.cpu().double() - wo).abs()
+        lerr = (lse.cpu().double() - wl).abs()
+        fig = {"max_abs": float(err.max()), "mean_abs": float(err.mean()), "lse_max_abs": float(lerr.max())}
+        if not (fig["max_abs"] <= 2e-3 and fig["mean_abs"] <= 2e-4 and fig["lse_max_abs"] <= 2e-3):
+            raise RuntimeError(f"parity failure before timing, layer {i}: {fig}")
+        worst = {k: max(worst[k], fig[k]) for k in worst}
+    worst["layers_checked"] = len(outs)
+    return worst, want
 
 
 def _time_store(ctx, kv_heads=8, head_dim=128):
@@ -157,8 +205,10 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
     request is written (the launch advances the device sequence counter), the sink + recent rows are
     gathered with the window arithmetic on the device, then split-KV + combine.  These four launches
     are one HIP graph; after each replay the host advances its mirror and packs the groups that
-    completed (one store launch, outside the timed replay).  Every request gets the same synthetic
-    rows (the kernels do not care).  Returns the JSON object."""
+    completed (one store launch, outside the timed replay), so the gather is told that the planes
+    lag the sequence by one token.  Every request gets the same synthetic rows (the kernels do not
+    care).  The outputs of the first replay whose token completes a group, and of the last replay,
+    are compared with the CPU checker.  Returns the JSON object."""
     import torch
     from open_ommx_serve_amd.attention import MultiSeqKVPool, WindowSpec, gather_tails, write_tokens
     from open_ommx_serve_amd.attention.paged_decode import (auto_num_kv_splits, make_attn_logits,
@@ -194,7 +244,7 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
         gather_tails(pool.k_hist, pool.v_hist, d["kt"], d["vt"], pool._ring_sink, pool._ring_rec,
                      seq=d["seq_dev"], slots=d["sel"], b_tail_len=d["b_tail"], b_seq_len=d["b_seq"],
                      window_sink=win.sink_tokens, window_recent=win.recent_window,
-                     group_tokens=win.group_tokens, err_flag=pool.err_flag)
+                     group_tokens=win.group_tokens, packed_lag=1, err_flag=pool.err_flag)
         ommx_paged_decode_attention_canonical(
             q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"], pl["v_main"], pl["v_scale"],
             pl["v_zp"], d["kt"], d["vt"], d["b_tail"], o, lse, pl["req_to_token"], pl["req_to_group"],
@@ -212,7 +262,30 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
             step()
     torch.cuda.current_stream().wait_stream(stream)
     d["seq_dev"].copy_(seq0)                      # capture ran no kernel
-    us, packed = [], 0
+    def check(s):
+        """Replay s has run and the host has not packed yet: request 0 against the CPU checker."""
+        import oracle.ommx_oracle as O
+        n = ctx + s + 1
+        edge = win.boundary(n - 1)                 # what the planes hold
+        rows = list(range(min(n, win.sink_tokens))) + list(range(edge, n))
+        if int(d["b_seq"][0]) != edge - win.sink_tokens or int(d["b_tail"][0]) != len(rows):
+            raise RuntimeError(f"pool step {s}: lengths {int(d['b_seq'][0])}/{int(d['b_tail'][0])}, "
+                               f"expected {edge - win.sink_tokens}/{len(rows)}")
+        if not torch.equal(d["kt"][0, :len(rows)].cpu(), K[rows]) or \
+                not torch.equal(d["vt"][0, :len(rows)].cpu(), V[rows]):
+            raise RuntimeError(f"pool step {s}: gathered tail rows differ from the appended rows")
+        planes = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in pool.request_planes(0).items()}
+        G = planes["k_scale"].shape[0]
+        wo, _ = O.decode_reference(q[:1].cpu(), planes, d["kt"][:1].cpu(), d["vt"][:1].cpu(), [len(rows)],
+                                   torch.arange(2 * G).reshape(1, -1), torch.arange(G).reshape(1, -1),
+                                   [edge - win.sink_tokens], sm_scale=D ** -0.5, page_size=win.page_size,
+                                   dtype=torch.float32)
+        err = (o[:1].cpu().double() - wo.double()).abs()
+        if not (float(err.max()) <= 2e-3 and float(err.mean()) <= 2e-4):
+            raise RuntimeError(f"pool step {s}: parity failure, max {float(err.max())} mean {float(err.mean())}")
+        return float(err.max())
+
+    us, packed, checked = [], 0, {}
     t0 = time.perf_counter()
     for s in range(warmup + steps):
         newK.copy_(Kd[ctx + s].unsqueeze(0).expand(B, H, D))
@@ -221,6 +294,10 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
         a.record()
         graph.replay()
         b.record()
+        completes = win.boundary(ctx + s + 1) != win.boundary(ctx + s)
+        if (completes and "group_completing_step" not in checked) or s == warmup + steps - 1:
+            torch.cuda.synchronize()
+            checked["group_completing_step" if completes else "last_step"] = round(check(s), 6)
         packed += pool._advance_host_and_pack(range(B))      # host mirror + pack of completed groups
         torch.cuda.synchronize()
         if s == warmup:
@@ -241,7 +318,7 @@ def _pool_step(batch, ctx, q_heads, steps, warmup, splits=0):
                                    f"ctx {ctx} growing by one token per step, ring history, page 16",
                        "num_kv_splits": S, "launch": "hip_graph", "bytes_per_step": nbytes,
                        "hbm_frac_step": round(nbytes / (p50 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                       "groups_packed_between_replays": packed,
+                       "groups_packed_between_replays": packed, "parity_max_abs": checked,
                        "note": "ms_per_step is wall time per step including the host mirror, the pack "
                                "launches and a synchronisation per step"},
             "roofline": None, "cpu_baseline": None}
@@ -317,23 +394,30 @@ def main() -> int:
             lens = torch.randint(1024, ctx + 1, (args.batch,), generator=g).tolist()
         case = build_decode_case(lens, q_heads=args.q_heads, seed=42, permute_tables=True,
                                  sparse_frac=0.005)
-        step, stage1, o, lse, S = _make_runner(case, args.splits or None)
+        # one cache per layer while they fit in 48 GiB, and never fewer than 4 (4 x 69 MB is
+        # already past the 256 MB last-level cache at the headline context)
+        n_copies = max(4, min(LAYERS, (48 << 30) // max(1, case.algorithmic_bytes())))
+        cases = _layer_copies(case, n_copies)
+        step, stage1, outs, S = _make_runner(cases, args.splits or None)
+        parity, want = _parity_gate(case, outs, step)
+        _parity_gate(case, outs, lambda i: (stage1(i), step(i)), want)   # both closures, same result
         # one model forward runs this operator once per layer inside a single graph, so the
         # steps are timed in graphs of LAYERS consecutive steps (steps is rounded up to that)
         def layers():
-            for _ in range(LAYERS):
-                step()
+            for i in range(LAYERS):
+                step(i % n_copies)
         run, mode = _graph_or_eager(layers)
         calls = -(-steps // LAYERS)
         wall_ms, us = _time_steps(run, calls, max(1, -(-warmup // LAYERS)), per_call=LAYERS)
         # the kernel alone: REP launches back to back inside one graph, so that the event
         # pair brackets kernel time and not the launch latency of a one-kernel graph
         def stage1_rep():
-            for _ in range(STAGE1_REP):
-                stage1()
+            for i in range(STAGE1_REP):
+                stage1(i % n_copies)
         run1, _ = _graph_or_eager(stage1_rep)
         _, us1 = _time_steps(run1, max(5, steps // STAGE1_REP), 2, per_call=STAGE1_REP)
-        return dict(case=case, o=o, lse=lse, S=S, mode=mode, wall_ms=wall_ms, us=us, us1=us1)
+        return dict(case=case, outs=outs, S=S, mode=mode, wall_ms=wall_ms, us=us, us1=us1,
+                    parity=parity, want=want, layer_copies=n_copies)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
@@ -374,26 +458,35 @@ def main() -> int:
     if headline and not args.no_store:
         store = _time_store(args.ctx)
 
+    # the outputs the timed replays left behind must still be the checked ones
+    wo = m["want"][0].double()
+    after = max(float((o.cpu().double() - wo).abs().max()) for o, _ in m["outs"])
+    if not after <= 2e-3:
+        print(f"PARITY FAILURE after timing: max_abs {after}", file=sys.stderr)
+        return 1
+    parity = dict(m["parity"], max_abs_after_timing=after)
+
     cpu = None
-    parity = None
     if not args.no_cpu_baseline:
         runs = 15 if args.ctx >= 32768 else 40          # about ten seconds of CPU work
-        times, (wo, wl) = _cpu_reference(case, runs)
-        err = (m["o"].cpu().double() - wo.double()).abs()
-        parity = {"max_abs": float(err.max()), "mean_abs": float(err.mean())}
-        if parity["max_abs"] > 2e-3 or parity["mean_abs"] > 2e-4:
-            print(f"PARITY FAILURE after timing: {parity}", file=sys.stderr)
-            return 1
+        times, _ = _cpu_reference(case, runs)
+        small = build_decode_case([1024], q_heads=args.q_heads, seed=42, permute_tables=True,
+                                  sparse_frac=0.005)
+        times_1k, _ = _cpu_reference(small, 200)
         cpu = {"value": round(statistics.median(times) * 1e6, 1), "unit": "us/step/layer",
                "cores": torch.get_num_threads(), "kind": "port",
                "sample": f"{runs} runs of the same ctx-{args.ctx} step (dequantise all planes, "
-                         f"fp32 attention per q head) on {os.cpu_count()} logical CPUs"}
+                         f"fp32 attention per q head) on {os.cpu_count()} logical CPUs",
+               "ctx1024": {"value": round(statistics.median(times_1k) * 1e6, 1), "unit": "us/step/layer",
+                           "sample": "200 runs of the ctx-1024 step of the same shape (the "
+                                     "configuration the reference's CPU path is quoted on)"}}
 
     out = {
         "metric": "p50 decode-attn us/step/layer, 8B shape bs1" if headline
                   else "p50 decode-attn us/step/layer",
         "value": round(p50, 3), "unit": "us/step/layer", "n_gpus": 1,
         "steps": -(-args.steps // LAYERS) * LAYERS, "warmup": -(-args.warmup // LAYERS) * LAYERS,
+        "steps_requested": args.steps, "warmup_requested": args.warmup,
         "ms_per_step": round(m["wall_ms"], 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": round(p50 / H200_P50_US_64K, 5) if (args.ctx == 65536 and headline) else None,
         "dtype": "u8 planes, bf16 q, f32 accumulate", "data": "synthetic",
@@ -403,7 +496,7 @@ def main() -> int:
                                f"{' in all' if args.ragged else ''} + {int(case.b_tail_len[0])} bf16 "
                                f"tail rows), page 16, permuted page/group tables, K outliers 4 "
                                f"channels x12 + 0.5% x8",
-                   "num_kv_splits": m["S"], "launch": m["mode"],
+                   "num_kv_splits": m["S"], "launch": m["mode"], "layer_caches": m["layer_copies"],
                    "bytes_per_step": step_bytes, "hbm_frac_step": round(
                        step_bytes / (p50 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
                    "ladder": ladder, "baseline_note": "vs_baseline = value / 563 us "
@@ -414,7 +507,7 @@ def main() -> int:
                      "bytes_per_launch": packed_bytes,
                      "avg_kernel_us": round(k1, 3)},
         "cpu_baseline": cpu,
-        "parity_after_timing": parity,
+        "parity_before_timing": parity,
         "store": store,
     }
     print(json.dumps(out))

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 6   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
+#define OMMX_ABI_VERSION 7   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
                                 5: decode without a workspace argument; 6: plane extents + error flag on
                                 the decode entry points, up to 512 splits */
 
@@ -289,7 +289,13 @@ int ommx_ring_write(const uint16_t* k, const uint16_t* v, int64_t k_stride_b, in
  *                     [0,min(sink,seq)) ++ [boundary,seq); and writes
  *                     b_tail_len[b] = min(rows, T), b_seq_len[b] = max(boundary-sink, 0)
  *                     (either may be NULL).  Rows past the count repeat position 0; the
- *                     decode kernels mask them by b_tail_len.
+ *                     decode kernels mask them by b_tail_len.  packed_lag (0..group_tokens)
+ *                     is the number of tokens appended since the planes were last packed:
+ *                     the boundary is then the one of seq - packed_lag, so a step that
+ *                     appends and decodes before the host packs (one graph replay) reads
+ *                     the group its token may have completed from the ring, not from a
+ *                     group slot nobody has written yet.  T must hold sink + recent +
+ *                     group_tokens - 1 + packed_lag rows, and so must the ring.
  *   tail_idx != NULL  int64[B,T] explicit absolute positions (kv_store_ops.py:42-61,71-76
  *                     _kv_gather_tail / gather_tail); the length outputs are not written.
  * Positions map to history rows as in ommx_ring_write; a row outside the history sets
@@ -300,7 +306,7 @@ int ommx_tail_gather(const uint16_t* k_hist, const uint16_t* v_hist, int64_t his
                      const int64_t* tail_idx,
                      uint16_t* k_tail, uint16_t* v_tail, int32_t* b_tail_len, int32_t* b_seq_len,
                      int B, int T, int H, int D, int sink_rows, int recent_rows, int group_tokens,
-                     int ring_span, int32_t* err_flag, void* stream);
+                     int ring_span, int packed_lag, int32_t* err_flag, void* stream);
 
 /*
  * Merge of partial attention states over disjoint KV segments (cascade / context-parallel /

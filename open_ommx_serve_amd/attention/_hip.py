@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
-ABI_VERSION = 6
+ABI_VERSION = 7
 INDEX_BITMAP, INDEX_RELIDX7, INDEX_COMBINADIC = 0, 1, 2
 SCALE_POW2_INT8, SCALE_POW2_BF16, SCALE_BF16 = 0, 1, 2
 
@@ -70,7 +70,7 @@ _SIGNATURES = {
     "ommx_index_plane_bytes": (_I, [_I, _I, _I]),
     "ommx_index_convert": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]),
     "ommx_tail_gather": (_I, [_P, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P,
-                              _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+                              _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
 }
 
 

@@ -195,7 +195,7 @@ class CanonicalKVStore:
         if pos.dtype != torch.int64 or pos.device != self.device:
             pos = pos.to(self.device, torch.int64)
         write_token(self.k_hist, self.v_hist, pos.reshape(-1)[:1].contiguous(), kb, vb,
-                    self._ring_sink, self._ring_rec)
+                    self._ring_sink, self._ring_rec, err_flag=self.err_flag)
 
     def advance_to(self, seq_len: int) -> int:
         """Set the sequence length and pack completed groups (kv_store.py:387-395)."""
@@ -208,7 +208,8 @@ class CanonicalKVStore:
         ``k_tail`` / ``v_tail [1, T, H, D]``; launch-only (kv_store.py:397-427)."""
         if tail_idx.device != self.device:
             tail_idx = tail_idx.to(self.device)
-        gather_tail(self.k_hist, self.v_hist, tail_idx, k_tail, v_tail, self._ring_sink, self._ring_rec)
+        gather_tail(self.k_hist, self.v_hist, tail_idx, k_tail, v_tail, self._ring_sink, self._ring_rec,
+                    err_flag=self.err_flag)
 
     def append_block(self, K: torch.Tensor, V: torch.Tensor) -> None:
         """Stash a prefill block ``[T, H, D]`` and pack its completed groups (kv_store.py:429-490)."""
@@ -339,7 +340,8 @@ class CanonicalKVStore:
         vt = torch.empty_like(kt)
         if n:
             ti = torch.tensor(idx, dtype=torch.int64).to(self.device)
-            gather_tail(self.k_hist, self.v_hist, ti, kt, vt, self._ring_sink, self._ring_rec)
+            gather_tail(self.k_hist, self.v_hist, ti, kt, vt, self._ring_sink, self._ring_rec,
+                        err_flag=self.err_flag)
         return kt, vt, n
 
     def decode_inputs(self) -> dict:

@@ -75,13 +75,16 @@ def write_tokens(k_hist: torch.Tensor, v_hist: torch.Tensor, pos: torch.Tensor, 
 
 
 def write_token(k_hist: torch.Tensor, v_hist: torch.Tensor, pos: torch.Tensor, k: torch.Tensor,
-                v: torch.Tensor, sink: int, recent: int) -> None:
-    """Single-sequence form, arguments as the reference: ``k_hist [rows, H, D]``, ``pos [1]``."""
+                v: torch.Tensor, sink: int, recent: int, *,
+                err_flag: Optional[torch.Tensor] = None) -> None:
+    """Single-sequence form, arguments as the reference: ``k_hist [rows, H, D]``, ``pos [1]``.
+    A position outside the history sets ``ERR_RING_RANGE`` in ``err_flag`` (the reference
+    asserts there, kv_store_ops.py:33-34); without a flag the row is dropped silently."""
     if k_hist.dim() != 3:
         raise ValueError("k_hist must be [rows, H, D]")
     H, D = int(k_hist.shape[1]), int(k_hist.shape[2])
     write_tokens(k_hist.unsqueeze(0), v_hist.unsqueeze(0), pos, k.reshape(1, H, D),
-                 v.reshape(1, H, D), sink, recent)
+                 v.reshape(1, H, D), sink, recent, err_flag=err_flag)
 
 
 def gather_tails(k_hist: torch.Tensor, v_hist: torch.Tensor, k_tail: torch.Tensor,
@@ -89,7 +92,7 @@ def gather_tails(k_hist: torch.Tensor, v_hist: torch.Tensor, k_tail: torch.Tenso
                  seq: Optional[torch.Tensor] = None, tail_idx: Optional[torch.Tensor] = None,
                  slots: Optional[torch.Tensor] = None, b_tail_len: Optional[torch.Tensor] = None,
                  b_seq_len: Optional[torch.Tensor] = None, window_sink: Optional[int] = None,
-                 window_recent: int = 32, group_tokens: int = 32,
+                 window_recent: int = 32, group_tokens: int = 32, packed_lag: int = 0,
                  err_flag: Optional[torch.Tensor] = None) -> None:
     """Gather the tail rows of ``B`` requests into ``k_tail`` / ``v_tail`` ``[B, T, H, D]``.
 
@@ -97,6 +100,9 @@ def gather_tails(k_hist: torch.Tensor, v_hist: torch.Tensor, k_tail: torch.Tenso
     positions and writes ``b_tail_len`` / ``b_seq_len``) or ``tail_idx`` (int64 ``[B, T]``
     absolute positions).  ``sink`` / ``recent_span`` describe the ring (span 0: whole
     history); ``window_sink`` / ``window_recent`` / ``group_tokens`` the attention window.
+    ``packed_lag``: tokens appended since the planes were last packed (``seq`` form only).  A
+    step that appends and decodes before the host packs passes 1: the boundary is then the one
+    the host has packed for, and the rows since come from the ring.
     """
     _check_hist(k_hist, v_hist)
     if k_hist.dim() != 4:
@@ -129,18 +135,20 @@ def gather_tails(k_hist: torch.Tensor, v_hist: torch.Tensor, k_tail: torch.Tenso
         _hip.ptr(slots), _hip.ptr(seq), _hip.ptr(tail_idx),
         k_tail.data_ptr(), v_tail.data_ptr(), _hip.ptr(b_tail_len), _hip.ptr(b_seq_len),
         B, T, H, D, wsink, int(window_recent), int(group_tokens), int(recent_span),
-        _hip.ptr(err_flag), _hip.current_stream_ptr(dev)), "ommx_tail_gather")
+        int(packed_lag), _hip.ptr(err_flag), _hip.current_stream_ptr(dev)), "ommx_tail_gather")
 
 
 def gather_tail(k_hist: torch.Tensor, v_hist: torch.Tensor, indices: torch.Tensor,
-                k_tail: torch.Tensor, v_tail: torch.Tensor, sink: int, recent: int) -> None:
+                k_tail: torch.Tensor, v_tail: torch.Tensor, sink: int, recent: int, *,
+                err_flag: Optional[torch.Tensor] = None) -> None:
     """Single-sequence form, arguments as the reference: ``k_hist [rows, H, D]``, ``indices [T]``
-    absolute positions, ``k_tail`` / ``v_tail`` ``[1, T, H, D]``."""
+    absolute positions, ``k_tail`` / ``v_tail`` ``[1, T, H, D]``.  A position outside the history
+    yields a zero row and sets ``ERR_RING_RANGE`` in ``err_flag`` (kv_store_ops.py:52-53 asserts)."""
     if k_hist.dim() != 3:
         raise ValueError("k_hist must be [rows, H, D]")
     idx = indices if indices.dtype == torch.int64 else indices.to(torch.int64)
     gather_tails(k_hist.unsqueeze(0), v_hist.unsqueeze(0), k_tail, v_tail, sink, recent,
-                 tail_idx=idx.reshape(1, -1).contiguous())
+                 tail_idx=idx.reshape(1, -1).contiguous(), err_flag=err_flag)
 
 
 __all__ = ["ring_slot", "write_token", "write_tokens", "gather_tail", "gather_tails"]

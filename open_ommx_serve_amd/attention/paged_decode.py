@@ -171,9 +171,32 @@ def ommx_paged_decode_attention_canonical(
             "ommx_paged_decode_attention_canonical requires q_head_num to be an integer "
             f"multiple of n_kv_heads; got q_head_num={Hq} n_kv_heads={Hkv}.")
     for name, t in (("k_base", k_base), ("v_main", v_main), ("v_scale", v_scale), ("v_zp", v_zp)):
-        if t.stride(0) != ps * t.stride(1) or t.stride(-1) != 1:
-            raise ValueError(f"{name} must be a contiguous [pages, page_size, h, w] plane "
-                             "(kv_loc addressing needs stride(0) == page_size*stride(1)).")
+        # the kernels address a row as page*page_size + token and a head as a fixed-width slice of
+        # it: the whole plane must be dense, a view that keeps only some heads or columns is not
+        if t.dim() != 4 or not t.is_contiguous() or int(t.shape[0]) != pages or int(t.shape[1]) != ps \
+                or int(t.shape[2]) != Hkv:
+            raise ValueError(f"{name} must be a contiguous [pages={pages}, page_size={ps}, Hkv={Hkv}, w] "
+                             f"plane; got shape {tuple(t.shape)} strides {tuple(t.stride())}")
+    if q.dim() != 3 or int(q.shape[2]) != D:
+        raise ValueError(f"q must be [B, Hq, D={D}]; got {tuple(q.shape)}")
+    if tuple(k_scale.shape) != (ngroups, Hkv, D) or tuple(k_zp.shape) != (ngroups, Hkv, D) \
+            or k_zp.dtype != torch.bfloat16:
+        raise ValueError(f"k_scale / k_zp must be [group_slots={ngroups}, Hkv={Hkv}, D={D}] (k_zp bf16); "
+                         f"got {tuple(k_scale.shape)} / {tuple(k_zp.shape)} {k_zp.dtype}")
+    if tuple(o.shape) != (B, Hq, D) or tuple(lse.shape) != (B, Hq):
+        raise ValueError(f"o must be [B={B}, Hq={Hq}, D={D}] and lse [B, Hq]; got {tuple(o.shape)} / "
+                         f"{tuple(lse.shape)}")
+    for name, t in (("b_seq_len", b_seq_len), ("b_tail_len", b_tail_len)):
+        if t is not None and (int(t.numel()) < B or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous tensor of at least B={B} entries")
+    for name, t in (("req_to_token", req_to_token), ("req_to_group", req_to_group)):
+        if t.dim() != 2 or int(t.shape[0]) < B:
+            raise ValueError(f"{name} must be [>= B={B}, columns]; got {tuple(t.shape)}")
+    for name, t in (("k_base", k_base), ("k_scale", k_scale), ("v_main", v_main), ("o", o), ("lse", lse),
+                    ("req_to_token", req_to_token), ("req_to_group", req_to_group),
+                    ("b_seq_len", b_seq_len)):
+        if t.device != q.device:
+            raise ValueError(f"{name} is on {t.device}, q on {q.device}")
     off = int(packed_start_offset or 0)
     if off < 0 or off >= ps:
         raise ValueError(f"packed_start_offset={off} must be in [0, page_size={ps})")
@@ -197,6 +220,14 @@ def ommx_paged_decode_attention_canonical(
     use_map = bool(kv_outlier_map) and k > 0
     if use_map and (k_fp4_mapscale is None or k_fp4_mapcenter is None):
         raise ValueError("kv_outlier_map=True requires k_fp4_mapscale + k_fp4_mapcenter planes.")
+    if use_map:
+        for name, t in (("k_fp4_mapscale", k_fp4_mapscale), ("k_fp4_mapcenter", k_fp4_mapcenter)):
+            if t.dtype != torch.bfloat16 or tuple(t.shape) != (ngroups, Hkv, D):
+                raise ValueError(f"{name} must be bf16 [group_slots={ngroups}, Hkv={Hkv}, D={D}]; "
+                                 f"got {t.dtype} {tuple(t.shape)}")
+    if k > 0 and (k_oval.dtype != torch.uint8 or tuple(k_oval.shape) != (ngroups, Hkv, D, (k + 1) // 2)):
+        raise ValueError(f"k_oval must be u8 [group_slots={ngroups}, Hkv={Hkv}, D={D}, {(k + 1) // 2}]; "
+                         f"got {k_oval.dtype} {tuple(k_oval.shape)}")
 
     unsupported = []
     if k > 16:
@@ -254,6 +285,17 @@ def ommx_paged_decode_attention_canonical(
     if o.dtype != torch.float32 or lse.dtype != torch.float32 or o.stride(-1) != 1 or lse.stride(-1) != 1:
         raise ValueError("o / lse must be fp32 with unit inner stride")
 
+    has_tail = gbase == 0 and k_tail is not None and v_tail is not None and b_tail_len is not None \
+        and int(k_tail.shape[1]) > 0 \
+        and (max_tail_len is None or int(max_tail_len) > 0)
+    if has_tail:
+        if k_tail.dtype != torch.bfloat16 or v_tail.dtype != torch.bfloat16 \
+                or k_tail.stride(-1) != 1 or v_tail.stride(-1) != 1 or k_tail.dim() != 4 \
+                or k_tail.shape != v_tail.shape or int(k_tail.shape[0]) < B \
+                or tuple(k_tail.shape[2:]) != (Hkv, D):
+            raise ValueError(f"k_tail / v_tail must be bf16 [>= B={B}, T, Hkv={Hkv}, D={D}] with unit inner "
+                             f"stride; got {tuple(k_tail.shape)} / {tuple(v_tail.shape)}")
+
     _hip.require_gpu(q.device)
     if max_seq_len is not None:
         max_seq = max(1, int(max_seq_len))
@@ -280,14 +322,6 @@ def ommx_paged_decode_attention_canonical(
                 or int(attn_logits.shape[3]) < D + 1 or attn_logits.stride(-1) != 1:
             raise ValueError(f"attn_logits must be fp32 [B={B}, Hq={Hq}, >= {S}, >= {D + 1}] "
                              f"with unit inner stride; got {tuple(attn_logits.shape)}")
-    has_tail = gbase == 0 and k_tail is not None and v_tail is not None and b_tail_len is not None \
-        and int(k_tail.shape[1]) > 0 \
-        and (max_tail_len is None or int(max_tail_len) > 0)
-    if has_tail:
-        if k_tail.dtype != torch.bfloat16 or v_tail.dtype != torch.bfloat16 \
-                or k_tail.stride(-1) != 1 or v_tail.stride(-1) != 1:
-            raise ValueError("k_tail / v_tail must be bf16 [B, T, Hkv, D] with unit inner stride")
-
     if err_flag is not None and (err_flag.dtype != torch.int32 or err_flag.device != q.device):
         raise ValueError("err_flag must be an int32 tensor on the device of q")
     lib = _hip.load()

@@ -201,10 +201,10 @@ extern "C" int ommx_tail_gather(
     const int64_t* slots, const int64_t* seq, const int64_t* tail_idx,
     uint16_t* k_tail, uint16_t* v_tail, int32_t* b_tail_len, int32_t* b_seq_len,
     int B, int T, int H, int D, int sink_rows, int recent_rows, int group_tokens, int ring_span,
-    int32_t* err_flag, void* stream) {
+    int packed_lag, int32_t* err_flag, void* stream) {
     using namespace ommx;
     if (B <= 0 || T <= 0 || H <= 0 || D <= 0 || hist_rows <= 0 || sink_rows < 0 || ring_span < 0 ||
-        recent_rows < 0 || group_tokens <= 0) {
+        recent_rows < 0 || group_tokens <= 0 || packed_lag < 0 || packed_lag > group_tokens) {
         set_error("ommx_tail_gather: bad shape");
         return -1;
     }
@@ -219,8 +219,12 @@ extern "C" int ommx_tail_gather(
     }
     RingArgs a{const_cast<uint16_t*>(k_hist), const_cast<uint16_t*>(v_hist), hist_stride_req,
                hist_rows, sink_rows, ring_span, H, D, slots, err_flag};
+    if (seq && ring_span > 0 && recent_rows + group_tokens - 1 + packed_lag > ring_span) {
+        set_error("ommx_tail_gather: the ring is too short for recent_rows + a group + packed_lag");
+        return -1;
+    }
     launch_tail_gather(a, seq, tail_idx, k_tail, v_tail, B, T, recent_rows, group_tokens,
-                       b_tail_len, b_seq_len, static_cast<hipStream_t>(stream));
+                       packed_lag, b_tail_len, b_seq_len, static_cast<hipStream_t>(stream));
     if (hipGetLastError() != hipSuccess) { set_error("ommx_tail_gather: launch failed"); return -2; }
     return 0;
 }

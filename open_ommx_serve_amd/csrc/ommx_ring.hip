@@ -59,15 +59,19 @@ __global__ void __launch_bounds__(256) ring_write_kernel(
 
 __global__ void __launch_bounds__(256) tail_gather_kernel(
     RingArgs a, const int64_t* seq, const int64_t* tail_idx, uint16_t* k_tail, uint16_t* v_tail,
-    int T, int recent, int gt, int32_t* b_tail_len, int32_t* b_seq_len, int vec) {
+    int T, int recent, int gt, int lag, int32_t* b_tail_len, int32_t* b_seq_len, int vec) {
     const int t = blockIdx.x, b = blockIdx.y;
     int64_t abs_pos;
     if (tail_idx) {
         abs_pos = tail_idx[(int64_t)b * T + t];
     } else {
-        // kv_pool.py:1080-1097: boundary, counts and the sink ++ recent position ramp
+        // kv_pool.py:1080-1097: boundary, counts and the sink ++ recent position ramp.  The
+        // packed boundary is the one of the length the planes were last packed for, `lag`
+        // tokens ago: rows appended since then are read from the ring, the group they may
+        // have completed included.
         const int64_t s = seq[b];
-        const int64_t extra = s - a.sink - recent;
+        const int64_t s_packed = s > lag ? s - lag : 0;
+        const int64_t extra = s_packed - a.sink - recent;
         const int64_t n_sink = s < a.sink ? s : a.sink;
         const int64_t boundary = extra <= 0 ? n_sink : a.sink + (extra / gt) * gt;
         const int64_t n_rec = s > boundary ? s - boundary : 0;
@@ -117,12 +121,12 @@ int launch_ring_write(const RingArgs& a, const uint16_t* k, const uint16_t* v, i
 
 int launch_tail_gather(const RingArgs& a, const int64_t* seq, const int64_t* tail_idx,
                        uint16_t* k_tail, uint16_t* v_tail, int B, int T, int recent, int gt,
-                       int32_t* b_tail_len, int32_t* b_seq_len, hipStream_t st) {
+                       int lag, int32_t* b_tail_len, int32_t* b_seq_len, hipStream_t st) {
     const int vec = (a.H * a.D) % 8 == 0 && aligned16(a.k_hist) && aligned16(a.v_hist) &&
                     aligned16(k_tail) && aligned16(v_tail) && a.req_stride % 8 == 0;
     const int threads = (a.H * a.D / (vec ? 8 : 1)) >= 256 ? 256 : 128;
     hipLaunchKernelGGL(tail_gather_kernel, dim3(T, B), dim3(threads), 0, st, a, seq, tail_idx,
-                       k_tail, v_tail, T, recent, gt, b_tail_len, b_seq_len, vec);
+                       k_tail, v_tail, T, recent, gt, lag, b_tail_len, b_seq_len, vec);
     return 0;
 }
 

@@ -20,6 +20,6 @@ int launch_ring_write(const RingArgs& a, const uint16_t* k, const uint16_t* v, i
                       int64_t* pos_next, int B, hipStream_t st);
 int launch_tail_gather(const RingArgs& a, const int64_t* seq, const int64_t* tail_idx,
                        uint16_t* k_tail, uint16_t* v_tail, int B, int T, int recent, int gt,
-                       int32_t* b_tail_len, int32_t* b_seq_len, hipStream_t st);
+                       int lag, int32_t* b_tail_len, int32_t* b_seq_len, hipStream_t st);
 
 }  // namespace ommx

@@ -162,6 +162,9 @@ class OMMXCanonicalMetadataBuilder(_BuilderBase):
                                    f"{s.manager.dead_reason}")
         if in_batched and s.bmanager is not None:
             s.bmanager.on_build(common)
+            if s.bmanager.dead:
+                raise RuntimeError("OMMX refuses to serve this step from the batched pool: "
+                                   f"{s.bmanager.dead_reason}")
 
     def build_for_cudagraph_capture(self, common_attn_metadata):
         s = _STATE
@@ -258,6 +261,8 @@ class OMMXCanonicalImpl(_ImplBase):
                 "Refusing to write rather than risk resetting a live sequence.")
         if st["batched_write"]:
             m = s.bmanager
+            if m is not None and m.dead:
+                raise RuntimeError(f"[ommx] batched pool dead: {m.dead_reason}")
             if (m is not None and m.graph and m.is_uniform_decode and n == int(m.cur_B) > 0):
                 self._batched_kv_update_captured(layer, key, value)
             else:

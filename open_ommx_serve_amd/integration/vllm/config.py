@@ -133,6 +133,12 @@ def resolve_serving_config(*, head_dim: Optional[int] = None, n_q_heads: Optiona
                       ("page_size", page_size), ("max_context", max_context)):
         if val is not None:
             setattr(cfg, name, int(val))
+    if cfg.recent_window < 1 or cfg.sink_tokens < 0:
+        # the step seam packs completed groups before the forward writes token seq-1; that token
+        # stays outside the packed region only while at least one recent row is kept as bf16
+        raise ValueError(f"OMMX_KV_RECENT must be >= 1 and OMMX_KV_SINK >= 0; got recent="
+                         f"{cfg.recent_window}, sink={cfg.sink_tokens}: with no recent row the "
+                         "seam would pack a group whose last token is not written yet")
     if cfg.k_format not in ("i2f4", "itf4"):
         raise ValueError(f"OMMX_ATTN_K_FORMAT must be i2f4|itf4; got {cfg.k_format!r}")
     if cfg.outlier_repr not in OUTLIER_REPRS:

@@ -33,7 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     for n in names:
         assert getattr(raw, n) is not None, n
     assert set(_hip.exported_symbols()) == set(names)
-    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 6
+    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 7
 
 
 def test_default_decision_table_is_the_exact_arithmetic_one():
@@ -185,6 +185,36 @@ def test_decode_argument_errors_precede_any_launch():
     with pytest.raises(ValueError, match="contiguous"):
         bad = list(args); bad[6] = args[6][:, ::2]
         D(*bad, **{**kw, "page_size": 8})
+    # operands whose shape or layout the kernels would otherwise take on trust
+    with pytest.raises(ValueError, match="k_base must be a contiguous"):
+        bad = list(args); bad[1] = args[1][:, :, :1]                  # a view that keeps one kv head
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="v_zp must be a contiguous"):
+        bad = list(args); bad[8] = args[8].transpose(2, 3).contiguous().transpose(2, 3)
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="o must be"):
+        bad = list(args); bad[12] = torch.zeros(1, 4, 32)
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="lse"):
+        bad = list(args); bad[13] = torch.zeros(1, 3)
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="b_seq_len"):
+        bad = list(args); bad[16] = torch.zeros(0, dtype=torch.int32)
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="req_to_group"):
+        bad = list(args); bad[15] = args[15].reshape(-1)
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="k_oval must be"):
+        bad = list(args); bad[5] = args[5][..., :2]
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="k_fp4_mapcenter must be"):
+        D(*args, **{**kw, "k_fp4_mapcenter": kw["k_fp4_mapcenter"][:1]})
+    with pytest.raises(ValueError, match="k_scale / k_zp"):
+        bad = list(args); bad[3] = args[3][:, :1]
+        D(*bad, **kw)
+    with pytest.raises(ValueError, match="k_tail / v_tail"):
+        bad = list(args); bad[9] = bad[10] = torch.zeros(1, 8, 1, 64, dtype=torch.bfloat16)
+        D(*bad, **kw)
     with pytest.raises(ValueError, match="k_crank must be"):          # the rank plane's own shape check
         D(*args, **{**kw, "combinadic_read": True, "bitmap_read": False,
                     "k_crank": torch.zeros(2, 2, 64, 4, dtype=torch.uint8)})

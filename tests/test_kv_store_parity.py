@@ -148,14 +148,18 @@ def _decode_bundle(q, bundle, sm_scale, k):
     return o.cpu(), lse.cpu()
 
 
-def _oracle_decode(q, K_hist, V_hist, win, sm_scale):
-    """Dequantise-then-attend over the full history of every request (fp64)."""
+def _oracle_decode(q, K_hist, V_hist, win, sm_scale, packed_for=None):
+    """Dequantise-then-attend over the full history of every request (fp64).  ``packed_for``:
+    the lengths the planes were last packed for (default: the current ones); rows past that
+    boundary are attended as bf16."""
     outs, lses = [], []
     for b, (K, V) in enumerate(zip(K_hist, V_hist)):
         n = int(K.shape[0])
-        edge = win.boundary(n)
-        Kf = [K[i].float() for i in win.tail_indices(n)]
-        Vf = [V[i].float() for i in win.tail_indices(n)]
+        edge = win.boundary(n if packed_for is None else packed_for[b])
+        rows = list(range(min(n, win.sink_tokens))) + list(range(max(edge, min(n, win.sink_tokens)), n))
+        assert packed_for is not None or rows == win.tail_indices(n)
+        Kf = [K[i].float() for i in rows]
+        Vf = [V[i].float() for i in rows]
         Kd = torch.stack(Kf) if Kf else torch.zeros(0, *K.shape[1:])
         Vd = torch.stack(Vf) if Vf else torch.zeros(0, *V.shape[1:])
         if edge > win.sink_tokens:
@@ -451,6 +455,32 @@ def test_store_prefill_write_token_advance_and_decode(ring):
     assert st.seq_len == 0 and st.packed_groups == 0
 
 
+def test_store_reports_a_position_outside_its_history():
+    """The launch-only write and gather of the single-sequence store carry the store's error
+    flag: a position beyond the history is dropped / zero-filled on the device and
+    ``check_errors`` raises what the reference's assert would have."""
+    H, D = 2, 64
+    st = CanonicalKVStore(D, H, max_seq_len=128, device=DEV, kv_ring=False, **RECIPE)
+    K, V = synth_kv(4, H, D, seed=5)
+    rows = int(st.k_hist.shape[0])
+    st.write_token(torch.tensor([3], device=DEV), K[0].to(DEV), V[0].to(DEV))
+    st.check_errors()
+    before = st.k_hist.clone()
+    st.write_token(torch.tensor([rows + 7], device=DEV), K[1].to(DEV), V[1].to(DEV))
+    with pytest.raises(IndexError):
+        st.check_errors()
+    assert torch.equal(st.k_hist, before)
+    st.check_errors()                                   # the flag was cleared by the raise
+    T = 8
+    kt = torch.ones(1, T, H, D, dtype=torch.bfloat16, device=DEV)
+    vt = torch.ones_like(kt)
+    idx = torch.tensor([3, 0, 0, rows + 1, 0, 0, 0, 0], dtype=torch.int64, device=DEV)
+    st.gather_tail_into(idx, kt, vt, 4)
+    with pytest.raises(IndexError):
+        st.check_errors()
+    assert torch.equal(kt[0, 0].cpu(), K[0]) and not kt[0, 3].any()
+
+
 def test_eager_append_matches_write_token():
     H, D = 2, 64
     K, V = synth_kv(120, H, D, seed=3)
@@ -559,7 +589,8 @@ def test_decode_step_replayed_from_a_hip_graph():
                      g_pool._ring_rec, slots=d["rows"], pos_next=d["seq_dev"], err_flag=g_pool.err_flag)
         gather_tails(g_pool.k_hist, g_pool.v_hist, d["kt"], d["vt"], g_pool._ring_sink, g_pool._ring_rec,
                      seq=d["seq_dev"], slots=d["sel"], b_tail_len=d["b_tail"], b_seq_len=d["b_seq"],
-                     window_sink=win.sink_tokens, window_recent=win.recent_window, group_tokens=win.group_tokens)
+                     window_sink=win.sink_tokens, window_recent=win.recent_window, group_tokens=win.group_tokens,
+                     packed_lag=1, err_flag=g_pool.err_flag)
         ommx_paged_decode_attention_canonical(
             q, pl["k_base"], pl["k_scale"], pl["k_zp"], None, pl["k_oval"], pl["v_main"], pl["v_scale"],
             pl["v_zp"], d["kt"], d["vt"], d["b_tail"], o, lse, pl["req_to_token"], pl["req_to_group"],
@@ -568,9 +599,9 @@ def test_decode_step_replayed_from_a_hip_graph():
             k_fp4_mapcenter=pl["k_fp4_mapcenter"], kv_outlier_map=True, kv_int8_scale=True,
             max_seq_len=600, max_tail_len=g_pool.max_tail_len, num_kv_splits=S, attn_logits=ws)
 
-    # A token becomes visible to the decode of the step that appends it only after the host
-    # has packed the group it may complete, so the captured step decodes BEFORE the pack of
-    # its own append; the eager pool mirrors exactly that order.
+    # The host packs between replays, so the captured step decodes BEFORE the pack of its own
+    # append: its tail gather is told that the planes lag the sequence by one token
+    # (packed_lag=1) and reads the group that token may have completed from the ring.
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     graph = torch.cuda.CUDAGraph()
@@ -584,6 +615,7 @@ def test_decode_step_replayed_from_a_hip_graph():
             step()
         d["seq_dev"].copy_(seq_before)          # capture does not run the kernels
     torch.cuda.current_stream().wait_stream(stream)
+    completed_steps = 0
     for s in range(steps):
         newK.copy_(torch.stack([Ks[i][prefill[i] + s] for i in range(B)]))
         newV.copy_(torch.stack([Vs[i][prefill[i] + s] for i in range(B)]))
@@ -598,17 +630,19 @@ def test_decode_step_replayed_from_a_hip_graph():
         assert d["seq_dev"].tolist() == cur
         # what the captured step attended: packed prefix as of the last host pack + tail as of now
         want_o, want_l = [], []
+        completing = 0
         for i in range(B):
             n, packed_groups = cur[i], g_pool.packed_groups[i]
-            edge = win.sink_tokens + packed_groups * win.group_tokens
-            assert int(d["b_seq"][i]) == win.packed_len(n)
-            if win.packed_len(n) != packed_groups * win.group_tokens:
-                continue                           # the group completed by this very token: see above
-            wo, wl = _oracle_decode(q[i:i + 1], [Ks[i][:n]], [Vs[i][:n]], win, sm_scale)
+            assert int(d["b_seq"][i]) == win.packed_len(n - 1) == packed_groups * win.group_tokens
+            assert int(d["b_tail"][i]) == n - win.packed_len(n - 1)
+            completing += win.packed_len(n) != win.packed_len(n - 1)
+            wo, wl = _oracle_decode(q[i:i + 1], [Ks[i][:n]], [Vs[i][:n]], win, sm_scale, packed_for=[n - 1])
             _check_out((o[i:i + 1].cpu(), lse[i:i + 1].cpu()), (wo, wl), f"replay {s} req {i}")
+        completed_steps += completing
         # host seam between replays: advance the mirrors and pack what completed
         packed = g_pool._advance_host_and_pack(range(B))
         assert packed == e_pool._advance_host_and_pack(range(B))
+    assert completed_steps >= B                 # steps whose token completed a group were checked too
     for name in PLANE_NAMES:
         assert torch.equal(getattr(g_pool, name), getattr(e_pool, name)), name
     assert torch.equal(g_pool.k_hist, e_pool.k_hist) and torch.equal(g_pool.v_hist, e_pool.v_hist)

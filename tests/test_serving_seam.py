@@ -114,6 +114,20 @@ def test_the_current_token_is_never_inside_the_packed_region(sink, recent, gt):
             assert b <= seq - recent
 
 
+def test_a_window_without_recent_rows_is_refused_at_the_seam(monkeypatch):
+    """recent = 0 would let the boundary reach seq itself: the seam packs before the forward
+    writes token seq-1, so that group would be packed with an unwritten row."""
+    assert any(packed_boundary(seq, 8, 0, 32) == seq for seq in range(1, 200))
+    with pytest.raises(ValueError, match="recent"):
+        OMMXStepManager(_cfg(recent_window=0), "cpu")
+    with pytest.raises(ValueError, match="recent"):
+        OMMXBatchedStepManager(_cfg(recent_window=0), "cpu", 2)
+    monkeypatch.setenv("OMMX_KV_RECENT", "0")
+    from open_ommx_serve_amd.integration.vllm.config import resolve_serving_config
+    with pytest.raises(ValueError, match="OMMX_KV_RECENT"):
+        resolve_serving_config(head_dim=64, n_q_heads=4, n_kv_heads=2)
+
+
 # ── single-request manager ───────────────────────────────────────────────────────────────
 
 class _Store:
