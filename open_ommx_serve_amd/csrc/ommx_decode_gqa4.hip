@@ -180,21 +180,6 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         return;
     }
 
-    // ---- LDS that starts out constant: zero tile, zero corrections, the zero and one rows ----
-    {
-        u32x4* p = reinterpret_cast<u32x4*>(sm + OFF_TILE);
-        for (int i = lane; i < 32 * TILE_ROW / 16; i += 64) p[i] = u32x4{0, 0, 0, 0};
-        if (lane < 32) reinterpret_cast<u32x4*>(sm + OFF_LC)[lane] = u32x4{0, 0, 0, 0};
-        if (lane < 16) reinterpret_cast<u32x4*>(sm + OFF_ZERO)[lane] =
-            lane < 8 ? u32x4{0, 0, 0, 0} : u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
-    }
-
-    f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
-    f32x4 accz = {0, 0, 0, 0};
-    float m_run[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
-
     // ---- addressing ---------------------------------------------------------------------------
     const uint32_t row_bytes = (uint32_t)Hkv * 32u;
     const int last = n_end - 1;
@@ -267,12 +252,26 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
         g_ov[g] = u32x2{ovp[0], ovp[1]};
     };
+    // The page and group ids of the first step are asked for here; what follows (clearing LDS, the
+    // A operands, the lane constants) needs none of it and runs while they are on their way.
     fetch_tables(n_begin);
-    fetch_k();
-    fetch_v();
-    fetch_params_g(0);
-    fetch_params_g(1);
-    fetch_tables(n_begin + 64);
+    asm volatile("" ::: "memory");
+
+    // ---- LDS that starts out constant: zero tile, zero corrections, the zero and one rows ----
+    {
+        u32x4* p = reinterpret_cast<u32x4*>(sm + OFF_TILE);
+        for (int i = lane; i < 32 * TILE_ROW / 16; i += 64) p[i] = u32x4{0, 0, 0, 0};
+        if (lane < 32) reinterpret_cast<u32x4*>(sm + OFF_LC)[lane] = u32x4{0, 0, 0, 0};
+        if (lane < 16) reinterpret_cast<u32x4*>(sm + OFF_ZERO)[lane] =
+            lane < 8 ? u32x4{0, 0, 0, 0} : u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+    }
+
+    f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    f32x4 accz = {0, 0, 0, 0};
+    float m_run[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
+
 
     // ---- A operand of QK: q * 2^(10-2m) of head j % 4 for this lane's 32-channel quarter, f16, in
     // pair order: k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2).  The base codes,
@@ -326,6 +325,13 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     const uint32_t code_sh = 2u * (c0 & 3u);                      // bit of channel c0's code in that byte; c0 + 1 sits two on
     const uint32_t nib_sh = 8u * ((6u * lane) & 3u);
     const float c2 = a.sm_scale * 1.4426950408889634f;
+
+    // in the order the first step needs them: K rows, the group parameters, then V
+    fetch_k();
+    fetch_params_g(0);
+    fetch_params_g(1);
+    fetch_v();
+    fetch_tables(n_begin + 64);
 
     for (int n0 = n_begin; n0 < n_end; n0 += 64) {
         const bool more = n0 + 64 < n_end;
@@ -557,7 +563,7 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
                 asm volatile("" : "+v"(mine));
                 const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
                     0, __builtin_bit_cast(int, mine), 0x4E, 0xF, 0xF, true));     // quad_perm [2,3,0,1]
-                x[r] = dsel[r] + __shfl(mine - other, gsel);
+                x[r] = dsel[r] + lane_value(mine - other, gsel);
             }
         }
         float pe[4];          // base-2 logit minus the running maximum
@@ -656,13 +662,18 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
 
     // ---- epilogue: o = (f*(acc - sum p*2^e) + sum p*zp) / l, f = 16 or 4; lse = m + ln l ----------
     // sums live in the lanes of the same column j: rows 0-3 (kq 0) zero points, 4-7 (kq 1) steps, 8 (kq 2) ones
-    const int h = j & 3, x = j >> 2;
-    const float l_tot = __shfl(accz[0], 32 + j);
+    // (lane-derived values are formed afresh here: carried over from the top of the kernel they
+    // would sit in registers the loop needs, or in scratch memory)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int je = lane_e & 15, kqe = lane_e >> 4;
+    const int h = je & 3, x = je >> 2;
+    const float l_tot = lane_value(accz[0], 32 + je);
     float z4[4], s4[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        z4[r] = __shfl(accz[r], j);
-        s4[r] = __shfl(accz[r], 16 + j);
+        z4[r] = lane_value(accz[r], je);
+        s4[r] = lane_value(accz[r], 16 + je);
     }
     const float inv = l_tot > 0.0f ? __builtin_amdgcn_rcpf(l_tot) : 0.0f;
     if (h < heads) {
@@ -672,16 +683,16 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 // row i = 4kq + r of block Y = 4*a2 + x: channel 16*(i & 7) + 8*(i >> 3) + Y, group (i & 7) / 2
-                const int cg_lo = 2 * (kq & 1);
-                const float pz = (r >> 1) ? ((kq & 1) ? z4[3] : z4[1]) : ((kq & 1) ? z4[2] : z4[0]);
-                const float psum = (r >> 1) ? ((kq & 1) ? s4[3] : s4[1]) : ((kq & 1) ? s4[2] : s4[0]);
+                const int cg_lo = 2 * (kqe & 1);
+                const float pz = (r >> 1) ? ((kqe & 1) ? z4[3] : z4[1]) : ((kqe & 1) ? z4[2] : z4[0]);
+                const float psum = (r >> 1) ? ((kqe & 1) ? s4[3] : s4[1]) : ((kqe & 1) ? s4[2] : s4[0]);
                 (void)cg_lo;
-                const int ch = 64 * (kq & 1) + 16 * r + 8 * (kq >> 1) + 4 * a2 + x;
+                const int ch = 64 * (kqe & 1) + 16 * r + 8 * (kqe >> 1) + 4 * a2 + x;
                 const float f = (x & 1) ? 4.0f : 16.0f;
                 dst[ch] = (f * (acc[a2][r] - psum) + pz) * inv;
             }
         }
-        if (x == 0 && kq == 0) {
+        if (x == 0 && kqe == 0) {
             const float mt = h == 0 ? m_run[0] : (h == 1 ? m_run[1] : (h == 2 ? m_run[2] : m_run[3]));
             dst[D] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
         }

@@ -39,6 +39,11 @@ __device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
 __device__ __forceinline__ float readlane_f32(float v, int l) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
 }
+// Value of `v` in lane `src_lane` (0..63), through the LDS crossbar; the lane number is the
+// caller's, so nothing about the reading lane has to be kept in a register for it.
+__device__ __forceinline__ float lane_value(float v, int src_lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
+}
 // Maxima of four values over the 64 lanes (results uniform).  The four reductions are
 // interleaved so that every DPP instruction is at least three instructions away from the
 // write of its source, which covers the two wait states the DPP read needs; steps: two
