@@ -6,8 +6,9 @@
 //
 // A wavefront owns one kv head (and its q heads) of one split and walks it 64 tokens at a time;
 // a workgroup is 4 waves = 4 neighbouring kv heads.  Measured on MI355X this operator is bound
-// by how many instructions one wave can issue (vector ALU first, LDS second), so the kernel is
-// built to keep THREE waves per SIMD resident: at most 168 vector registers and 13.5 KB of LDS
+// by how many instructions a SIMD can issue (vector ALU first, LDS second, a 16-byte LDS access
+// taking four issue slots), so the kernel is built for few instructions per token and to keep
+// THREE waves per SIMD resident: at most 168 vector registers, no scratch memory, 13.4 KB of LDS
 // per wave.  What that takes, against the kernel in ommx_decode.hip:
 //   * P.V runs transposed (rows = V channels, columns = q heads), the V step 2^e sits in the
 //     exponent field of the V operand, and the four column replicas of the q heads each take
@@ -16,14 +17,18 @@
 //     p*zp (a row of ones), the running maximum is refreshed only when a logit exceeds it by
 //     more than 2^8 (any bound that keeps exp2 in range serves an online softmax);
 //   * the V staging area of LDS is the K staging area of the same step, reused once QK is done.
-// Arithmetic is that of ommx_decode.hip: exact 16-bit operands, fp32 accumulation.
-//   K base   B = (1 + code*2^(2k-7)) * 2^e as bf16 (code dropped into mantissa bits [2k+1:2k],
-//            k = 1 or 2 per channel pair), A = q * 2^(7-2k); the constant terms sum q*zp and
-//            sum A*2^e come from one small "bias" MFMA per 64 tokens.
-//   outliers a channel-major pass (one lane = two channels) overwrites the base code of every
-//            outlier position in the staged K rows by 0 or 3, whichever is nearer (ds_mskor_b32),
-//            and scatters (outlier - zp - code*2^e) as f16 into a [32 tokens][128 channels]
-//            tile that is the B operand of an f16 MFMA against A = q.  Deltas whose f16 rounding
+// Arithmetic: exact 16-bit operands, fp32 accumulation, as in ommx_decode.hip.
+//   A (QK)   q * 2^(10-2m) as f16 in pair order, m = 1..4 fixed per channel pair; this one operand
+//            set serves the base codes, the outlier tile and the bias columns.
+//   K base   B = (1 + code*2^(2m-10)) * 2^e as f16: the 2-bit code is dropped into mantissa bits
+//            [2m+1:2m] of a per-(group, channel) pattern that carries the exponent, one and-or per
+//            channel pair.  The constant terms sum q*zp and sum A*2^e come from one small "bias"
+//            MFMA per 64 tokens (zero points are staged divided by the channel's 2^(10-2m), exact).
+//   outliers a channel-major pass (one lane = two channels) reads the stored 2-bit code of every
+//            outlier position back from the staged K rows (the base MFMA takes every position as
+//            stored; nothing is cleared there) and scatters
+//            (outlier - zp - code*2^e) / 2^(10-2m) as f16 into a [32 tokens][128 channels] tile
+//            that is the B operand of an f16 MFMA against the same A.  Entries whose f16 rounding
 //            could show on a logit add their rounding residual times q through LDS float atomics.
 //   P.V      A = (1 + code/4 | 1 + code/16) * 2^e_v as f16 for 8 tokens of one channel, B = p (f16).
 #include <type_traits>
