@@ -55,15 +55,25 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const int d = tid;
         float w[32];
         bool fin = true;
+        if (a.src_rows) {
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const int64_t row = a.src_rows ? a.src_rows[g * 32 + i] : (int64_t)g * 32 + i;
-            w[i] = load_elem<F32>(a.K, row * a.k_ts + (int64_t)h * a.k_hs + d);
-            if (!FAST6) fin = fin && is_finite_f32(w[i]);
+            for (int i = 0; i < 32; ++i) {
+                const int64_t row = a.src_rows[g * 32 + i];
+                w[i] = load_elem<F32>(a.K, row * a.k_ts + (int64_t)h * a.k_hs + d);
+            }
+        } else {            // consecutive rows: one base, 32 strides
+            const int64_t base = (int64_t)g * 32 * a.k_ts + (int64_t)h * a.k_hs + d;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) w[i] = load_elem<F32>(a.K, base + i * a.k_ts);
+        }
+        if (!FAST6) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) fin = fin && is_finite_f32(w[i]);
         }
 
         uint32_t top = 0, bot = 0;
         int key_hi[3] = {0, 0, 0}, key_lo[3] = {0, 0, 0};    // FAST6: sorted keys of the chosen lanes
+        int t4 = INT_MIN, b4 = INT_MAX;                      // FAST6: keys of the fourth largest / smallest lane
         auto select_generic = [&]() {
             if (select_abs) {
                 // the kout largest magnitudes, ties to the lower index (stable descending sort
@@ -104,31 +114,53 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                 if (bi >= 0) bot |= 1u << bi;
             }
         };
-        bool fast_done = false;
+        bool fast_done = false, ranks_clean = false;
         if (FAST6) {
             // bf16 inputs leave 16 free bits under the value: key = ordered value bits | tie
             // breaker.  Largest three: tie breaker 31-i with max (equal values: lower index
             // first, the stable descending sort).  Smallest three: tie breaker i with min.
             // One pass each through a three-deep max / median network.
+            // (a fourth rank on either side: the largest and the smallest of the lanes that stay)
             int t1 = INT_MIN, t2 = INT_MIN, t3 = INT_MIN;
             int b1 = INT_MAX, b2 = INT_MAX, b3 = INT_MAX;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
                 const int kt_i = ordered_bits(w[i] + 0.0f) | (31 - i);
                 const int kb_i = kt_i ^ 31;
-                const int n3 = med3_i32(t2, t3, kt_i), n2 = med3_i32(t1, t2, kt_i);
-                t1 = max(t1, kt_i); t2 = n2; t3 = n3;
-                const int m3 = med3_i32(b2, b3, kb_i), m2 = med3_i32(b1, b2, kb_i);
-                b1 = min(b1, kb_i); b2 = m2; b3 = m3;
+                const int n4 = med3_i32(t3, t4, kt_i), n3 = med3_i32(t2, t3, kt_i), n2 = med3_i32(t1, t2, kt_i);
+                t1 = max(t1, kt_i); t2 = n2; t3 = n3; t4 = n4;
+                const int m4 = med3_i32(b3, b4, kb_i), m3 = med3_i32(b2, b3, kb_i), m2 = med3_i32(b1, b2, kb_i);
+                b1 = min(b1, kb_i); b2 = m2; b3 = m3; b4 = m4;
             }
+            // (the fourth ranks are pinned here: left to the compiler, their two chains of 32 steps
+            // move down into the one branch that reads them, and all 64 keys stay live until then)
+            asm volatile("" : "+v"(t4), "+v"(b4));
             top = (1u << (31 - (t1 & 31))) | (1u << (31 - (t2 & 31))) | (1u << (31 - (t3 & 31)));
             bot = (1u << (b1 & 31)) | (1u << (b2 & 31)) | (1u << (b3 & 31));
             key_hi[0] = t1; key_hi[1] = t2; key_hi[2] = t3;
             key_lo[0] = b1; key_lo[1] = b2; key_lo[2] = b3;
             // The reference takes the smallest three of the vector with the top lanes moved
             // to +1e9.  That is the same set unless a top lane is among the overall smallest
-            // three (heavy ties): then redo the selection the slow way.
-            fast_done = (top & bot) == 0u;
+            // three (heavy ties): then the bottom ranks are taken again with those lanes at +1e9.
+            // (A pass with three running values, not the general selection below: that one
+            // keeps two 32-element arrays in registers and would set this kernel's register
+            // count.)
+            ranks_clean = (top & bot) == 0u;
+            if (!ranks_clean) {
+                b1 = INT_MAX; b2 = INT_MAX; b3 = INT_MAX;
+#pragma unroll
+                for (int i = 0; i < 32; ++i) {
+                    float wi = w[i];
+                    asm volatile("" : "+v"(wi));      // formed again here: 32 keys kept from the first pass would cost 32 registers
+                    // (the reference's own sentinel, so that a vector it refuses is refused here too)
+                    const int kb_i = ordered_bits(((top >> i) & 1u) ? 1e9f : wi + 0.0f) | i;
+                    const int m3 = med3_i32(b2, b3, kb_i), m2 = med3_i32(b1, b2, kb_i);
+                    b1 = min(b1, kb_i); b2 = m2; b3 = m3;
+                }
+                bot = (1u << (b1 & 31)) | (1u << (b2 & 31)) | (1u << (b3 & 31));
+                key_lo[0] = b1; key_lo[1] = b2; key_lo[2] = b3;
+            }
+            fast_done = true;
         }
         if (!fast_done) select_generic();
         const uint32_t om = top | bot;
@@ -145,13 +177,29 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
 
         // affine base over the non-outlier lanes (pack.py:455-465)
         float mn = 1e9f, mx = -1e9f, omn = 1e9f, omx = -1e9f;
+        // With three lanes taken from either end, what stays starts at the fourth rank, and the
+        // outliers span the first ranks: no pass over the vector.  (With equal values around
+        // the fourth rank its VALUE is still the extreme of the lanes that stay.)  A zero
+        // minimum, or zero at both outlier ends, goes the long way: which sign a zero result
+        // takes depends on the lanes, not on the ranks.
+        bool ranks_do = false;
+        if (FAST6 && ranks_clean) {
+            mn = from_ordered_bits(b4);
+            mx = from_ordered_bits(t4);
+            omn = from_ordered_bits(key_lo[0]);
+            omx = from_ordered_bits(key_hi[0]);
+            ranks_do = mn != 0.0f && (omn != 0.0f || omx != 0.0f);
+        }
+        if (!ranks_do) {
+            mn = 1e9f; mx = -1e9f; omn = 1e9f; omx = -1e9f;
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const bool o = (om >> i) & 1u;
-            mn = fminf(mn, o ? 1e9f : w[i]);
-            mx = fmaxf(mx, o ? -1e9f : w[i]);
-            omn = fminf(omn, o ? w[i] : 1e9f);
-            omx = fmaxf(omx, o ? w[i] : -1e9f);
+            for (int i = 0; i < 32; ++i) {
+                const bool o = (om >> i) & 1u;
+                mn = fminf(mn, o ? 1e9f : w[i]);
+                mx = fmaxf(mx, o ? -1e9f : w[i]);
+                omn = fminf(omn, o ? w[i] : 1e9f);
+                omx = fmaxf(omx, o ? w[i] : -1e9f);
+            }
         }
         if (mn > 1e8f) mn = 0.0f;
         if (mx < -1e8f) mx = 0.0f;
@@ -187,9 +235,14 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         uint32_t nib = 0;
         bool mfin = true;
         if (FAST6 && fast_done) {
+            if (inv_ok) {                 // one branch per vector, not one per element
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, inv_ok));
+                for (int i = 0; i < 32; ++i)
+                    s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, true));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, false));
             }
             // |(w - mc) * ms| is largest at the extreme lanes, which are outliers: they decide
             // whether every mapped value is finite (codec.py:55-57 checks all of them)
@@ -306,12 +359,15 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         }
         bool fin = true;
         float mn = 0.0f, mx = 0.0f;
+        // finite <=> exponent field not all ones: the largest exponent field of the vector decides
+        uint32_t emax = 0;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
-            fin = fin && is_finite_f32(v[c]);
+            emax = max(emax, __float_as_uint(v[c]) & 0x7F800000u);
             mn = c == 0 ? v[c] : fminf(mn, v[c]);
             mx = c == 0 ? v[c] : fmaxf(mx, v[c]);
         }
+        fin = emax != 0x7F800000u;
         if (!fin) err |= OMMX_ERR_NONFINITE_V;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
         const Step st = make_step(raw, scale_mode, tab);
@@ -322,9 +378,14 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const bool inv_ok = st.inv_ok;
         const float inv_scale = st.inv;
         uint64_t vb8 = 0;
+        if (inv_ok) {
 #pragma unroll
-        for (int c = 0; c < 32; ++c) {
-            vb8 |= static_cast<uint64_t>(int2_code(v[c] - zp, scale, inv_scale, inv_ok)) << (2 * c);
+            for (int c = 0; c < 32; ++c)
+                vb8 |= static_cast<uint64_t>(int2_code(v[c] - zp, scale, inv_scale, true)) << (2 * c);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 32; ++c)
+                vb8 |= static_cast<uint64_t>(int2_code(v[c] - zp, scale, inv_scale, false)) << (2 * c);
         }
         const int64_t vidx = (prow * a.H + h) * NGV + j;
         reinterpret_cast<uint64_t*>(a.v_main)[vidx] = vb8;
