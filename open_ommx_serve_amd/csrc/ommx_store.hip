@@ -21,6 +21,11 @@ __device__ __forceinline__ int ordered_bits(float x) {
     const int b = __float_as_int(x);
     return (b ^ ((b >> 31) & 0x7FFFFFFF)) & static_cast<int>(0xFFFF0000u);
 }
+// The same for a value whose low 16 bits are zero (a bf16 widened to fp32): nothing to clear.
+__device__ __forceinline__ int ordered_bits_bf16(float x) {
+    const int b = __float_as_int(x);
+    return b ^ ((b >> 31) & 0x7FFF0000);
+}
 __device__ __forceinline__ float from_ordered_bits(int k) {
     const int s = k & static_cast<int>(0xFFFF0000u);
     // negative images had their low 16 bits set before the clearing; restore them
@@ -33,8 +38,11 @@ __device__ __forceinline__ int med3_i32(int a, int b, int c) {
 // IDXT: index plane known at compile time (0 bitmap, 1 relidx7) or read from the arguments (2)
 template <bool F32, bool FAST6, int IDXT>
 __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
+    static_assert(!(F32 && FAST6), "the tuned path reads bf16 input");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int D = a.D;
+    // head_dim 128 is compiled in for the tuned instantiations (their launch checks it): row offsets
+    // of the code tile become instruction immediates
+    const int D = FAST6 ? 128 : a.D;
     uint8_t* s_codes = smem;                       // [32][D] one code per byte
     uint8_t* s_oval = smem + 32 * D;               // [D][nval] nibble bytes, packed as in memory
     uint8_t* s_oidx = smem + 36 * D;               // [D][nidx] position stream bytes (relidx7 only)
@@ -125,7 +133,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             int b1 = INT_MAX, b2 = INT_MAX, b3 = INT_MAX;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                const int kt_i = ordered_bits(w[i] + 0.0f) | (31 - i);
+                const int kt_i = ordered_bits_bf16(w[i] + 0.0f) | (31 - i);      // FAST6 is a bf16-input instantiation
                 const int kb_i = kt_i ^ 31;
                 const int n4 = med3_i32(t3, t4, kt_i), n3 = med3_i32(t2, t3, kt_i), n2 = med3_i32(t1, t2, kt_i);
                 t1 = max(t1, kt_i); t2 = n2; t3 = n3; t4 = n4;
@@ -341,7 +349,11 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const int64_t row = a.src_rows ? a.src_rows[tok] : tok;
         const int64_t vbase = row * a.v_ts + (int64_t)h * a.v_hs + 32 * j;
         float v[32];
+        bool fin = true;
+        // finite <=> exponent field not all ones: the largest exponent field of the vector decides
         if (!F32 && a.v_vec) {                    // 64 contiguous bytes: four 16-byte loads
+            typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+            u16x2 e2 = {0, 0};                    // largest exponent field of the even / of the odd channels
             const uint4* vp = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.V) + vbase);
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
@@ -351,23 +363,25 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                 for (int k = 0; k < 4; ++k) {
                     v[8 * q4 + 2 * k] = __uint_as_float(uw[k] << 16);
                     v[8 * q4 + 2 * k + 1] = __uint_as_float(uw[k] & 0xFFFF0000u);
+                    e2 = __builtin_elementwise_max(e2, __builtin_bit_cast(u16x2, uw[k] & 0x7F807F80u));
                 }
             }
+            fin = e2[0] != 0x7F80 && e2[1] != 0x7F80;
         } else {
+            uint32_t emax = 0;
 #pragma unroll
-            for (int c = 0; c < 32; ++c) v[c] = load_elem<F32>(a.V, vbase + c);
+            for (int c = 0; c < 32; ++c) {
+                v[c] = load_elem<F32>(a.V, vbase + c);
+                emax = max(emax, __float_as_uint(v[c]) & 0x7F800000u);
+            }
+            fin = emax != 0x7F800000u;
         }
-        bool fin = true;
         float mn = 0.0f, mx = 0.0f;
-        // finite <=> exponent field not all ones: the largest exponent field of the vector decides
-        uint32_t emax = 0;
 #pragma unroll
         for (int c = 0; c < 32; ++c) {
-            emax = max(emax, __float_as_uint(v[c]) & 0x7F800000u);
             mn = c == 0 ? v[c] : fminf(mn, v[c]);
             mx = c == 0 ? v[c] : fmaxf(mx, v[c]);
         }
-        fin = emax != 0x7F800000u;
         if (!fin) err |= OMMX_ERR_NONFINITE_V;
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
         const Step st = make_step(raw, scale_mode, tab);
@@ -473,7 +487,7 @@ extern "C" int ommx_store_pack(const void* K, const void* V, int in_dtype,
     }
     const dim3 grid(T / 32, H), block(D);
     const size_t shm = 32 * (size_t)D + 4 * (size_t)D + (index_repr ? 8 * (size_t)D : 0);
-    const bool tuned = k_outliers == 6 && !select_abs && scale_mode == 0 && k_ms;   // the serving recipe
+    const bool tuned = k_outliers == 6 && !select_abs && scale_mode == 0 && k_ms && D == 128;   // the serving recipe
     if (in_dtype == 1)
         hipLaunchKernelGGL((store_pack_kernel<true, false, 2>), grid, block, shm, st, a);
     else if (tuned && index_repr == 0)
