@@ -57,7 +57,7 @@ def check_serving_recipe(*, k_format: str, outlier_select: str, outlier_repr: st
     if group_tokens not in (16, 32, 64, 128):
         raise ValueError(f"group_tokens must be in {{16,32,64,128}}; got {group_tokens}")
     bad = []
-    if str(v_format).lower() != "i2":
+    if str(v_format).lower() not in ("i2", "bf16"):
         bad.append(f"v_format={v_format!r}")
     if str(outlier_repr).lower() == "combinadic" and k > 8:
         bad.append("combinadic ranks with more than 8 outliers (their decode twin is the bitmask plane)")

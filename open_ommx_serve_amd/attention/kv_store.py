@@ -67,7 +67,9 @@ class CanonicalKVStore:
                              scale_dtype=scale_dtype, outliers_per_vector=outliers_per_vector,
                              v_format=v_format)
         self.D, self.H, self.max_seq_len = int(head_dim), int(n_kv_heads), int(max_seq_len)
-        self.k_format, self.v_format = str(k_format).lower(), "i2"     # "itf4" is the same format
+        # "itf4" names the same K planes; V is INT2 codes or, with "bf16", the rows as they came
+        # (kv_store.py:120-127, 183-188)
+        self.k_format, self.v_format = str(k_format).lower(), str(v_format).lower()
         self.k = int(outliers_per_vector)
         self.outlier_select = str(outlier_select).lower()
         self.outlier_repr = str(outlier_repr).lower()
@@ -89,7 +91,10 @@ class CanonicalKVStore:
 
         dev, bf, z = self.device, torch.bfloat16, torch.zeros
         self.k_base = z(self.P_cap, self.ps, self.H, self.k_base_w, dtype=torch.uint8, device=dev)
-        self.v_main = z(self.P_cap, self.ps, self.H, self.D // 4, dtype=torch.uint8, device=dev)
+        if self.v_format == "bf16":
+            self.v_main = z(self.P_cap, self.ps, self.H, self.D, dtype=bf, device=dev)
+        else:
+            self.v_main = z(self.P_cap, self.ps, self.H, self.D // 4, dtype=torch.uint8, device=dev)
         sdt = torch.int8 if self.kv_int8_scale else bf      # exponents, or the steps themselves
         self.k_scale = z(self.G_cap, self.H, self.D, dtype=sdt, device=dev)
         self.k_zp = z(self.G_cap, self.H, self.D, dtype=bf, device=dev)
@@ -287,7 +292,7 @@ class CanonicalKVStore:
         store_pack_into(K_blk, V_blk, self._planes_for_store(), outliers_per_vector=self.k,
                         outlier_repr=self.outlier_repr, outlier_select=self.outlier_select,
                         use_pow2=self.use_pow2, kv_int8_scale=self.kv_int8_scale,
-                        group_tokens=self.gt, group_channels=self.gc,
+                        group_tokens=self.gt, group_channels=self.gc, v_format=self.v_format,
                         page_size=self.ps, src_rows=src_rows,
                         dst_pages=self._req_to_token_full.view(-1)[g0 * ppg:g1 * ppg],
                         dst_groups=self._req_to_group_full.view(-1)[g0:g1],

@@ -262,7 +262,9 @@ def test_store_classes_refuse_other_recipes_and_the_cpu():
                          group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
     check_serving_recipe(**{**good, "outlier_repr": "relidx7"}, kv_outlier_map=True, kv_int8_scale=True,
                          group_tokens=32, group_channels=32, scale_dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError, match="v_format"):
+    with pytest.raises(ValueError, match="v_format"):
+        CanonicalKVStore(128, 8, 256, device="cpu", v_format="fp8", **good)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):          # bf16 V rows are a served recipe
         CanonicalKVStore(128, 8, 256, device="cpu", v_format="bf16", **good)
     with pytest.raises(ValueError, match="k_format"):
         MultiSeqKVPool(128, 8, 2, 256, device="cpu", **{**good, "k_format": "i3"})

@@ -148,7 +148,7 @@ def _decode_bundle(q, bundle, sm_scale, k):
     return o.cpu(), lse.cpu()
 
 
-def _oracle_decode(q, K_hist, V_hist, win, sm_scale, packed_for=None):
+def _oracle_decode(q, K_hist, V_hist, win, sm_scale, packed_for=None, v_format="i2"):
     """Dequantise-then-attend over the full history of every request (fp64).  ``packed_for``:
     the lengths the planes were last packed for (default: the current ones); rows past that
     boundary are attended as bf16."""
@@ -163,7 +163,8 @@ def _oracle_decode(q, K_hist, V_hist, win, sm_scale, packed_for=None):
         Kd = torch.stack(Kf) if Kf else torch.zeros(0, *K.shape[1:])
         Vd = torch.stack(Vf) if Vf else torch.zeros(0, *V.shape[1:])
         if edge > win.sink_tokens:
-            planes = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size)
+            planes = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size,
+                               v_format=v_format)
             Kp, Vp = O.dequant_kv(planes)
             Kd, Vd = torch.cat([Kp, Kd]), torch.cat([Vp, Vd])
         o, lse = O.attend(q[b].cpu(), Kd, Vd, sm_scale, dtype=torch.float64)
@@ -453,6 +454,49 @@ def test_store_prefill_write_token_advance_and_decode(ring):
     st.check_errors()
     st.reset_inplace()
     assert st.seq_len == 0 and st.packed_groups == 0
+
+
+@pytest.mark.parametrize("ring", [False, True])
+def test_store_with_v_kept_as_bf16_rows(ring):
+    """``v_format="bf16"`` on the single-sequence store (kv_store.py:120-127, 183-188): V rows go
+    into ``v_main`` as they come, K is packed as always.  Planes bit for bit against the oracle
+    packer after the prefill and after every incremental pack, decode against the oracle."""
+    H, D, Hq = 4, 128, 16
+    win = WindowSpec()
+    prefill, steps = 200, 40
+    K, V = synth_kv(prefill + steps, H, D, seed=91, sparse_frac=0.005)
+    st = CanonicalKVStore(D, H, max_seq_len=400, window=win, device=DEV, kv_ring=ring, v_format="bf16", **RECIPE)
+    assert st.v_main.dtype == torch.bfloat16 and tuple(st.v_main.shape[1:]) == (win.page_size, H, D)
+
+    def planes_equal(n, what):
+        got, edge = st.decode_planes(), win.boundary(n)
+        assert got["v_format"] == "bf16" and got["num_tokens"] == edge - win.sink_tokens
+        want = O.pack_kv(K[win.sink_tokens:edge], V[win.sink_tokens:edge], page_size=win.page_size, v_format="bf16")
+        for name in PLANE_NAMES:
+            a, b = got[name].cpu(), want[name]
+            assert a.shape == b.shape and a.dtype == b.dtype, (what, name, a.shape, b.shape, a.dtype, b.dtype)
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"{what}: plane {name} differs"
+
+    st.append_block(K[:prefill].to(DEV), V[:prefill].to(DEV))
+    planes_equal(prefill, "prefill")
+    pos = torch.zeros(1, dtype=torch.int64, device=DEV)
+    sm_scale = 1.0 / math.sqrt(D)
+    qs = synth_q(steps, Hq, D, seed=10)
+    packs = 0
+    for s in range(steps):
+        n = prefill + s + 1
+        pos.fill_(n - 1)
+        st.write_token(pos, K[n - 1].to(DEV), V[n - 1].to(DEV))
+        if st.advance_to(n):
+            packs += 1
+            planes_equal(n, f"step {s}")
+        if s % 13 == 0 or s == steps - 1:
+            q = qs[s:s + 1].to(DEV)
+            got = _decode_bundle(q, st.decode_inputs(), sm_scale, 6)
+            want = _oracle_decode(q, [K[:n]], [V[:n]], win, sm_scale, v_format="bf16")
+            _check_out(got, want, f"bf16 V store ring={ring} step {s}")
+    assert packs >= 1
+    st.check_errors()
 
 
 def test_store_reports_a_position_outside_its_history():
