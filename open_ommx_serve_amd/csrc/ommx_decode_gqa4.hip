@@ -167,13 +167,17 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
             qraw[r] = *reinterpret_cast<const uint32_t*>(
                 a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
     }
-    // The 32-token groups are dealt out evenly: split s takes groups [s*G/S, (s+1)*G/S), so no two
-    // splits differ by more than one group and none is empty while G >= S.  (The combine weighs the
-    // states by their lse, -inf for an empty split, so it need not know this rule.)
+    // The 32-token groups are dealt out evenly: every split takes G/S groups and the first G%S
+    // splits one more, so no two splits differ by more than one group and none is empty while
+    // G >= S.  (One 32-bit division; the combine weighs the states by their lse, -inf for an
+    // empty split, so it need not know this rule.)
     if (L < 0) { L = 0; report_table_range(a.err, true); }      // a negative length: nothing packed, reported
-    const int G = (L + 31) >> 5;
-    const int n_begin = static_cast<int>((static_cast<int64_t>(sp) * G) / a.S) << 5;
-    const int n_end = min(static_cast<int>((static_cast<int64_t>(sp + 1) * G) / a.S) << 5, L);
+    const uint32_t G = static_cast<uint32_t>(L + 31) >> 5, S = static_cast<uint32_t>(a.S);
+    const uint32_t g_each = G / S, g_more = G - g_each * S;
+    const uint32_t g_first = static_cast<uint32_t>(sp) * g_each + min(static_cast<uint32_t>(sp), g_more);
+    const uint32_t g_count = g_each + (static_cast<uint32_t>(sp) < g_more ? 1u : 0u);
+    const int n_begin = static_cast<int>(g_first << 5);
+    const int n_end = min(static_cast<int>((g_first + g_count) << 5), L);
 
     if (n_begin >= n_end) {       // an empty split: the state of nothing attended
         for (int r = 0; r < heads; ++r) {
