@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define OMMX_ABI_VERSION 7   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
+#define OMMX_ABI_VERSION 8   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
                                 5: decode without a workspace argument; 6: plane extents + error flag on
                                 the decode entry points, up to 512 splits */
 
@@ -208,7 +208,10 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
  * b_tail_len == NULL (then k_tail, v_tail, q may be NULL too) combines the splits alone:
  * the un-merged state of a group-range segment (paged_decode.py:2892-2902).
  * k_tail rows must be 16-byte aligned (base pointer and strides multiples of 8 elements);
- * num_splits <= 512.
+ * num_splits <= 512.  tail_rows = Tmax, the rows every request's tail buffer holds (0 when
+ * unknown): the kernel asks for the first min(64, tail_rows) rows before b_tail_len has
+ * arrived, which takes one memory round trip off its critical path; rows past a request's
+ * b_tail_len are read but never used, so they only have to be addressable.
  */
 int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,
@@ -220,7 +223,7 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
                         float* o, int64_t o_stride_b, int64_t o_stride_h,
                         float* lse, int64_t lse_stride_b,
                         int B, int Hq, int Hkv, int D, int num_splits, int group_tokens,
-                        float sm_scale, float logit_cap, void* stream);
+                        int tail_rows, float sm_scale, float logit_cap, void* stream);
 
 /*
  * Whole decode step (split-KV stage, then the combine with the bf16 tail) for callers that
@@ -251,7 +254,7 @@ int ommx_decode_attention_noalloc(
     const int32_t* b_tail_len,
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int v_bf16, int num_splits,
+    int group_tokens, int group_channels, int v_bf16, int num_splits, int tail_rows,
     float sm_scale, float logit_cap, int packed_start_offset,
     int num_pages, int num_group_slots, int32_t* err_flag, void* stream);
 

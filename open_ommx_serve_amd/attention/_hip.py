@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 _lib: Optional[C.CDLL] = None
 
 STORE_TABLE_FLOATS = 264
-ABI_VERSION = 7
+ABI_VERSION = 8
 INDEX_BITMAP, INDEX_RELIDX7, INDEX_COMBINADIC = 0, 1, 2
 SCALE_POW2_INT8, SCALE_POW2_BF16, SCALE_BF16 = 0, 1, 2
 
@@ -56,13 +56,13 @@ _SIGNATURES = {
     "ommx_decode_splitkv_ref": (_I, _DECODE_ARGS),
     "ommx_clamp_table_id": (_I, [_I, _I, _P]),
     "ommx_decode_combine": (_I, [_P, _L, _L, _L, _P, _L, _L, _P, _P, _L, _L, _L, _L, _L, _L,
-                                 _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _I, _F, _F, _P]),
+                                 _P, _P, _P, _L, _L, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P]),
     "ommx_decode_attention_noalloc": (_I, [
         _P, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P,      # q, K planes, V planes
         _P, _L, _P, _L, _I, _P,                                  # tables, b_seq_len
         _P, _P, _L, _L, _L, _L, _L, _L, _P,                      # tail rows, strides, b_tail_len
         _P, _L, _L, _P, _L,                                      # o, lse
-        _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,          # B Hq Hkv D ps kout repr scale_bf16 gt gc v_bf16 S
+        _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,      # B Hq Hkv D ps kout repr scale_bf16 gt gc v_bf16 S tail_rows
         _F, _F, _I, _I, _I, _P, _P]),                            # sm_scale cap off num_pages num_group_slots err stream
     "ommx_ring_write": (_I, [_P, _P, _L, _L, _L, _L, _P, _P, _L, _I, _P, _P, _P,
                              _I, _I, _I, _I, _I, _P, _P]),

@@ -349,7 +349,8 @@ def ommx_paged_decode_attention_canonical(
             attn_logits.data_ptr(), attn_logits.stride(0), attn_logits.stride(1), attn_logits.stride(2),
             q.data_ptr(), q.stride(0), q.stride(1), *tail_args[:8], tail_args[8], b_seq_len.data_ptr(),
             o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(0),
-            B, Hq, Hkv, D, S, group_tokens, float(sm_scale), float(logit_cap), stream)
+            B, Hq, Hkv, D, S, group_tokens, int(k_tail.shape[1]) if has_tail else 0,
+            float(sm_scale), float(logit_cap), stream)
         _hip.check(rc, "ommx_decode_combine")
 
 

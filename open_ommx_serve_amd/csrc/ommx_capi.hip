@@ -135,11 +135,11 @@ extern "C" int ommx_decode_combine(
     int64_t vt_stride_b, int64_t vt_stride_t, int64_t vt_stride_h,
     const int32_t* b_tail_len, const int32_t* b_seq_len,
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
-    int B, int Hq, int Hkv, int D, int num_splits, int group_tokens, float sm_scale, float logit_cap,
-    void* stream) {
+    int B, int Hq, int Hkv, int D, int num_splits, int group_tokens, int tail_rows, float sm_scale,
+    float logit_cap, void* stream) {
     using namespace ommx;
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || num_splits < 1 || !(D == 64 || D == 128) ||
-        group_tokens < 16 || group_tokens > 128 || (group_tokens & (group_tokens - 1))) {
+        group_tokens < 16 || group_tokens > 128 || (group_tokens & (group_tokens - 1)) || tail_rows < 0) {
         set_error("ommx_decode_combine: bad shape");
         return -1;
     }
@@ -161,7 +161,7 @@ extern "C" int ommx_decode_combine(
                   k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h,
                   vt_stride_b, vt_stride_t, vt_stride_h, b_tail_len, b_seq_len,
                   o, o_stride_b, o_stride_h, lse, lse_stride_b, B, Hq, Hkv, num_splits,
-                  sm_scale, logit_cap, group_tokens};
+                  sm_scale, logit_cap, group_tokens, b_tail_len ? tail_rows : 0};
     if (launch_combine(a, D, static_cast<hipStream_t>(stream)) != 0) {
         set_error("ommx_decode_combine: unsupported head_dim");
         return -1;
@@ -279,7 +279,7 @@ extern "C" int ommx_decode_attention_noalloc(
     const int32_t* b_tail_len,
     float* o, int64_t o_stride_b, int64_t o_stride_h, float* lse, int64_t lse_stride_b,
     int B, int Hq, int Hkv, int D, int page_size, int k_outliers, int index_repr, int scale_bf16,
-    int group_tokens, int group_channels, int v_bf16, int num_splits,
+    int group_tokens, int group_channels, int v_bf16, int num_splits, int tail_rows,
     float sm_scale, float logit_cap, int packed_start_offset,
     int num_pages, int num_group_slots, int32_t* err_flag, void* stream) {
     using namespace ommx;
@@ -314,5 +314,5 @@ extern "C" int ommx_decode_attention_noalloc(
                                k_tail, v_tail, kt_stride_b, kt_stride_t, kt_stride_h, vt_stride_b,
                                vt_stride_t, vt_stride_h, b_tail_len, b_seq_len, o, o_stride_b,
                                o_stride_h, lse, lse_stride_b, B, Hq, Hkv, D, num_splits, group_tokens,
-                               sm_scale, logit_cap, stream);
+                               tail_rows, sm_scale, logit_cap, stream);
 }

@@ -81,18 +81,27 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
     // Every quarter computes all the logits (they need the whole q and K rows) and its own
     // channels of P.V.
     float t_m = -INFINITY, t_l = 0.0f, t_acc = 0.0f;
-    for (int r0 = 0; r0 < tail; r0 += ROWS) {
-        const int nr = min(ROWS, tail - r0);
-        // loads first: 16 bytes of one K row, PER elements of V
-        const int row = tid >> 4, part = tid & 15;
-        const uint4 ku = *reinterpret_cast<const uint4*>(
-            a.kt + b * a.kt_b + (int64_t)(r0 + min(row, nr - 1)) * a.kt_t + (int64_t)kvh * a.kt_h +
+    const int row = tid >> 4, part = tid & 15;
+    // loads of one chunk: 16 bytes of one K row, PER elements of V; rows from `last` on repeat it
+    uint4 ku;
+    uint32_t vv[PER];
+    auto load_rows = [&](int r0, int last) {
+        ku = *reinterpret_cast<const uint4*>(
+            a.kt + b * a.kt_b + (int64_t)(r0 + min(row, last)) * a.kt_t + (int64_t)kvh * a.kt_h +
             (part * 8) % D);
-        uint32_t vv[PER];
 #pragma unroll
         for (int i = 0; i < PER; ++i)
-            vv[i] = a.vt[b * a.vt_b + (int64_t)(r0 + min(sg + NSG * i, nr - 1)) * a.vt_t +
+            vv[i] = a.vt[b * a.vt_b + (int64_t)(r0 + min(sg + NSG * i, last)) * a.vt_t +
                          (int64_t)kvh * a.vt_h + d];
+    };
+    // When the caller has said how many rows the tail buffers hold, the first chunk is asked for
+    // here, with the split loads and before the tail length has arrived (its uses below wait for
+    // it): rows past the tail are addressable, and neither their logits nor their V are used.
+    const bool early = a.T > 0 && a.tail != nullptr;
+    if (early) load_rows(0, min(ROWS, a.T) - 1);
+    for (int r0 = 0; r0 < tail; r0 += ROWS) {
+        const int nr = min(ROWS, tail - r0);
+        if (!(early && r0 == 0)) load_rows(r0, nr - 1);
         __syncthreads();                              // s_q ready (and previous chunk consumed)
         float dot = 0.0f;
         if (part * 8 < D) {
@@ -108,12 +117,12 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
         for (int o = 1; o < 16; o <<= 1) dot += __shfl_xor(dot, o);
         if (part == 0) s_logit[row] = row < nr ? apply_cap(dot * a.sm_scale, a.cap) : -INFINITY;
         __syncthreads();
-        float mx = -INFINITY;                         // s_logit holds -inf past nr
+        // maximum of the chunk's logits: one logit per lane, reduced over the wave (every thread
+        // reading all ROWS of them cost 16 LDS reads of 16 bytes each); s_logit holds -inf past nr
+        static_assert(ROWS <= 64, "one logit per lane");
+        float mx = (tid & 63) < ROWS ? s_logit[tid & 63] : -INFINITY;
 #pragma unroll
-        for (int i = 0; i < ROWS / 4; ++i) {
-            const float4 v4 = reinterpret_cast<const float4*>(s_logit)[i];
-            mx = fmaxf(mx, fmaxf(fmaxf(v4.x, v4.y), fmaxf(v4.z, v4.w)));
-        }
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
         const float m_new = fmaxf(t_m, mx);
         const float alpha = (t_m == -INFINITY) ? 0.0f : __expf(t_m - m_new);
         t_l *= alpha;

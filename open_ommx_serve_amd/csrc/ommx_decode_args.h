@@ -66,6 +66,8 @@ struct CombineArgs {
     int B, Hq, Hkv, S;
     float sm_scale, cap;
     int gt;                          // tokens per K group: the splits are rounded to it
+    int T;                           // rows every request's tail buffer holds (0: not told): rows below it
+                                     // may be read before b_tail_len has arrived
 };
 
 int launch_decode_ref(const DecodeArgs& a, int D, int R, hipStream_t st);

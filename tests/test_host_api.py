@@ -33,7 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     for n in names:
         assert getattr(raw, n) is not None, n
     assert set(_hip.exported_symbols()) == set(names)
-    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 7
+    assert lib.ommx_abi_version() == _hip.ABI_VERSION == 8
 
 
 def test_default_decision_table_is_the_exact_arithmetic_one():

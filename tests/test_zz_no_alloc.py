@@ -44,7 +44,7 @@ def _noalloc(case, S):
             case.b_tail_len.data_ptr(),
             o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(0),
             B, Hq, case.kv_heads, D, case.page_size, case.outliers_per_vector, _hip.INDEX_BITMAP, 0,
-            32, 32, 0, S, float(case.sm_scale), 0.0, 0, int(p["k_base"].shape[0]), int(p["k_scale"].shape[0]), None,
+            32, 32, 0, S, int(case.k_tail.shape[1]), float(case.sm_scale), 0.0, 0, int(p["k_base"].shape[0]), int(p["k_scale"].shape[0]), None,
             _hip.current_stream_ptr(dev))
     return rc, o, lse
 
