@@ -15,6 +15,33 @@
 
 namespace ommx {
 
+namespace {
+// Lane exchanges inside the vector ALU (DPP): no trip through the LDS crossbar, no index arithmetic.
+template <int CTRL>
+__device__ __forceinline__ float dpp_of(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+// sum over each row of 16 lanes, left in every lane of the row
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_of<0xB1>(v);        // quad_perm [1,0,3,2]
+    v += dpp_of<0x4E>(v);        // quad_perm [2,3,0,1]
+    v += dpp_of<0x141>(v);       // row_half_mirror
+    v += dpp_of<0x140>(v);       // row_mirror
+    return v;
+}
+// maximum over the 64 lanes, uniform
+__device__ __forceinline__ float wave64_max(float v) {
+    v = fmaxf(v, dpp_of<0xB1>(v));
+    v = fmaxf(v, dpp_of<0x4E>(v));
+    v = fmaxf(v, dpp_of<0x141>(v));
+    v = fmaxf(v, dpp_of<0x140>(v));
+    v = fmaxf(v, dpp_of<0x142>(v));      // row_bcast15: lane 15 of a row into the next row
+    v = fmaxf(v, dpp_of<0x143>(v));      // row_bcast31: lane 31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+}  // namespace
+
 // NT threads per workgroup, at most MAXS splits: 1024 / 256 in general, 512 / 64 when many
 // (request, head) pairs with few splits each fill the chip (fewer idle lanes per workgroup).
 template <int D, int Q, int NT = 1024, int MAXS = 256>
@@ -71,9 +98,7 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
 
     if (tid < D) s_q[tid] = __uint_as_float(q_raw << 16);
     if (tid < MAXS) {
-        float wm = my_lse;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) wm = fmaxf(wm, __shfl_xor(wm, o));
+        const float wm = wave64_max(my_lse);
         if ((tid & 63) == 0) s_wmax[tid >> 6] = wm;
     }
 
@@ -113,16 +138,13 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
                 dot = fmaf(qq[2 * i + 1], __uint_as_float(w[i] & 0xFFFF0000u), dot);
             }
         }
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) dot += __shfl_xor(dot, o);
+        dot = row16_sum(dot);
         if (part == 0) s_logit[row] = row < nr ? apply_cap(dot * a.sm_scale, a.cap) : -INFINITY;
         __syncthreads();
         // maximum of the chunk's logits: one logit per lane, reduced over the wave (every thread
         // reading all ROWS of them cost 16 LDS reads of 16 bytes each); s_logit holds -inf past nr
         static_assert(ROWS <= 64, "one logit per lane");
-        float mx = (tid & 63) < ROWS ? s_logit[tid & 63] : -INFINITY;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        const float mx = wave64_max((tid & 63) < ROWS ? s_logit[tid & 63] : -INFINITY);
         const float m_new = fmaxf(t_m, mx);
         const float alpha = (t_m == -INFINITY) ? 0.0f : __expf(t_m - m_new);
         t_l *= alpha;
