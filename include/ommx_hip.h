@@ -28,7 +28,8 @@ extern "C" {
 
 #define OMMX_ABI_VERSION 8   /* 2: ring, tail-gather, state-merge; 3: index_repr arguments; 4: index-plane conversion;
                                 5: decode without a workspace argument; 6: plane extents + error flag on
-                                the decode entry points, up to 512 splits */
+                                the decode entry points, up to 512 splits; 7: packed_lag on the tail gather;
+                                8: tail_rows on the combine and on the decode without a workspace */
 
 /* step of the INT2 quantisers and the dtype of the k_scale / v_scale planes */
 #define OMMX_SCALE_POW2_INT8  0
