@@ -306,8 +306,8 @@ def ommx_paged_decode_attention_canonical(
             mean_seq_len = sum(lens) / len(lens)
     else:
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
-    # the kernel for up to 4 q heads per kv head (serving recipe shapes) keeps three workgroups per
-    # compute unit resident, the others two; it also serves the call in one launch
+    # the serving-recipe kernel keeps three workgroups per compute unit resident with up to 4 q heads
+    # per kv head (two with 8, and so do the other kernels); it also serves the call in one launch
     lean = (D == 128 and Hq // Hkv <= 4 and k == 6 and group_tokens == 32 and group_channels == 32
             and not scale_bf16 and not v_bf16 and not _force_reference_kernel)
     if num_kv_splits is None:

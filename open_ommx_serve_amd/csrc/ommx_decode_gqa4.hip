@@ -1,8 +1,8 @@
-// Split-KV decode kernel for gfx950, serving shape: head_dim 128, 1, 2 or 4 q heads per kv head,
+// Split-KV decode kernel for gfx950, serving shape: head_dim 128, 1, 2, 4 or 8 q heads per kv head,
 // 6 outliers per K vector of 32 tokens (either index plane, either outlier map), INT2 V with
 // 32-channel vectors, int8 exponents.  Same operator as
 // ommx_gpu_serve/attention/paged_decode.py:1255-2284; the other shapes of the matrix-core path
-// (8 q heads per kv head, longer groups, no outliers) stay on the kernel in ommx_decode.hip.
+// (longer groups, no outliers) stay on the kernel in ommx_decode.hip.
 //
 // A wavefront owns one kv head (and its q heads) of one split and walks it 64 tokens at a time;
 // a workgroup is 4 waves = 4 neighbouring kv heads.  Measured on MI355X this operator is bound
@@ -17,6 +17,10 @@
 //     p*zp (a row of ones), the running maximum is refreshed only when a logit exceeds it by
 //     more than 2^8 (any bound that keeps exp2 in range serves an online softmax);
 //   * the V staging area of LDS is the K staging area of the same step, reused once QK is done.
+// With 8 q heads per kv head (NH = 8) the sixteen matrix rows / columns are two replicas of the
+// heads instead of four: a lane then keeps four heads of one token of either group, the output
+// takes four accumulators, and two workgroups fit a compute unit (190 registers, 14.1 KB of LDS
+// per wave); everything up to the logits is the same code.
 // Arithmetic: exact 16-bit operands, fp32 accumulation, as in ommx_decode.hip.
 //   A (QK)   q * 2^(10-2m) as f16 in pair order, m = 1..4 fixed per channel pair; this one operand
 //            set serves the base codes, the outlier tile and the bias columns.
@@ -62,16 +66,21 @@ constexpr int OFF_MAG = OFF_KT + 64 * KT_ROW;       // [2 groups][128] f16 2^e, 
 constexpr int OFF_ZPP = OFF_MAG + 512;              // same order, f16 zero points over the A scale
 // after QK the same bytes hold what P.V needs
 constexpr int OFF_VT = OFF_KT;                      // [8 dword columns][VT_COL] V code dwords
-constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [4 heads][PT_ROW] f16 softmax weights
-constexpr int OFF_VZ = OFF_PT + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 V zero points
-constexpr int OFF_VS = OFF_VZ + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 2^e_v
-constexpr int OFF_STAGE_END = (OFF_VS + 4 * PT_ROW * 2 > OFF_ZPP + 512) ? OFF_VS + 4 * PT_ROW * 2 : OFF_ZPP + 512;
-constexpr int OFF_LC = OFF_STAGE_END;                 // [32 tokens][4 heads] f32 logit corrections of one group
-constexpr int OFF_ZERO = OFF_LC + 512;              // 128 B of zeros, never written again
-constexpr int OFF_ONES = OFF_ZERO + 128;            // 128 B of f16 1.0, never written again
-constexpr int LDS_WAVE = OFF_ONES + 128;            // 13568: three 4-wave workgroups fit a CU's 160 KB
-static_assert(OFF_KT % 16 == 0 && OFF_PT % 16 == 0 && OFF_VZ % 16 == 0 && OFF_LC % 16 == 0, "b128 alignment");
-static_assert(3 * 4 * LDS_WAVE <= 160 * 1024, "three workgroups per compute unit");
+constexpr int OFF_PT = OFF_VT + 8 * VT_COL * 4;     // [NH heads][PT_ROW] f16 softmax weights
+// what follows the weights depends on the number of q heads per kv head (NH = 4 or 8)
+template <int NH>
+struct LdsMap {
+    static constexpr int OFF_VZ = OFF_PT + NH * PT_ROW * 2;    // [4 channel groups][PT_ROW] f16 V zero points
+    static constexpr int OFF_VS = OFF_VZ + 4 * PT_ROW * 2;     // [4 channel groups][PT_ROW] f16 2^e_v
+    static constexpr int OFF_STAGE_END = (OFF_VS + 4 * PT_ROW * 2 > OFF_ZPP + 512) ? OFF_VS + 4 * PT_ROW * 2 : OFF_ZPP + 512;
+    static constexpr int OFF_LC = OFF_STAGE_END;               // [32 tokens][NH heads] f32 logit corrections of one group
+    static constexpr int OFF_ZERO = OFF_LC + 32 * NH * 4;      // 128 B of zeros, never written again
+    static constexpr int OFF_ONES = OFF_ZERO + 128;            // 128 B of f16 1.0, never written again
+    static constexpr int LDS_WAVE = OFF_ONES + 128;            // 13568 (4 heads) / 14656 (8 heads)
+    static_assert(OFF_KT % 16 == 0 && OFF_PT % 16 == 0 && OFF_VZ % 16 == 0 && OFF_LC % 16 == 0, "b128 alignment");
+};
+static_assert(3 * 4 * LdsMap<4>::LDS_WAVE <= 160 * 1024, "4 heads: three workgroups per compute unit");
+static_assert(2 * 4 * LdsMap<8>::LDS_WAVE <= 160 * 1024, "8 heads: two workgroups per compute unit");
 
 // One f16 carries 11 bits: rounding an outlier delta d costs up to |d| * 2^-11, i.e. up to
 // |d| * max|q| * 2^-11 * sm_scale on a logit.  A delta with |d| * max|q| >= BIG_DELTA * 16
@@ -106,8 +115,13 @@ __device__ __forceinline__ uint32_t pk_u16(uint32_t lo, uint32_t hi) { return (l
 // base scale and zero point.  PARTIAL: the kv head serves 1 or 2 q heads (spare head slots repeat
 // the last head and are not written).  ORDER: 0 one request, 1 up to 64 requests served longest
 // first, 2 up to 256 (radix select); see ommx_decode.hip.
-template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER>
-__global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
+// NH: q heads per kv head the matrix rows and columns are laid out for, 4 or 8.
+template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER, int NH = 4>
+__global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
+    static_assert(NH == 4 || (NH == 8 && !PARTIAL), "4 heads (or fewer, PARTIAL) or exactly 8");
+    using Lds = LdsMap<NH>;
+    constexpr int OFF_VZ = Lds::OFF_VZ, OFF_VS = Lds::OFF_VS, OFF_LC = Lds::OFF_LC, OFF_ZERO = Lds::OFF_ZERO,
+                  OFF_ONES = Lds::OFF_ONES, LDS_WAVE = Lds::LDS_WAVE;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_all[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // uniform: keeps the plane pointers scalar
@@ -118,7 +132,7 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     const int Hkv = a.Hkv;
     const int waves = blockDim.x >> 6;
     const int kvh = blockIdx.y * waves + wave;
-    const int heads = PARTIAL ? a.Hq / Hkv : 4;
+    const int heads = PARTIAL ? a.Hq / Hkv : NH;
     const int qh0 = kvh * heads;
     const int sp = blockIdx.x;
     int b = blockIdx.z, L;
@@ -154,16 +168,16 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     } else {
         L = a.seq[b];
     }
-    // q: this lane's 32 channels of head j % 4 (16 dwords, channel 2i in the low half of dword i)
+    // q: this lane's 32 channels of head j % NH (16 dwords, channel 2i in the low half of dword i)
     // and channels 2*lane, 2*lane+1 of every head (for the channel pass)
-    uint32_t qw[16], qraw[4];      // qraw: channels 2*lane, 2*lane+1 of every head, for the thresholds below
+    uint32_t qw[16], qraw[NH];      // qraw: channels 2*lane, 2*lane+1 of every head, for the thresholds below
     {
         const uint32_t* qh = reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & 3, heads - 1)) * a.q_sh + 32 * kq);
+            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & (NH - 1), heads - 1)) * a.q_sh + 32 * kq);
 #pragma unroll
         for (int i = 0; i < 16; ++i) qw[i] = qh[i];
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < NH; ++r)
             qraw[r] = *reinterpret_cast<const uint32_t*>(
                 a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
     }
@@ -270,12 +284,17 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     {
         u32x4* p = reinterpret_cast<u32x4*>(sm + OFF_TILE);
         for (int i = lane; i < 32 * TILE_ROW / 16; i += 64) p[i] = u32x4{0, 0, 0, 0};
-        if (lane < 32) reinterpret_cast<u32x4*>(sm + OFF_LC)[lane] = u32x4{0, 0, 0, 0};
+        if (lane < 8 * NH) reinterpret_cast<u32x4*>(sm + OFF_LC)[lane] = u32x4{0, 0, 0, 0};
         if (lane < 16) reinterpret_cast<u32x4*>(sm + OFF_ZERO)[lane] =
             lane < 8 ? u32x4{0, 0, 0, 0} : u32x4{0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
     }
 
-    f32x4 acc[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
+    // output accumulators: with 4 heads the 16 columns are 4 replicas of the heads and replica x takes
+    // the channel blocks Y = x, x + 4 (two accumulators); with 8 heads they are 2 replicas and replica x
+    // takes Y = x, x + 2, x + 4, x + 6 (four)
+    f32x4 acc[NH / 2];
+#pragma unroll
+    for (int i = 0; i < NH / 2; ++i) acc[i] = f32x4{0, 0, 0, 0};
     f32x4 accz = {0, 0, 0, 0};
     float m_run[4];
 #pragma unroll
@@ -326,7 +345,7 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     for (int u = 0; u < 2; ++u) {
         float qm = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < NH; ++r)
             qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
         big_thr[u] = (BIG_DELTA * 16.0f) * (u ? cs1 : cs0) * __builtin_amdgcn_rcpf(qm);
     }
@@ -386,7 +405,12 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
 #endif
 
         // ------------------------------------------------------------------ QK
-        f32x4 dsel = {0, 0, 0, 0};
+        // 4 heads: the lane keeps the logits of its own token n0 + lane (one 16-token block of one group);
+        // 8 heads: rows 4kq..4kq+3 are heads 4(kq & 1)..+3, and the lane keeps those four heads of token
+        // 16(kq >> 1) + j of either group
+        f32x4 dsel[NH / 4];
+#pragma unroll
+        for (int i = 0; i < NH / 4; ++i) dsel[i] = f32x4{0, 0, 0, 0};
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             if (g == 1 && !g1_live) break;
@@ -457,8 +481,8 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
                         if (fabsf(dl) >= big_thr[u]) {
                             const float lo = (dl - static_cast<float>(hi)) * __builtin_amdgcn_rcpf(cs);
 #pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                __hip_atomic_fetch_add(lc + pos[sidx] * 4 + r, lo * q_of(u, r), __ATOMIC_RELAXED,
+                            for (int r = 0; r < NH; ++r)
+                                __hip_atomic_fetch_add(lc + pos[sidx] * NH + r, lo * q_of(u, r), __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
                         }
                     }
@@ -506,15 +530,25 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
                     d[t2] = mfma_f16(aq[2 * hf + 1], u32x4{k_pair<4>(w[t2], wu[t2], wd[t2], mb[0]), k_pair<5>(w[t2], wu[t2], wd[t2], mb[1]),
                                                            k_pair<6>(w[t2], wu[t2], wd[t2], mb[2]), k_pair<7>(w[t2], wu[t2], wd[t2], mb[3])}, d[t2]);
             }
-            // rows 4kq..4kq+3 of every result hold the four heads: the lane keeps its own token block
+            if constexpr (NH == 4) {
+                // rows 4kq..4kq+3 of every result hold the four heads: the lane keeps its own token block
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
-                if (kq == 2 * g + t2) dsel = d[t2];
-            if (res0 || res1) {       // exact residuals of this group's large deltas, then zero again
-                const f32x4 corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * (lane & 31));
-                if ((kq >> 1) == g) dsel += corr;
-                lds_fence();
-                *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * (lane & 31)) = u32x4{0, 0, 0, 0};
+                for (int t2 = 0; t2 < 2; ++t2)
+                    if (kq == 2 * g + t2) dsel[0] = d[t2];
+                if (res0 || res1) {       // exact residuals of this group's large deltas, then zero again
+                    const f32x4 corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * (lane & 31));
+                    if ((kq >> 1) == g) dsel[0] += corr;
+                    lds_fence();
+                    *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * (lane & 31)) = u32x4{0, 0, 0, 0};
+                }
+            } else {
+                dsel[g] = (kq >> 1) ? d[1] : d[0];
+                if (res0 || res1) {
+                    // the lane's token of this group, its four heads
+                    dsel[g] += *reinterpret_cast<const f32x4*>(sm + OFF_LC + 32 * (16 * (kq >> 1) + j) + 16 * (kq & 1));
+                    lds_fence();
+                    *reinterpret_cast<u32x4*>(sm + OFF_LC + 16 * lane) = u32x4{0, 0, 0, 0};
+                }
             }
             lds_fence();
         }
@@ -559,81 +593,170 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
         if (more) fetch_v();
 
         // ------------------------------------------------------------------ softmax
-        // the lane owns token n0 + lane and the four heads; bias of (group, head) = sum q*zp - sum A*2^e
-        float x[4];
-        {
-            const int gsel = lane >> 5;
+        if constexpr (NH == 4) {
+            // the lane owns token n0 + lane and the four heads; bias of (group, head) = sum q*zp - sum A*2^e
+            float x[4];
+            {
+                const int gsel = lane >> 5;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    // lane 0 / 1 of every row: column 0 / 1 (zp) minus column 2 / 3 (2^e)
+                    // (each row goes through a register of its own first: read straight out of the 4-register
+                    // result, the four moves came out as one, all reading row 0)
+                    float mine = dbias[r];
+                    asm volatile("" : "+v"(mine));
+                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                        0, __builtin_bit_cast(int, mine), 0x4E, 0xF, 0xF, true));     // quad_perm [2,3,0,1]
+                    x[r] = dsel[0][r] + lane_value(mine - other, gsel);
+                }
+            }
+            float pe[4];          // base-2 logit minus the running maximum
+            if (a.cap > 0.0f) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int r = 0; r < 4; ++r) x[r] = apply_cap(x[r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) pe[r] = x[r] - m_run[r];
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    x[r] *= c2;
+                    pe[r] = x[r] - m_run[r];
+                }
+            }
+            const bool tok_ok = n0 + lane < n_end;
+            if (n0 + 64 > n_end) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (!tok_ok) { x[r] = -INFINITY; pe[r] = -INFINITY; }
+                }
+            }
+            if (__any(fmaxf(fmaxf(pe[0], pe[1]), fmaxf(pe[2], pe[3])) > MAX_SLACK)) {
+                // refresh the running maxima (always on the first step) and rescale what is summed so far
+                float mxs[4] = {x[0], x[1], x[2], x[3]};
+                wave_max4(mxs);
+                float alpha[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float m_new = fmaxf(m_run[r], mxs[r]);
+                    alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                    m_run[r] = m_new;
+                    pe[r] = x[r] - m_new;
+                }
+                // accumulators hold column (x, head j % 4) in every register
+                const float al = (j & 3) == 0 ? alpha[0] : ((j & 3) == 1 ? alpha[1] : ((j & 3) == 2 ? alpha[2] : alpha[3]));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { acc[0][i] *= al; acc[1][i] *= al; accz[i] *= al; }
+            }
+            {
+                const uint32_t p01 = pack_f16x2(__builtin_amdgcn_exp2f(pe[0]), __builtin_amdgcn_exp2f(pe[1]));
+                const uint32_t p23 = pack_f16x2(__builtin_amdgcn_exp2f(pe[2]), __builtin_amdgcn_exp2f(pe[3]));
+                uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT) + lane;
+                pt[0] = static_cast<uint16_t>(p01);
+                pt[PT_ROW] = static_cast<uint16_t>(p01 >> 16);
+                pt[2 * PT_ROW] = static_cast<uint16_t>(p23);
+                pt[3 * PT_ROW] = static_cast<uint16_t>(p23 >> 16);
+            }
+        } else {
+            // the lane owns tokens n0 + 32g + 16(kq >> 1) + j, g = 0, 1, and heads 4(kq & 1)..+3.  Every quad
+            // of a row holds the bias columns (zp g0, zp g1, 2^e g0, 2^e g1) of the row's own heads.
+            float x[2][4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                // lane 0 / 1 of every row: column 0 / 1 (zp) minus column 2 / 3 (2^e)
-                // (each row goes through a register of its own first: read straight out of the 4-register
-                // result, the four moves came out as one, all reading row 0)
                 float mine = dbias[r];
                 asm volatile("" : "+v"(mine));
                 const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
                     0, __builtin_bit_cast(int, mine), 0x4E, 0xF, 0xF, true));     // quad_perm [2,3,0,1]
-                x[r] = dsel[r] + lane_value(mine - other, gsel);
+                float t = mine - other;                                           // lanes 0, 1 of a quad: bias of group 0, 1
+                asm volatile("" : "+v"(t));
+                x[0][r] = dsel[0][r] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                    0, __builtin_bit_cast(int, t), 0x00, 0xF, 0xF, true));        // quad_perm [0,0,0,0]
+                x[1][r] = dsel[1][r] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                    0, __builtin_bit_cast(int, t), 0x55, 0xF, 0xF, true));        // quad_perm [1,1,1,1]
             }
-        }
-        float pe[4];          // base-2 logit minus the running maximum
-        if (a.cap > 0.0f) {
-            asm volatile("" ::: "memory");
+            float pe[2][4];
+            if (a.cap > 0.0f) {
+                asm volatile("" ::: "memory");
 #pragma unroll
-            for (int r = 0; r < 4; ++r) x[r] = apply_cap(x[r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+                for (int g = 0; g < 2; ++g)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) pe[r] = x[r] - m_run[r];
-        } else {
+                    for (int r = 0; r < 4; ++r) x[g][r] = apply_cap(x[g][r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+            } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                x[r] *= c2;
-                pe[r] = x[r] - m_run[r];
+                for (int g = 0; g < 2; ++g)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) x[g][r] *= c2;
             }
-        }
-        const bool tok_ok = n0 + lane < n_end;
-        if (n0 + 64 > n_end) {
+            const int tk = 16 * (kq >> 1) + j;           // the lane's token inside either group
+            if (n0 + 64 > n_end) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (!tok_ok) { x[r] = -INFINITY; pe[r] = -INFINITY; }
+                for (int g = 0; g < 2; ++g) {
+                    const bool tok_ok = n0 + 32 * g + tk < n_end;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (!tok_ok) x[g][r] = -INFINITY;
+                }
             }
-        }
-        if (__any(fmaxf(fmaxf(pe[0], pe[1]), fmaxf(pe[2], pe[3])) > MAX_SLACK)) {
-            // refresh the running maxima (always on the first step) and rescale what is summed so far
-            float mxs[4] = {x[0], x[1], x[2], x[3]};
-            wave_max4(mxs);
-            float alpha[4];
+            float over = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float m_new = fmaxf(m_run[r], mxs[r]);
-                alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
-                m_run[r] = m_new;
-                pe[r] = x[r] - m_new;
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pe[g][r] = x[g][r] - m_run[r];
+                    over = fmaxf(over, pe[g][r]);
+                }
+            if (__any(over > MAX_SLACK)) {
+                // refresh the running maxima of the lane's four heads (rows kq and kq ^ 2 hold the same
+                // heads) and rescale what is summed so far
+                float mxs[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mxs[r] = fmaxf(x[0][r], x[1][r]);
+                rowpair_max4(mxs);
+                float alpha[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float m_new = fmaxf(m_run[r], mxs[r]);
+                    alpha[r] = (m_run[r] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run[r] - m_new);
+                    m_run[r] = m_new;
+                    pe[0][r] = x[0][r] - m_new;
+                    pe[1][r] = x[1][r] - m_new;
+                }
+                // accumulators hold column (x, head j % 8) in every register: the factor of that head is
+                // the lane's own when (j >> 2 & 1) == (kq & 1), else that of the neighbouring row
+                float al_own = (j & 3) == 0 ? alpha[0] : ((j & 3) == 1 ? alpha[1] : ((j & 3) == 2 ? alpha[2] : alpha[3]));
+                const float al_nb = lane_value(al_own, lane ^ 16);
+                const float al = (((j >> 2) & 1) == (kq & 1)) ? al_own : al_nb;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[0][i] *= al; acc[1][i] *= al; acc[2][i] *= al; acc[3][i] *= al; accz[i] *= al;
+                }
             }
-            // accumulators hold column (x, head j % 4) in every register
-            const float al = (j & 3) == 0 ? alpha[0] : ((j & 3) == 1 ? alpha[1] : ((j & 3) == 2 ? alpha[2] : alpha[3]));
+            {
+                uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT) + 4 * (kq & 1) * PT_ROW + tk;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { acc[0][i] *= al; acc[1][i] *= al; accz[i] *= al; }
-        }
-        {
-            const uint32_t p01 = pack_f16x2(__builtin_amdgcn_exp2f(pe[0]), __builtin_amdgcn_exp2f(pe[1]));
-            const uint32_t p23 = pack_f16x2(__builtin_amdgcn_exp2f(pe[2]), __builtin_amdgcn_exp2f(pe[3]));
-            uint16_t* pt = reinterpret_cast<uint16_t*>(sm + OFF_PT) + lane;
-            pt[0] = static_cast<uint16_t>(p01);
-            pt[PT_ROW] = static_cast<uint16_t>(p01 >> 16);
-            pt[2 * PT_ROW] = static_cast<uint16_t>(p23);
-            pt[3 * PT_ROW] = static_cast<uint16_t>(p23 >> 16);
+                for (int g = 0; g < 2; ++g) {
+                    const uint32_t p01 = pack_f16x2(__builtin_amdgcn_exp2f(pe[g][0]), __builtin_amdgcn_exp2f(pe[g][1]));
+                    const uint32_t p23 = pack_f16x2(__builtin_amdgcn_exp2f(pe[g][2]), __builtin_amdgcn_exp2f(pe[g][3]));
+                    pt[32 * g] = static_cast<uint16_t>(p01);
+                    pt[32 * g + PT_ROW] = static_cast<uint16_t>(p01 >> 16);
+                    pt[32 * g + 2 * PT_ROW] = static_cast<uint16_t>(p23);
+                    pt[32 * g + 3 * PT_ROW] = static_cast<uint16_t>(p23 >> 16);
+                }
+            }
         }
         lds_fence();
 
         // ------------------------------------------------------------------ P.V (transposed)
         // Lane addresses of this phase, formed here from the lane number rather than carried through
         // the QK phase, where registers are shortest (the copy below keeps them from being hoisted).
-        // Row i = j of the V operand is channel 16*(j & 7) + 8*(j >> 3) + Y; column j is (x = j >> 2, head j & 3).
+        // Row i = j of the V operand is channel 16*(j & 7) + 8*(j >> 3) + Y; column j is (x = j >> 2, head j & 3),
+        // or (x = j >> 3, head j & 7) with 8 heads.
         int lane_pv = lane;
         asm volatile("" : "+v"(lane_pv));
         const int jp = lane_pv & 15, kqp = lane_pv >> 4;
         const uint32_t vt_addr = OFF_VT + ((jp & 7) * VT_COL + 8 * kqp) * 4;
         const uint32_t vs_addr = OFF_VS + (((jp & 7) >> 1) * PT_ROW + 8 * kqp) * 2;
-        const uint32_t pt_addr = OFF_PT + ((jp & 3) * PT_ROW + 8 * kqp) * 2;
+        const uint32_t pt_addr = OFF_PT + ((jp & (NH - 1)) * PT_ROW + 8 * kqp) * 2;
         // rows of the sums operand: 0-3 V zero points, 4-7 V steps, 8 ones, others zero
         const uint32_t az_addr = jp < 8 ? OFF_VZ + (jp * PT_ROW + 8 * kqp) * 2 : (jp == 8 ? OFF_ONES : OFF_ZERO) + 16 * kqp;
         const uint32_t vsel = (jp & 8) ? 0x07060302u : 0x05040100u;
@@ -651,18 +774,32 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
             const uint32_t mg1 = __builtin_amdgcn_perm(va[3], va[2], vsel);
             const uint32_t mg2 = __builtin_amdgcn_perm(vb[1], vb[0], vsel);
             const uint32_t mg3 = __builtin_amdgcn_perm(vb[3], vb[2], vsel);
-            // column replica x takes the channel blocks Y with Y % 4 == x: for the others the weights are zeroed
-#define OMMX_PVX(X)                                                                                   \
-            {                                                                                         \
-                const bool mine = (jp >> 2) == X;                                                     \
-                const u32x4 bx = {mine ? pw[0] : 0u, mine ? pw[1] : 0u, mine ? pw[2] : 0u, mine ? pw[3] : 0u}; \
-                acc[0] = mfma_f16(u32x4{v_pair<X>(mg0, sw[0]), v_pair<X>(mg1, sw[1]),                 \
-                                        v_pair<X>(mg2, sw[2]), v_pair<X>(mg3, sw[3])}, bx, acc[0]);   \
-                acc[1] = mfma_f16(u32x4{v_pair<4 + X>(mg0, sw[0]), v_pair<4 + X>(mg1, sw[1]),         \
-                                        v_pair<4 + X>(mg2, sw[2]), v_pair<4 + X>(mg3, sw[3])}, bx, acc[1]); \
-            }
-            OMMX_PVX(0) OMMX_PVX(1) OMMX_PVX(2) OMMX_PVX(3)
+            if constexpr (NH == 4) {
+                // column replica x takes the channel blocks Y with Y % 4 == x: for the others the weights are zeroed
+#define OMMX_PVX(X)                                                                                       \
+                {                                                                                         \
+                    const bool mine = (jp >> 2) == X;                                                     \
+                    const u32x4 bx = {mine ? pw[0] : 0u, mine ? pw[1] : 0u, mine ? pw[2] : 0u, mine ? pw[3] : 0u}; \
+                    acc[0] = mfma_f16(u32x4{v_pair<X>(mg0, sw[0]), v_pair<X>(mg1, sw[1]),                 \
+                                            v_pair<X>(mg2, sw[2]), v_pair<X>(mg3, sw[3])}, bx, acc[0]);   \
+                    acc[1] = mfma_f16(u32x4{v_pair<4 + X>(mg0, sw[0]), v_pair<4 + X>(mg1, sw[1]),         \
+                                            v_pair<4 + X>(mg2, sw[2]), v_pair<4 + X>(mg3, sw[3])}, bx, acc[1]); \
+                }
+                OMMX_PVX(0) OMMX_PVX(1) OMMX_PVX(2) OMMX_PVX(3)
 #undef OMMX_PVX
+            } else {
+                // two column replicas: x takes the channel blocks Y with Y % 2 == x; blocks 2i and 2i + 1 share
+                // accumulator i
+                const bool first = (jp >> 3) == 0;
+                const u32x4 bx0 = {first ? pw[0] : 0u, first ? pw[1] : 0u, first ? pw[2] : 0u, first ? pw[3] : 0u};
+                const u32x4 bx1 = {first ? 0u : pw[0], first ? 0u : pw[1], first ? 0u : pw[2], first ? 0u : pw[3]};
+#define OMMX_PVY(Y)                                                                                       \
+                acc[(Y) >> 1] = mfma_f16(u32x4{v_pair<Y>(mg0, sw[0]), v_pair<Y>(mg1, sw[1]),              \
+                                               v_pair<Y>(mg2, sw[2]), v_pair<Y>(mg3, sw[3])},             \
+                                         ((Y) & 1) ? bx1 : bx0, acc[(Y) >> 1]);
+                OMMX_PVY(0) OMMX_PVY(1) OMMX_PVY(2) OMMX_PVY(3) OMMX_PVY(4) OMMX_PVY(5) OMMX_PVY(6) OMMX_PVY(7)
+#undef OMMX_PVY
+            }
         }
         lds_fence();
     }
@@ -676,7 +813,7 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
     const int je = lane_e & 15, kqe = lane_e >> 4;
-    const int h = je & 3, x = je >> 2;
+    const int h = je & (NH - 1), x = NH == 8 ? je >> 3 : je >> 2;
     const float l_tot = lane_value(accz[0], 32 + je);
     float z4[4], s4[4];
 #pragma unroll
@@ -688,21 +825,22 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
     if (h < heads) {
         float* dst = a.al + b * a.al_b + (int64_t)(qh0 + h) * a.al_h + (int64_t)sp * a.al_s;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2) {
+        for (int a2 = 0; a2 < NH / 2; ++a2) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                // row i = 4kq + r of block Y = 4*a2 + x: channel 16*(i & 7) + 8*(i >> 3) + Y, group (i & 7) / 2
-                const int cg_lo = 2 * (kqe & 1);
+                // row i = 4kq + r of block Y (4*a2 + x with 4 heads, 2*a2 + x with 8): channel
+                // 16*(i & 7) + 8*(i >> 3) + Y, group (i & 7) / 2
                 const float pz = (r >> 1) ? ((kqe & 1) ? z4[3] : z4[1]) : ((kqe & 1) ? z4[2] : z4[0]);
                 const float psum = (r >> 1) ? ((kqe & 1) ? s4[3] : s4[1]) : ((kqe & 1) ? s4[2] : s4[0]);
-                (void)cg_lo;
-                const int ch = 64 * (kqe & 1) + 16 * r + 8 * (kqe >> 1) + 4 * a2 + x;
+                const int ch = 64 * (kqe & 1) + 16 * r + 8 * (kqe >> 1) + (NH == 8 ? 2 : 4) * a2 + x;
                 const float f = (x & 1) ? 4.0f : 16.0f;
                 dst[ch] = (f * (acc[a2][r] - psum) + pz) * inv;
             }
         }
-        if (x == 0 && kqe == 0) {
-            const float mt = h == 0 ? m_run[0] : (h == 1 ? m_run[1] : (h == 2 ? m_run[2] : m_run[3]));
+        // the running maximum of head h: with 8 heads it lives in the rows with (kq & 1) == h >> 2
+        if (x == 0 && kqe == (NH == 8 ? (h >> 2) : 0)) {
+            const int hr = h & 3;
+            const float mt = hr == 0 ? m_run[0] : (hr == 1 ? m_run[1] : (hr == 2 ? m_run[2] : m_run[3]));
             dst[D] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
         }
     }
@@ -712,31 +850,35 @@ __global__ void __launch_bounds__(256, OMMX_GQA4_WAVES) decode_gqa4_kernel(Decod
 
 // Returns 0 when launched, 1 when the shape belongs to another kernel.
 int launch_decode_gqa4(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
-    if (Dh != 128 || !(R == 1 || R == 2 || R == 4)) return 1;
+    if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8)) return 1;
     if (a.kout != 6 || a.scale_bf16 || a.v_bf16 || a.gt != 32 || a.gc != 32) return 1;
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * LDS_WAVE;
+    const size_t shm = (size_t)waves * (R == 8 ? LdsMap<8>::LDS_WAVE : LdsMap<4>::LDS_WAVE);
     const bool own_map = a.k_ms != nullptr;
     const int order = a.B == 1 ? 0 : (a.B > 64 && a.B <= 256 ? 2 : 1);
-#define OMMX_GO(IDX, MAP, PART, ORD) \
-    hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD>), grid, block, shm, st, a)
-#define OMMX_GO_ORD(IDX, MAP, PART)                                  \
+#define OMMX_GO(IDX, MAP, PART, ORD, NH) \
+    hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD, NH>), grid, block, shm, st, a)
+#define OMMX_GO_ORD(IDX, MAP, PART, NH)                              \
     do {                                                             \
-        if (order == 0) OMMX_GO(IDX, MAP, PART, 0);                  \
-        else if (order == 2) OMMX_GO(IDX, MAP, PART, 2);             \
-        else OMMX_GO(IDX, MAP, PART, 1);                             \
+        if (order == 0) OMMX_GO(IDX, MAP, PART, 0, NH);              \
+        else if (order == 2) OMMX_GO(IDX, MAP, PART, 2, NH);         \
+        else OMMX_GO(IDX, MAP, PART, 1, NH);                         \
     } while (0)
-    switch ((R < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
-        case 0: OMMX_GO_ORD(0, false, false); break;
-        case 1: OMMX_GO_ORD(0, true, false); break;
-        case 2: OMMX_GO_ORD(1, false, false); break;
-        case 3: OMMX_GO_ORD(1, true, false); break;
-        case 4: OMMX_GO(0, false, true, 1); break;
-        case 5: OMMX_GO(0, true, true, 1); break;
-        case 6: OMMX_GO(1, false, true, 1); break;
-        default: OMMX_GO(1, true, true, 1); break;
+    switch ((R == 8 ? 8 : 0) | (R < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
+        case 0: OMMX_GO_ORD(0, false, false, 4); break;
+        case 1: OMMX_GO_ORD(0, true, false, 4); break;
+        case 2: OMMX_GO_ORD(1, false, false, 4); break;
+        case 3: OMMX_GO_ORD(1, true, false, 4); break;
+        case 4: OMMX_GO(0, false, true, 1, 4); break;
+        case 5: OMMX_GO(0, true, true, 1, 4); break;
+        case 6: OMMX_GO(1, false, true, 1, 4); break;
+        case 7: OMMX_GO(1, true, true, 1, 4); break;
+        case 8: OMMX_GO_ORD(0, false, false, 8); break;
+        case 9: OMMX_GO_ORD(0, true, false, 8); break;
+        case 10: OMMX_GO_ORD(1, false, false, 8); break;
+        default: OMMX_GO_ORD(1, true, false, 8); break;
     }
 #undef OMMX_GO
 #undef OMMX_GO_ORD

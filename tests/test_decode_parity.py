@@ -414,6 +414,39 @@ def test_logit_cap_and_caller_workspace():
     assert (o[0].double() - want).abs().max().item() <= MAX_ABS
 
 
+def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
+    """The serving-recipe kernel laid out for 8 q heads per kv head (a lane keeps four heads of one
+    token of either group): lengths that end inside the first / second group of a 64-token step,
+    more splits than groups, one kv head alone in its workgroup, and capped logits."""
+    case = build_decode_case([2048, 700], q_heads=16, kv_heads=2, seed=17, permute_tables=True, sparse_frac=0.01,
+                             sparse_gain=40.0)
+    full = case.b_seq_len.clone()
+    for cut in ((1, 31), (33, 64), (65, 97), (1000, 2), (1971, 640)):
+        case.b_seq_len.copy_(torch.tensor(cut, dtype=torch.int32))
+        case.extra["packed_lens"] = list(cut)
+        want = _oracle(case)
+        for S in (1, 3, 40):
+            _check(_run(case, num_kv_splits=S), want, f"cut {cut} S{S}")
+    case.b_seq_len.copy_(full)
+    case.extra["packed_lens"] = full.tolist()
+    one = build_decode_case([900], q_heads=8, kv_heads=1, seed=18, sparse_frac=0.005)
+    _check(_run(one, num_kv_splits=5), _oracle(one), "one kv head")
+    cap = 5.0
+    planes = _cpu_planes(case)
+    o, _ = _run(case, num_kv_splits=7, logit_cap=cap)
+    for b in range(2):
+        Kd, Vd = O.gather_request(planes, case.req_to_token[b].cpu(), case.req_to_group[b].cpu(),
+                                  case.b_seq_len.tolist()[b], page_size=16)
+        tl = case.b_tail_len.tolist()[b]
+        Kf = torch.cat([Kd, case.k_tail[b, :tl].cpu().float()]).double()
+        Vf = torch.cat([Vd, case.v_tail[b, :tl].cpu().float()]).double()
+        want = torch.zeros(16, 128, dtype=torch.float64)
+        for h in range(16):
+            s_ = (Kf[:, h // 8] @ case.q[b, h].cpu().double()) * case.sm_scale
+            want[h] = torch.softmax(cap * torch.tanh(s_ / cap), 0) @ Vf[:, h // 8]
+        assert (o[b].double() - want).abs().max().item() <= MAX_ABS, f"cap, request {b}"
+
+
 @pytest.mark.parametrize("gt,kw", [(32, {}), (64, dict(group_tokens=64, group_channels=64, outlier_repr="relidx7")),
                                    (128, dict(group_tokens=128, group_channels=128, outlier_repr="relidx7",
                                               outliers_per_vector=10)),
