@@ -76,7 +76,7 @@ struct LdsMap {
     static constexpr int OFF_LC = OFF_STAGE_END;               // [32 tokens][NH heads] f32 logit corrections of one group
     static constexpr int OFF_ZERO = OFF_LC + 32 * NH * 4;      // 128 B of zeros, never written again
     static constexpr int OFF_ONES = OFF_ZERO + 128;            // 128 B of f16 1.0, never written again
-    static constexpr int LDS_WAVE = OFF_ONES + 128;            // 13568 (4 heads) / 14656 (8 heads)
+    static constexpr int LDS_WAVE = OFF_ONES + 128;            // 13376 (4 heads) / 14464 (8 heads)
     static_assert(OFF_KT % 16 == 0 && OFF_PT % 16 == 0 && OFF_VZ % 16 == 0 && OFF_LC % 16 == 0, "b128 alignment");
 };
 static_assert(3 * 4 * LdsMap<4>::LDS_WAVE <= 160 * 1024, "4 heads: three workgroups per compute unit");
