@@ -26,6 +26,9 @@ struct DecodeArgs {
     // OR-ed into *err (may be NULL).  0 = extent not given: ids are used as they are.
     int n_pages, n_gslots;
     int32_t* err;
+    // set by the launcher of the serving-recipe kernel only: head_dim is 64 and Hkv counts PAIRS of kv
+    // heads (the planes of two neighbouring 64-channel heads read like one 128-channel head)
+    int half;
 };
 
 // 7-bit position streams (pack.py:128-164): position s of a frame at bits [7s, 7s+7)

@@ -1,6 +1,7 @@
 // Split-KV decode kernel for gfx950, serving shape: head_dim 128, 1, 2, 4 or 8 q heads per kv head,
 // 6 outliers per K vector of 32 tokens (either index plane, either outlier map), INT2 V with
-// 32-channel vectors, int8 exponents.  Same operator as
+// 32-channel vectors, int8 exponents; in a general form (GEN) also 1..8 outliers on the bitmap
+// plane and head_dim 64 with 1, 2 or 4 q heads per kv head.  Same operator as
 // ommx_gpu_serve/attention/paged_decode.py:1255-2284; the other shapes of the matrix-core path
 // (longer groups, no outliers) stay on the kernel in ommx_decode.hip.
 //
@@ -116,9 +117,17 @@ __device__ __forceinline__ uint32_t pk_u16(uint32_t lo, uint32_t hi) { return (l
 // the last head and are not written).  ORDER: 0 one request, 1 up to 64 requests served longest
 // first, 2 up to 256 (radix select); see ommx_decode.hip.
 // NH: q heads per kv head the matrix rows and columns are laid out for, 4 or 8.
-template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER, int NH = 4>
-__global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
+// GEN: the general form of the recipe: 1..8 outliers per vector (a.kout, bitmap plane only), and
+// head_dim 64 (a.half): the planes of two neighbouring 64-channel kv heads read exactly like one
+// 128-channel head, so a wave takes the pair as one head whose q heads are those of both, each
+// zero on the other one's channels, and writes each q head only its own half of the output.
+template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER, int NH = 4, bool GEN = false>
+__global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
     static_assert(NH == 4 || (NH == 8 && !PARTIAL), "4 heads (or fewer, PARTIAL) or exactly 8");
+    static_assert(!GEN || IDX == 0, "the general form reads bitmaps");
+    constexpr int KMAX = GEN ? 8 : 6;                 // outliers per vector, upper bound
+    const int kout = GEN ? a.kout : 6;
+    const bool half = GEN && a.half;
     using Lds = LdsMap<NH>;
     constexpr int OFF_VZ = Lds::OFF_VZ, OFF_VS = Lds::OFF_VS, OFF_LC = Lds::OFF_LC, OFF_ZERO = Lds::OFF_ZERO,
                   OFF_ONES = Lds::OFF_ONES, LDS_WAVE = Lds::LDS_WAVE;
@@ -134,6 +143,8 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
     const int kvh = blockIdx.y * waves + wave;
     const int heads = PARTIAL ? a.Hq / Hkv : NH;
     const int qh0 = kvh * heads;
+    const int r_half = max(heads >> 1, 1);            // head_dim 64: q heads per kv head of the pair
+    const int Dout = half ? 64 : D;                   // channels of an output state
     const int sp = blockIdx.x;
     int b = blockIdx.z, L;
     if (ORDER >= 1 && a.B > 1 && a.B <= 64) {
@@ -172,14 +183,20 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
     // and channels 2*lane, 2*lane+1 of every head (for the channel pass)
     uint32_t qw[16], qraw[NH];      // qraw: channels 2*lane, 2*lane+1 of every head, for the thresholds below
     {
+        const int slot = min(j & (NH - 1), heads - 1);
+        // head_dim 64: the head's 64 channels are the pair's channels 64 * (slot / r_half) .. + 63
+        const bool q_real = !half || (kq >> 1) == slot / r_half;
         const uint32_t* qh = reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + min(j & (NH - 1), heads - 1)) * a.q_sh + 32 * kq);
+            a.q + b * a.q_sb + (int64_t)(qh0 + slot) * a.q_sh + (half ? 32 * (kq & 1) : 32 * kq));
 #pragma unroll
-        for (int i = 0; i < 16; ++i) qw[i] = qh[i];
+        for (int i = 0; i < 16; ++i) qw[i] = q_real ? qh[i] : 0u;
 #pragma unroll
-        for (int r = 0; r < NH; ++r)
-            qraw[r] = *reinterpret_cast<const uint32_t*>(
-                a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
+        for (int r = 0; r < NH; ++r) {
+            const int sl = min(r, heads - 1);
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(
+                a.q + b * a.q_sb + (int64_t)(qh0 + sl) * a.q_sh + (half ? (2 * lane) & 63 : 2 * lane));
+            qraw[r] = (!half || (lane >> 5) == sl / r_half) ? w : 0u;
+        }
     }
     // The 32-token groups are dealt out evenly: every split takes G/S groups and the first G%S
     // splits one more, so no two splits differ by more than one group and none is empty while
@@ -197,8 +214,8 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
         for (int r = 0; r < heads; ++r) {
             float* dst = a.al + b * a.al_b + (int64_t)(qh0 + r) * a.al_h + (int64_t)sp * a.al_s;
             dst[lane] = 0.0f;
-            dst[64 + lane] = 0.0f;
-            if (lane == 0) dst[D] = -INFINITY;
+            if (!half) dst[64 + lane] = 0.0f;
+            if (lane == 0) dst[Dout] = -INFINITY;
         }
         return;
     }
@@ -272,8 +289,16 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
             g_bm[g] = u32x2{ixp[0], ixp[1]};
             g_bx[g] = ixp[2];
         }
-        const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
-        g_ov[g] = u32x2{ovp[0], ovp[1]};
+        if constexpr (!GEN) {
+            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
+            g_ov[g] = u32x2{ovp[0], ovp[1]};
+        } else {
+            // (kout + 1) / 2 bytes per channel, two channels per lane: the dword(s) that hold them
+            const uint32_t kb = static_cast<uint32_t>(kout + 1) >> 1;
+            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * kb, (2 * kb * lane_b) & ~3u));
+            g_ov[g][0] = ovp[0];
+            g_ov[g][1] = kb > 2 ? ovp[1] : 0u;       // 1 or 2 bytes per channel: one dword holds the pair
+        }
     };
     // The page and group ids of the first step are asked for here; what follows (clearing LDS, the
     // A operands, the lane constants) needs none of it and runs while they are on their way.
@@ -325,8 +350,10 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
 #else
     // q of head r, channel 2*lane + u: read again where it is needed (the residual walk, seldom taken)
     auto q_of = [&](int u, int r) {
-        const uint32_t w = *reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + min(r, heads - 1)) * a.q_sh + 2 * lane);
+        const int sl = min(r, heads - 1);
+        uint32_t w = *reinterpret_cast<const uint32_t*>(
+            a.q + b * a.q_sb + (int64_t)(qh0 + sl) * a.q_sh + (half ? (2 * lane) & 63 : 2 * lane));
+        if (half && (lane >> 5) != sl / r_half) w = 0u;
         return __uint_as_float(u ? (w & 0xFFFF0000u) : (w << 16));
     };
 #endif
@@ -351,7 +378,8 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
     }
     const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
     const uint32_t code_sh = 2u * (c0 & 3u);                      // bit of channel c0's code in that byte; c0 + 1 sits two on
-    const uint32_t nib_sh = 8u * ((6u * lane) & 3u);
+    const uint32_t kbytes = static_cast<uint32_t>(kout + 1) >> 1;            // nibble bytes per channel
+    const uint32_t nib_sh = 8u * ((2u * kbytes * lane) & 3u);
     const float c2 = a.sm_scale * 1.4426950408889634f;
 
     // in the order the first step needs them: K rows, the group parameters, then V
@@ -442,11 +470,13 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
                     ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
                 }
                 const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
-                const uint32_t nib = static_cast<uint32_t>(ov64 >> (nib_sh + 24 * u)) & 0xFFFFFFu;
+                const uint32_t nib = GEN ? static_cast<uint32_t>(ov64 >> (nib_sh + 8 * kbytes * u))
+                                         : static_cast<uint32_t>(ov64 >> (nib_sh + 24 * u)) & 0xFFFFFFu;
                 const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
                 const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
                 const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
-                const float lv[6] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1]};
+                const f32x2 l67 = GEN ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 3) : f32x2{0.0f, 0.0f};
+                const float lv[8] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1], l67[0], l67[1]};
                 // The base MFMA takes every position of the K rows as it is stored; the tile entry of an
                 // outlier is what is missing on top of its stored 2-bit code, which the lane looks up
                 // in the staged K rows (a byte read per outlier; the packer's code of an outlier is the
@@ -454,13 +484,14 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
                 const uint8_t* kt = sm + kt_lane + g * 32 * KT_ROW;
                 float* lc = reinterpret_cast<float*>(sm + OFF_LC);
                 uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_TILE) + hw0 + 2 * u;      // pair order, like MAG
-                int pos[6];
-                uint32_t cb[6];
+                int pos[KMAX];
+                uint32_t cb[KMAX];
 #pragma unroll
-                for (int sidx = 0; sidx < 6; ++sidx) {
+                for (int sidx = 0; sidx < KMAX; ++sidx) {
+                    if (GEN && sidx >= kout) break;
                     if constexpr (IDX == 0) {
                         pos[sidx] = __builtin_ctz(bm) & 31;
-                        if (sidx < 5) bm &= bm - 1;
+                        if (sidx < KMAX - 1) bm &= bm - 1;
                     } else {
                         pos[sidx] = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
                                   : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
@@ -469,7 +500,8 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
                     cb[sidx] = kt[pos[sidx] * KT_ROW];
                 }
 #pragma unroll
-                for (int sidx = 0; sidx < 6; ++sidx) {
+                for (int sidx = 0; sidx < KMAX; ++sidx) {
+                    if (GEN && sidx >= kout) break;
                     const float dl0 = fmaf(lv[sidx], a1, b1);
                     const float code = static_cast<float>((cb[sidx] >> (code_sh + 2 * u)) & 3u);
                     const float dl = fmaf(-code, sc, dl0);
@@ -834,14 +866,16 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
                 const float psum = (r >> 1) ? ((kqe & 1) ? s4[3] : s4[1]) : ((kqe & 1) ? s4[2] : s4[0]);
                 const int ch = 64 * (kqe & 1) + 16 * r + 8 * (kqe >> 1) + (NH == 8 ? 2 : 4) * a2 + x;
                 const float f = (x & 1) ? 4.0f : 16.0f;
-                dst[ch] = (f * (acc[a2][r] - psum) + pz) * inv;
+                const float val = (f * (acc[a2][r] - psum) + pz) * inv;
+                if (!half) dst[ch] = val;
+                else if ((kqe & 1) == h / r_half) dst[ch & 63] = val;     // the head's own 64 channels
             }
         }
         // the running maximum of head h: with 8 heads it lives in the rows with (kq & 1) == h >> 2
         if (x == 0 && kqe == (NH == 8 ? (h >> 2) : 0)) {
             const int hr = h & 3;
             const float mt = hr == 0 ? m_run[0] : (hr == 1 ? m_run[1] : (hr == 2 ? m_run[2] : m_run[3]));
-            dst[D] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
+            dst[Dout] = l_tot > 0.0f ? (mt + log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
         }
     }
 }
@@ -849,32 +883,51 @@ __global__ void __launch_bounds__(256, NH == 8 ? 2 : OMMX_GQA4_WAVES) decode_gqa
 }  // namespace
 
 // Returns 0 when launched, 1 when the shape belongs to another kernel.
-int launch_decode_gqa4(const DecodeArgs& a, int Dh, int R, hipStream_t st) {
-    if (Dh != 128 || !(R == 1 || R == 2 || R == 4 || R == 8)) return 1;
-    if (a.kout != 6 || a.scale_bf16 || a.v_bf16 || a.gt != 32 || a.gc != 32) return 1;
+int launch_decode_gqa4(const DecodeArgs& a_in, int Dh, int R, hipStream_t st) {
+    DecodeArgs a = a_in;
+    a.half = 0;
+    if (a.scale_bf16 || a.v_bf16 || a.gt != 32 || a.gc != 32 || a.kout < 1 || a.kout > 8) return 1;
     if ((reinterpret_cast<uintptr_t>(a.q) & 3) || (a.q_sb & 1) || (a.q_sh & 1)) return 1;
+    int nh;                                   // q heads of a wave's (pair of) kv head(s)
+    if (Dh == 128 && (R == 1 || R == 2 || R == 4 || R == 8)) {
+        nh = R;
+    } else if (Dh == 64 && (R == 1 || R == 2 || R == 4) && a.Hkv % 2 == 0) {
+        a.half = 1;                           // two 64-channel kv heads read as one 128-channel head
+        a.Hkv /= 2;
+        nh = 2 * R;
+    } else {
+        return 1;
+    }
+    const bool general = a.half || a.kout != 6;
+    if (general && a.idx_repr != 0) return 1;       // the general form reads bitmaps only
     const int waves = (a.Hkv % 4 == 0) ? 4 : ((a.Hkv % 2 == 0) ? 2 : 1);
     const dim3 grid(a.S, a.Hkv / waves, a.B), block(64 * waves);
-    const size_t shm = (size_t)waves * (R == 8 ? LdsMap<8>::LDS_WAVE : LdsMap<4>::LDS_WAVE);
+    const size_t shm = (size_t)waves * (nh == 8 ? LdsMap<8>::LDS_WAVE : LdsMap<4>::LDS_WAVE);
     const bool own_map = a.k_ms != nullptr;
     const int order = a.B == 1 ? 0 : (a.B > 64 && a.B <= 256 ? 2 : 1);
-#define OMMX_GO(IDX, MAP, PART, ORD, NH) \
-    hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD, NH>), grid, block, shm, st, a)
+#define OMMX_GO(IDX, MAP, PART, ORD, NH, GEN) \
+    hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD, NH, GEN>), grid, block, shm, st, a)
 #define OMMX_GO_ORD(IDX, MAP, PART, NH)                              \
     do {                                                             \
-        if (order == 0) OMMX_GO(IDX, MAP, PART, 0, NH);              \
-        else if (order == 2) OMMX_GO(IDX, MAP, PART, 2, NH);         \
-        else OMMX_GO(IDX, MAP, PART, 1, NH);                         \
+        if (order == 0) OMMX_GO(IDX, MAP, PART, 0, NH, false);       \
+        else if (order == 2) OMMX_GO(IDX, MAP, PART, 2, NH, false);  \
+        else OMMX_GO(IDX, MAP, PART, 1, NH, false);                  \
     } while (0)
-    switch ((R == 8 ? 8 : 0) | (R < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
+    if (general) {
+        // one instantiation per (outlier map, head layout): outlier count, head count and head_dim at run time
+        if (nh == 8) { if (own_map) OMMX_GO(0, true, false, 2, 8, true); else OMMX_GO(0, false, false, 2, 8, true); }
+        else { if (own_map) OMMX_GO(0, true, true, 2, 4, true); else OMMX_GO(0, false, true, 2, 4, true); }
+        return 0;
+    }
+    switch ((nh == 8 ? 8 : 0) | (nh < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
         case 0: OMMX_GO_ORD(0, false, false, 4); break;
         case 1: OMMX_GO_ORD(0, true, false, 4); break;
         case 2: OMMX_GO_ORD(1, false, false, 4); break;
         case 3: OMMX_GO_ORD(1, true, false, 4); break;
-        case 4: OMMX_GO(0, false, true, 1, 4); break;
-        case 5: OMMX_GO(0, true, true, 1, 4); break;
-        case 6: OMMX_GO(1, false, true, 1, 4); break;
-        case 7: OMMX_GO(1, true, true, 1, 4); break;
+        case 4: OMMX_GO(0, false, true, 1, 4, false); break;
+        case 5: OMMX_GO(0, true, true, 1, 4, false); break;
+        case 6: OMMX_GO(1, false, true, 1, 4, false); break;
+        case 7: OMMX_GO(1, true, true, 1, 4, false); break;
         case 8: OMMX_GO_ORD(0, false, false, 8); break;
         case 9: OMMX_GO_ORD(0, true, false, 8); break;
         case 10: OMMX_GO_ORD(1, false, false, 8); break;

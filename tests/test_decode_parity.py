@@ -414,6 +414,48 @@ def test_logit_cap_and_caller_workspace():
     assert (o[0].double() - want).abs().max().item() <= MAX_ABS
 
 
+@pytest.mark.parametrize("D,hq,hkv", [(128, 32, 8), (128, 16, 2), (128, 2, 2), (64, 4, 2), (64, 16, 4), (64, 4, 4),
+                                      (64, 8, 8)])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 7, 8])
+def test_other_outlier_counts_and_head_dim_64_on_the_matrix_core_kernel(D, hq, hkv, k):
+    """1..8 outliers per vector (bitmap plane) and head_dim 64 run on the serving-recipe kernel's general
+    form: against the oracle and against the plain kernel, ragged lengths cut inside a group, permuted
+    tables, several split counts, both outlier maps."""
+    for own_map in (True, False):
+        case = build_decode_case([1700, 90, 600], q_heads=hq, kv_heads=hkv, head_dim=D, seed=700 + 10 * k + D,
+                                 permute_tables=True, sparse_frac=0.005,
+                                 outliers_per_vector=k, kv_outlier_map=own_map)
+        cut = torch.tensor([1700 - 13, 90, 600 - 31], dtype=torch.int32)
+        cut = torch.minimum(cut, case.b_seq_len.cpu()).to(case.b_seq_len.device)
+        case.b_seq_len.copy_(cut)
+        case.extra["packed_lens"] = cut.tolist()
+        want = _oracle(case)
+        ref = _run(case, num_kv_splits=4, ref_kernel=True)
+        for S in (None, 1, 5):
+            got = _run(case, num_kv_splits=S)
+            _check(got, want, f"D{D} {hq}/{hkv} k{k} map{own_map} S{S}")
+            assert (got[0] - ref[0]).abs().max().item() <= MAX_ABS
+
+
+def test_head_dim_64_serving_recipe_with_cap_and_int64_tables():
+    case = build_decode_case([2100, 333], q_heads=8, kv_heads=2, head_dim=64, seed=77, permute_tables=True,
+                             sparse_frac=0.005, table_dtype=torch.int64)
+    _check(_run(case, num_kv_splits=6), _oracle(case), "d64 k6")
+    cap = 4.0
+    planes = _cpu_planes(case)
+    o, _ = _run(case, num_kv_splits=3, logit_cap=cap)
+    for b in range(2):
+        Kd, Vd = O.gather_request(planes, case.req_to_token[b].cpu(), case.req_to_group[b].cpu(),
+                                  case.b_seq_len.tolist()[b], page_size=16)
+        tl = case.b_tail_len.tolist()[b]
+        Kf = torch.cat([Kd, case.k_tail[b, :tl].cpu().float()]).double()
+        Vf = torch.cat([Vd, case.v_tail[b, :tl].cpu().float()]).double()
+        for h in range(8):
+            s_ = (Kf[:, h // 4] @ case.q[b, h].cpu().double()) * case.sm_scale
+            want = torch.softmax(cap * torch.tanh(s_ / cap), 0) @ Vf[:, h // 4]
+            assert (o[b, h].double() - want).abs().max().item() <= MAX_ABS, f"cap, request {b} head {h}"
+
+
 def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
     """The serving-recipe kernel laid out for 8 q heads per kv head (a lane keeps four heads of one
     token of either group): lengths that end inside the first / second group of a 64-token step,
