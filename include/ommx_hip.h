@@ -212,7 +212,9 @@ int ommx_decode_splitkv_ref(const uint16_t* q, int64_t q_stride_b, int64_t q_str
  * num_splits <= 512.  tail_rows = Tmax, the rows every request's tail buffer holds (0 when
  * unknown): the kernel asks for the first min(64, tail_rows) rows before b_tail_len has
  * arrived, which takes one memory round trip off its critical path; rows past a request's
- * b_tail_len are read but never used, so they only have to be addressable.
+ * b_tail_len are read but never used, so they only have to be addressable.  With tail_rows
+ * given, a b_tail_len above it counts as tail_rows and a negative one as 0: no row address
+ * leaves the buffers whatever the length tensor holds.
  */
 int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t al_stride_h,
                         int64_t al_stride_s,

@@ -66,7 +66,11 @@ __global__ void __launch_bounds__(NT) combine_kernel(CombineArgs a) {
     const float* base = a.al + b * a.al_b + (int64_t)h * a.al_h;
     // the two scalars that everything after the split loads waits for: requested first
     const int L = a.seq[b];
-    const int tail = a.tail ? a.tail[b] : 0;
+    // a length outside the tail buffer (when the caller has said how many rows it holds) is held
+    // inside it, so that no row address leaves the buffer whatever b_tail_len contains
+    int tail = a.tail ? a.tail[b] : 0;
+    tail = max(tail, 0);
+    if (a.T > 0) tail = min(tail, a.T);
 
     // ---- all loads of the split part --------------------------------------------------
     // They depend on the arguments only, so they go out before anything is read from
@@ -242,7 +246,11 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
     const int h0 = kvh * R;
     const float* base = a.al + b * a.al_b + (int64_t)h0 * a.al_h;
     const int L = a.seq[b];
-    const int tail = a.tail ? a.tail[b] : 0;
+    // a length outside the tail buffer (when the caller has said how many rows it holds) is held
+    // inside it, so that no row address leaves the buffer whatever b_tail_len contains
+    int tail = a.tail ? a.tail[b] : 0;
+    tail = max(tail, 0);
+    if (a.T > 0) tail = min(tail, a.T);
 
     // ---- split weights: wave r, lane s ----------------------------------------------------
     if (a.q) {

@@ -456,6 +456,24 @@ def test_head_dim_64_serving_recipe_with_cap_and_int64_tables():
             assert (o[b, h].double() - want).abs().max().item() <= MAX_ABS, f"cap, request {b} head {h}"
 
 
+@pytest.mark.parametrize("B", [2, 70])
+def test_tail_length_outside_the_buffer_is_held_inside_it(B):
+    """b_tail_len is a device tensor nobody checks on the host: with the buffer's row count known to the
+    combine (tail_rows), a length above it reads as the row count and a negative one as 0, in the kernel
+    with one workgroup per q head and in the one with one per kv head (70 requests of 8 kv heads)."""
+    case = build_decode_case([200] * B, q_heads=32, kv_heads=8, seed=19)
+    T = int(case.k_tail.shape[1])
+    good = case.b_tail_len.clone()
+    case.b_tail_len.fill_(T)
+    case.b_tail_len[1] = 0
+    want = _run(case, num_kv_splits=3)
+    case.b_tail_len.fill_(T + 100000)
+    case.b_tail_len[1] = -7
+    got = _run(case, num_kv_splits=3)
+    case.b_tail_len.copy_(good)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
 def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
     """The serving-recipe kernel laid out for 8 q heads per kv head (a lane keeps four heads of one
     token of either group): lengths that end inside the first / second group of a 64-token step,
