@@ -228,7 +228,10 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 // head) and there are at most 64 splits.  Wave r < R owns the scalars of head r (split weights, running tail maximum
 // and sum); the channel work is dealt out as (head, channel) for the splits and as (channel
 // pair, row group) for the tail's P.V.
-template <int D, int R>
+// EARLY: the tail rows of the first pass are asked for before the split part and held in registers
+// (32 more: one workgroup per compute unit instead of two, which pays while the grid is no larger
+// than the chip).
+template <int D, int R, bool EARLY>
 __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
     constexpr int NT = 512, MAXS = 64;
     constexpr int ROWS = 128;              // tail rows per pass (two per thread of the logit layout)
@@ -275,6 +278,40 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
     }
     __syncthreads();
 
+    // ---- the tail rows of the first pass are asked for here, before the split part waits for its
+    // own loads: thread (row, part) holds CHP channels of K rows row and row + 64, thread (channel
+    // pair, row group) the V dwords of rows rg, rg + NRG, ...
+    constexpr int VPT = ROWS / NRG;        // V rows per thread and pass
+    const int dp = tid % (D / 2), rg = tid / (D / 2);
+    uint4 kk[2][CHP / 8];
+    uint32_t vv[VPT];
+    auto ask_rows = [&](int r0, int nr) {
+        const int part = tid & 7, row = tid >> 3;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            const int t = row + 64 * h2;
+#pragma unroll
+            for (int c8 = 0; c8 < CHP / 8; ++c8) kk[h2][c8] = uint4{0u, 0u, 0u, 0u};
+            if (t < nr) {
+                const uint16_t* kp = a.kt + b * a.kt_b + (int64_t)(r0 + t) * a.kt_t +
+                                     (int64_t)kvh * a.kt_h + part * CHP;
+#pragma unroll
+                for (int c8 = 0; c8 < CHP / 8; ++c8) kk[h2][c8] = reinterpret_cast<const uint4*>(kp)[c8];
+            }
+        }
+        if constexpr (EARLY) {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int t = rg + NRG * i;
+                vv[i] = 0u;
+                if (t < nr)
+                    vv[i] = *reinterpret_cast<const uint32_t*>(
+                        a.vt + b * a.vt_b + (int64_t)(r0 + t) * a.vt_t + (int64_t)kvh * a.vt_h + 2 * dp);
+            }
+        }
+    };
+    if constexpr (EARLY) ask_rows(0, min(ROWS, tail));
+
     // ---- split part: item (head, channel) ---------------------------------------------------
     // Every split slot is read (it exists; an absent split's content is stale and is dropped by
     // the select), so that the loads carry no branch and go out eight at a time.
@@ -306,9 +343,9 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
     float acc[R][2];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r][0] = acc[r][1] = 0.0f;
-    const int dp = tid % (D / 2), rg = tid / (D / 2);
     for (int r0 = 0; r0 < tail; r0 += ROWS) {
         const int nr = min(ROWS, tail - r0);
+        if (!EARLY || r0 > 0) ask_rows(r0, nr);
         {   // logits: thread (row, part) takes CHP channels of rows row and row + 64
             const int part = tid & 7, row = tid >> 3;
 #pragma unroll
@@ -318,11 +355,9 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) dot[r] = 0.0f;
                 if (t < nr) {
-                    const uint16_t* kp = a.kt + b * a.kt_b + (int64_t)(r0 + t) * a.kt_t +
-                                         (int64_t)kvh * a.kt_h + part * CHP;
 #pragma unroll
                     for (int c8 = 0; c8 < CHP / 8; ++c8) {
-                        const uint4 ku = reinterpret_cast<const uint4*>(kp)[c8];
+                        const uint4 ku = kk[rr / 64][c8];
                         const uint32_t w[4] = {ku.x, ku.y, ku.z, ku.w};
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
@@ -368,15 +403,31 @@ __global__ void __launch_bounds__(512) combine_grouped_kernel(CombineArgs a) {
                 acc[r][0] *= al;
                 acc[r][1] *= al;
             }
-            for (int t = rg; t < nr; t += NRG) {
-                const uint32_t vv = *reinterpret_cast<const uint32_t*>(
-                    a.vt + b * a.vt_b + (int64_t)(r0 + t) * a.vt_t + (int64_t)kvh * a.vt_h + 2 * dp);
-                const float v0 = __uint_as_float(vv << 16), v1 = __uint_as_float(vv & 0xFFFF0000u);
+            if constexpr (EARLY) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const float p = s_p[r][t];
-                    acc[r][0] = fmaf(p, v0, acc[r][0]);
-                    acc[r][1] = fmaf(p, v1, acc[r][1]);
+                for (int i = 0; i < VPT; ++i) {
+                    const int t = rg + NRG * i;
+                    if (t < nr) {
+                        const float v0 = __uint_as_float(vv[i] << 16), v1 = __uint_as_float(vv[i] & 0xFFFF0000u);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const float p = s_p[r][t];
+                            acc[r][0] = fmaf(p, v0, acc[r][0]);
+                            acc[r][1] = fmaf(p, v1, acc[r][1]);
+                        }
+                    }
+                }
+            } else {
+                for (int t = rg; t < nr; t += NRG) {
+                    const uint32_t vw = *reinterpret_cast<const uint32_t*>(
+                        a.vt + b * a.vt_b + (int64_t)(r0 + t) * a.vt_t + (int64_t)kvh * a.vt_h + 2 * dp);
+                    const float v0 = __uint_as_float(vw << 16), v1 = __uint_as_float(vw & 0xFFFF0000u);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        const float p = s_p[r][t];
+                        acc[r][0] = fmaf(p, v0, acc[r][0]);
+                        acc[r][1] = fmaf(p, v1, acc[r][1]);
+                    }
                 }
             }
         }
@@ -428,15 +479,23 @@ int launch_combine(const CombineArgs& a, int D, hipStream_t st) {
     const dim3 grid(a.B, a.Hq, split2 ? 2 : 1);
     const bool small = !split2 && a.S <= 64;
     const int R = a.Hq / a.Hkv;
-    // a whole kv head per workgroup once those alone are two per compute unit (128 requests of 8
-    // kv heads: 29 against 47 us; with fewer, one workgroup per q head spreads the work better)
-    if (small && (R == 4 || R == 8) && a.Hq == R * a.Hkv && a.B * a.Hkv >= 512) {
+    // a whole kv head per workgroup once those alone are one per compute unit (32 requests of 8 kv
+    // heads: 10 against 16 us; 128 requests: 25 against 47 us; with fewer, one workgroup per q head
+    // spreads the work better: 16 requests 9.8 against 13 us)
+    if (small && (R == 4 || R == 8) && a.Hq == R * a.Hkv && a.B * a.Hkv >= 256) {
         const dim3 g2(a.B, a.Hkv);
-        if (D == 128 && R == 4) hipLaunchKernelGGL((combine_grouped_kernel<128, 4>), g2, dim3(512), 0, st, a);
-        else if (D == 128) hipLaunchKernelGGL((combine_grouped_kernel<128, 8>), g2, dim3(512), 0, st, a);
-        else if (D == 64 && R == 4) hipLaunchKernelGGL((combine_grouped_kernel<64, 4>), g2, dim3(512), 0, st, a);
-        else if (D == 64) hipLaunchKernelGGL((combine_grouped_kernel<64, 8>), g2, dim3(512), 0, st, a);
+        const bool early = a.B * a.Hkv <= 320;       // about one workgroup per compute unit
+#define OMMX_GROUPED(DD, RR)                                                                              \
+        do {                                                                                              \
+            if (early) hipLaunchKernelGGL((combine_grouped_kernel<DD, RR, true>), g2, dim3(512), 0, st, a);  \
+            else hipLaunchKernelGGL((combine_grouped_kernel<DD, RR, false>), g2, dim3(512), 0, st, a);       \
+        } while (0)
+        if (D == 128 && R == 4) OMMX_GROUPED(128, 4);
+        else if (D == 128) OMMX_GROUPED(128, 8);
+        else if (D == 64 && R == 4) OMMX_GROUPED(64, 4);
+        else if (D == 64) OMMX_GROUPED(64, 8);
         else return -1;
+#undef OMMX_GROUPED
         return 0;
     }
     if (a.S > 256) {        // 257..512 splits: the same kernel with twice the split slots per thread
