@@ -135,15 +135,16 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 o (normalised) in [0,D) and lse at D; an empty split writes o=0,
  *                 lse=-inf (paged_decode.py:2262-2284)
  * How the tokens are dealt out to the splits is the kernel's own business (the reference rounds
- * ceil(L/S) up to whole groups, paged_decode.py:1429-1432; the kernel for up to 4 q heads per kv
- * head deals whole groups out evenly): every split writes its state, an empty one o = 0 and
+ * ceil(L/S) up to whole groups, paged_decode.py:1429-1432; the serving-recipe kernel deals whole
+ * groups out evenly): every split writes its state, an empty one o = 0 and
  * lse = -inf, and ommx_decode_combine weighs the states by their lse.
  * Hq = Hkv * r with r in {1,2,4,8}; D = 128 or 64; num_splits <= 512; planes 8-byte aligned.
  *   group_tokens / group_channels   tokens per K group and channels per V vector: 16, 32, 64, 128
  *   scale_bf16 = 1   k_scale / v_scale hold the steps themselves as bf16, not int8 exponents
  *   v_bf16 = 1       v_main is bf16 [P,ps,H,D]; v_scale / v_zp are ignored
- * The matrix-core kernel runs head_dim 128, INT2 V, int8 exponents, either outlier map, and
+ * The matrix-core kernels run INT2 V, int8 exponents, either outlier map, and, at head_dim 128,
  *   32-token groups with 32-channel V vectors and 6 (or 0) outliers, either index plane;
+ *   the same with 1..8 outliers on the bitmap plane, also at head_dim 64 (r in {1,2,4}, Hkv even);
  *   64- or 128-token groups with 32/64/128-channel V vectors and 6 outliers, relidx7 plane;
  *   128-token groups with 10 outliers, relidx7 plane (4 or 8 q heads per kv head).
  * Every other supported shape or recipe (k_outliers up to 16) runs on the plain fp32 kernel.

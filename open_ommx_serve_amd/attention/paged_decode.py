@@ -40,8 +40,8 @@ def auto_num_kv_splits(max_seq_len: int, batch: int, kv_heads: int, n_cu: int = 
                        mean_seq_len: Optional[float] = None, resident: int = 2) -> int:
     """Split count for one decode call.  A workgroup is four waves of one split (a wave covers one
     kv head and all of its q heads, so ``q_per_kv`` does not enter); ``resident`` workgroups fit a
-    compute unit at a time (3 for the kernel that serves up to 4 q heads per kv head, 2 for the
-    others).  Requests about equally long (``mean_seq_len`` at least 0.9 of the longest) get one
+    compute unit at a time (3 for the serving-recipe kernel with up to 4 q heads per kv head, 2
+    otherwise).  Requests about equally long (``mean_seq_len`` at least 0.9 of the longest) get one
     round of workgroups: little is left to even out, and a second round mostly pays the start-up of
     a workgroup (about one step) again.  Requests of different length get two rounds, so that they
     even out, and four when a workgroup would otherwise run for more than sixteen steps.  Never
