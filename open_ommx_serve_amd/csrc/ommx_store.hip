@@ -243,7 +243,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         uint32_t nib = 0;
         bool mfin = true;
         if (FAST6 && fast_done) {
-            if (inv_ok) {                 // one branch per vector, not one per element
+            const float zc = -zp * inv_scale;
+            if (inv_ok && fabsf(zc) < INFINITY) {      // one branch per vector, not one per element
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    s_codes[i * D + d] = static_cast<uint8_t>(int2_code_fused(w[i], inv_scale, zc));
+            } else if (inv_ok) {
 #pragma unroll
                 for (int i = 0; i < 32; ++i)
                     s_codes[i * D + d] = static_cast<uint8_t>(int2_code(w[i] - zp, scale, inv_scale, true));
@@ -392,7 +397,12 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const bool inv_ok = st.inv_ok;
         const float inv_scale = st.inv;
         uint64_t vb8 = 0;
-        if (inv_ok) {
+        const float zc = -zp * inv_scale;
+        if (inv_ok && fabsf(zc) < INFINITY) {
+#pragma unroll
+            for (int c = 0; c < 32; ++c)
+                vb8 |= static_cast<uint64_t>(int2_code_fused(v[c], inv_scale, zc)) << (2 * c);
+        } else if (inv_ok) {
 #pragma unroll
             for (int c = 0; c < 32; ++c)
                 vb8 |= static_cast<uint64_t>(int2_code(v[c] - zp, scale, inv_scale, true)) << (2 * c);

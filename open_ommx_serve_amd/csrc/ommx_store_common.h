@@ -97,6 +97,15 @@ __device__ __forceinline__ uint32_t int2_code(float x, float scale, float inv_sc
     return static_cast<uint32_t>(static_cast<int>(c));
 }
 
+// The same code from w, 2^-e and c = -zp * 2^-e in one fused multiply-add.  (w - zp) * 2^-e as the
+// reference computes it is fl(w - zp) scaled exactly; the fused form rounds the exact (w - zp) * 2^-e
+// once, and scaling by a power of two commutes with rounding while nothing under- or overflows: an
+// underflowing quotient gives code 0 and an overflowing one code 3 either way.  The caller checks
+// that c is finite (a huge zero point over a tiny step would make it infinite).
+__device__ __forceinline__ uint32_t int2_code_fused(float w, float inv_scale, float c) {
+    return __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_fmaf(w, inv_scale, c), 3.0f), 0u, 0u);
+}
+
 int launch_store_generic(const StoreArgs& a, int T, int in_dtype, hipStream_t st);
 
 }  // namespace ommx
