@@ -86,8 +86,11 @@ static_assert(2 * 4 * LdsMap<8>::LDS_WAVE <= 160 * 1024, "8 heads: two workgroup
 // One f16 carries 11 bits: rounding an outlier delta d costs up to |d| * 2^-11, i.e. up to
 // |d| * max|q| * 2^-11 * sm_scale on a logit.  A delta with |d| * max|q| >= BIG_DELTA * 16
 // (at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its residual added exactly; smaller
-// ones stay below that and average a quarter of it.
+// ones stay below that and average a quarter of it.  The bound is held at other sm_scale values
+// (head_dim 64: 64^-0.5) by dividing the threshold by sm_scale / 128^-0.5; the general form, with
+// up to 8 entries per vector, takes three quarters of it.
 constexpr float BIG_DELTA = 2.0f;
+constexpr float BIG_DELTA_SM_SCALE = 0.08838834764831845f;
 // the running maximum of the online softmax is refreshed when a logit (base 2) exceeds it by this
 constexpr float MAX_SLACK = 8.0f;
 
@@ -374,7 +377,8 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
 #pragma unroll
         for (int r = 0; r < NH; ++r)
             qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
-        big_thr[u] = (BIG_DELTA * 16.0f) * (u ? cs1 : cs0) * __builtin_amdgcn_rcpf(qm);
+        big_thr[u] = ((GEN ? 0.75f : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
+                     __builtin_amdgcn_rcpf(qm * a.sm_scale);
     }
     const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
     const uint32_t code_sh = 2u * (c0 & 3u);                      // bit of channel c0's code in that byte; c0 + 1 sits two on

@@ -474,6 +474,17 @@ def test_tail_length_outside_the_buffer_is_held_inside_it(B):
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
 
 
+def test_head_dim_64_eight_outliers_many_requests_stay_inside_the_tolerance():
+    """At head_dim 64 a logit weighs 64^-0.5 instead of 128^-0.5, so the f16 rounding of an outlier's
+    tile entry shows more: the kernel lowers the size from which an entry's residual is added exactly
+    in step (this shape measured 2.2e-3 with the head_dim-128 threshold)."""
+    g = torch.Generator().manual_seed(5)
+    lens = [int(torch.randint(1, 2500, (1,), generator=g)) for _ in range(70)]
+    case = build_decode_case(lens, q_heads=16, kv_heads=8, head_dim=64, seed=9132, permute_tables=True,
+                             sparse_frac=0.02, outliers_per_vector=8)
+    _check(_run(case, num_kv_splits=5), _oracle(case), "d64 k8 70 requests")
+
+
 def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
     """The serving-recipe kernel laid out for 8 q heads per kv head (a lane keeps four heads of one
     token of either group): lengths that end inside the first / second group of a 64-token step,
