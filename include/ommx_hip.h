@@ -57,6 +57,8 @@ extern "C" {
 /* error bit OR-ed into *err_flag by the decode entry points */
 #define OMMX_ERR_TABLE_RANGE  64   /* a page id or group slot outside the planes (kv_pool.py:526-550 guards these on the host) */
 /* error bit OR-ed into *err_flag by ommx_index_convert */
+#define OMMX_ERR_VALUE_RANGE 128   /* decode: a K step above 2^15 (K values beyond some 1e5) does not fit the f16
+                                      operands of the matrix-core kernels; it is held at 2^15 and the result is off */
 #define OMMX_ERR_INDEX_PLANE  32   /* a vector that does not name exactly k positions below group_tokens
                                       (codec.py:173-178 raises ValueError there) */
 
@@ -154,6 +156,8 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 access leaves the planes, and OMMX_ERR_TABLE_RANGE is OR-ed into *err_flag
  *                 (NULL allowed; the caller zeroes it).  0 = extent not given, entries used as
  *                 they are.  A negative b_seq_len counts as 0 and is reported the same way.
+ *                 OMMX_ERR_VALUE_RANGE: a K step above 2^15 met by the serving-recipe kernel, whose
+ *                 f16 operands end there (the step is held at 2^15: finite output, but off).
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,

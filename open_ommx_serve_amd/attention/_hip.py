@@ -30,6 +30,7 @@ def scale_mode(use_pow2: bool, kv_int8_scale: bool) -> int:
 ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE = 1, 2, 4, 8, 16
 ERR_INDEX_PLANE = 32
 ERR_TABLE_RANGE = 64
+ERR_VALUE_RANGE = 128
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 

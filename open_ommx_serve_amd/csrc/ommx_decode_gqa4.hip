@@ -88,11 +88,20 @@ static_assert(2 * 4 * LdsMap<8>::LDS_WAVE <= 160 * 1024, "8 heads: two workgroup
 // (at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its residual added exactly; smaller
 // ones stay below that and average a quarter of it.  The bound is held at other sm_scale values
 // (head_dim 64: 64^-0.5) by dividing the threshold by sm_scale / 128^-0.5; the general form, with
-// up to 8 entries per vector, takes three quarters of it.
+// up to 8 entries per vector or fewer outlier slots than a vector has large values, takes half of it.
 constexpr float BIG_DELTA = 2.0f;
 constexpr float BIG_DELTA_SM_SCALE = 0.08838834764831845f;
 // the running maximum of the online softmax is refreshed when a logit (base 2) exceeds it by this
 constexpr float MAX_SLACK = 8.0f;
+// The base operand (1 + code*2^(2m-10)) * 2^e carries a constant A*2^e per channel, up to 2^8 times
+// the signal, which the bias MFMA takes out again: two large sums that cancel in fp32.  From steps
+// of 2^EXACT_STEP_EXP on (values a hundred or more wide inside one vector) that shows on the logits, and
+// the step's two groups take the operand code*2^(2m-10+e) instead (one packed subtraction more per operand
+// register, exact: both terms share the exponent) and drops the 2^e bias column.
+constexpr int EXACT_STEP_EXP = 5;
+// f16 operands: steps above 2^15 do not fit (K values beyond some 1e5); such a step is held at 2^15
+// and OMMX_ERR_VALUE_RANGE is reported
+constexpr int MAX_STEP_EXP = 15;
 
 // K pair p of a code dword: channels p (low half) and p+8 (high half) as f16 with the 2-bit
 // code at mantissa bits [2m+1:2m], m = k_pos(p) in 1..4, where the element reads
@@ -248,6 +257,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
         }
     };
     bool bad_id = false;            // a table entry outside the planes was seen (and clamped)
+    bool over_step = false;         // a K step above 2^MAX_STEP_EXP was seen (and held there); wave-uniform
     u32x4 kr[2], vr[2];
     u32x2 vzp;
     uint32_t vsc, vrow;
@@ -377,7 +387,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
 #pragma unroll
         for (int r = 0; r < NH; ++r)
             qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
-        big_thr[u] = ((GEN ? 0.75f : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
+        big_thr[u] = ((GEN ? 0.5f : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
                      __builtin_amdgcn_rcpf(qm * a.sm_scale);
     }
     const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
@@ -405,6 +415,16 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
         }
 
         // ------------------------------------------------------------------ stage K
+        bool exact_step;                        // some step of these 64 tokens is 2^EXACT_STEP_EXP or more (wave-uniform)
+        {
+            typedef short s16x2e __attribute__((ext_vector_type(2)));
+            const s16x2e top2 = __builtin_elementwise_max(
+                __builtin_bit_cast(s16x2e, __builtin_amdgcn_perm(0u, g_sc[0], 0x010C000Cu)),
+                __builtin_bit_cast(s16x2e, __builtin_amdgcn_perm(0u, g_sc[1], 0x010C000Cu)));
+            const short e_top = top2[0] > top2[1] ? top2[0] : top2[1];
+            exact_step = __any(e_top >= EXACT_STEP_EXP * 256) != 0;
+            if (__builtin_expect(exact_step, 0)) over_step |= __any(e_top > MAX_STEP_EXP * 256) != 0;
+        }
         {
             u32x2* krow = reinterpret_cast<u32x2*>(sm + OFF_KT + lane * KT_ROW);
             krow[0] = u32x2{kr[0][0], kr[0][1]};
@@ -420,7 +440,9 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
                 const uint32_t e2 = __builtin_amdgcn_perm(0u, g_sc[g], 0x010C000Cu);       // (e1 << 8, e0 << 8)
                 typedef short s16x2 __attribute__((ext_vector_type(2)));
                 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-                const s16x2 ec = __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256});
+                const s16x2 ec = __builtin_elementwise_min(
+                    __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256}),
+                    s16x2{MAX_STEP_EXP * 256, MAX_STEP_EXP * 256});
                 const uint32_t m2 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, ec) * u16x2{4, 4} + u16x2{0x3C00, 0x3C00});
                 mg[g * 128] = static_cast<uint16_t>(m2);
                 mg[g * 128 + 2] = static_cast<uint16_t>(m2 >> 16);
@@ -551,20 +573,35 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
                 }
             }
             const u32x4* mg = reinterpret_cast<const u32x4*>(sm + OFF_MAG + g * 256 + kq * 64);
+            auto base_mfmas = [&](auto EX) {
+                // EX: the operand without its constant, code * 2^(2m-10+e) = pattern - 2^e
+                auto op = [&](uint32_t pat, uint32_t mag) {
+                    if constexpr (!decltype(EX)::value) return pat;
+                    else return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, pat) - __builtin_bit_cast(f16x2, mag));
+                };
 #pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {          // code dword: channels 16*hf .. 16*hf+15 of the quarter
-                uint32_t w[2], wu[2], wd[2];
+                for (int hf = 0; hf < 2; ++hf) {          // code dword: channels 16*hf .. 16*hf+15 of the quarter
+                    uint32_t w[2], wu[2], wd[2];
 #pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2) { w[t2] = kw[t2][hf]; wu[t2] = w[t2] << 2; wd[t2] = w[t2] >> 6; }
-                const u32x4 ma = mg[2 * hf], mb = mg[2 * hf + 1];
+                    for (int t2 = 0; t2 < 2; ++t2) { w[t2] = kw[t2][hf]; wu[t2] = w[t2] << 2; wd[t2] = w[t2] >> 6; }
+                    const u32x4 ma = mg[2 * hf], mb = mg[2 * hf + 1];
 #pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2)
-                    d[t2] = mfma_f16(aq[2 * hf], u32x4{k_pair<0>(w[t2], wu[t2], wd[t2], ma[0]), k_pair<1>(w[t2], wu[t2], wd[t2], ma[1]),
-                                                       k_pair<2>(w[t2], wu[t2], wd[t2], ma[2]), k_pair<3>(w[t2], wu[t2], wd[t2], ma[3])}, d[t2]);
+                    for (int t2 = 0; t2 < 2; ++t2)
+                        d[t2] = mfma_f16(aq[2 * hf], u32x4{op(k_pair<0>(w[t2], wu[t2], wd[t2], ma[0]), ma[0]), op(k_pair<1>(w[t2], wu[t2], wd[t2], ma[1]), ma[1]),
+                                                           op(k_pair<2>(w[t2], wu[t2], wd[t2], ma[2]), ma[2]), op(k_pair<3>(w[t2], wu[t2], wd[t2], ma[3]), ma[3])}, d[t2]);
 #pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2)
-                    d[t2] = mfma_f16(aq[2 * hf + 1], u32x4{k_pair<4>(w[t2], wu[t2], wd[t2], mb[0]), k_pair<5>(w[t2], wu[t2], wd[t2], mb[1]),
-                                                           k_pair<6>(w[t2], wu[t2], wd[t2], mb[2]), k_pair<7>(w[t2], wu[t2], wd[t2], mb[3])}, d[t2]);
+                    for (int t2 = 0; t2 < 2; ++t2)
+                        d[t2] = mfma_f16(aq[2 * hf + 1], u32x4{op(k_pair<4>(w[t2], wu[t2], wd[t2], mb[0]), mb[0]), op(k_pair<5>(w[t2], wu[t2], wd[t2], mb[1]), mb[1]),
+                                                               op(k_pair<6>(w[t2], wu[t2], wd[t2], mb[2]), mb[2]), op(k_pair<7>(w[t2], wu[t2], wd[t2], mb[3]), mb[3])}, d[t2]);
+                }
+            };
+            if (__builtin_expect(exact_step, 0)) {
+                base_mfmas(std::true_type{});
+                // the bias MFMA must not take the constant out a second time: its 2^e column of this group reads zeros
+                lds_fence();
+                reinterpret_cast<uint32_t*>(sm + OFF_MAG + g * 256)[lane] = 0u;
+            } else {
+                base_mfmas(std::false_type{});
             }
             if constexpr (NH == 4) {
                 // rows 4kq..4kq+3 of every result hold the four heads: the lane keeps its own token block
@@ -841,6 +878,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
     }
 
     report_table_range(a.err, bad_id);
+    if (over_step && a.err && lane == 0) atomicOr(a.err, OMMX_ERR_VALUE_RANGE);
 
     // ---- epilogue: o = (f*(acc - sum p*2^e) + sum p*zp) / l, f = 16 or 4; lse = m + ln l ----------
     // sums live in the lanes of the same column j: rows 0-3 (kq 0) zero points, 4-7 (kq 1) steps, 8 (kq 2) ones

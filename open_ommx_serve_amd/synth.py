@@ -115,7 +115,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
                       table_dtype: torch.dtype = torch.int32, sparse_gain: float = 8.0,
                       outlier_repr: str = "bitmap", kv_outlier_map: bool = True,
                       use_pow2: bool = True, kv_int8_scale: bool = True,
-                      group_tokens: int = 32, group_channels: int = 32, v_format: str = "i2") -> DecodeCase:
+                      group_tokens: int = 32, group_channels: int = 32, v_format: str = "i2",
+                      outlier_gain: float = 12.0) -> DecodeCase:
     """Synthesize ``len(seq_lens)`` requests, store their packed prefixes, gather their tails.
 
     Each request gets its own slice of page / group-slot ids out of one shared pool; with
@@ -157,7 +158,8 @@ def build_decode_case(seq_lens: Sequence[int], *, q_heads: int = 32, kv_heads: i
     src = []
     po = go = 0
     for b, n in enumerate(int(x) for x in seq_lens):
-        K, V = synth_kv(n, H, D, seed, sparse_frac=sparse_frac, sparse_gain=sparse_gain, stream=b)
+        K, V = synth_kv(n, H, D, seed, sparse_frac=sparse_frac, sparse_gain=sparse_gain, stream=b,
+                        outlier_gain=outlier_gain)
         edge = win.boundary(n)
         ti = win.tail_indices(n)
         tails.append(len(ti))

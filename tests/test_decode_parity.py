@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import oracle.ommx_oracle as O
+from open_ommx_serve_amd.attention import _hip
 from open_ommx_serve_amd.attention.kv_window import WindowSpec
 from open_ommx_serve_amd.attention.paged_decode import (make_attn_logits,
                                                         ommx_paged_decode_attention_canonical)
@@ -483,6 +484,47 @@ def test_head_dim_64_eight_outliers_many_requests_stay_inside_the_tolerance():
     case = build_decode_case(lens, q_heads=16, kv_heads=8, head_dim=64, seed=9132, permute_tables=True,
                              sparse_frac=0.02, outliers_per_vector=8)
     _check(_run(case, num_kv_splits=5), _oracle(case), "d64 k8 70 requests")
+
+
+@pytest.mark.parametrize("hq,hkv,D,k,own_map", [(32, 8, 128, 6, True), (64, 8, 128, 6, True), (32, 8, 128, 5, False),
+                                                 (8, 8, 128, 3, True), (16, 8, 64, 6, True)])
+def test_large_steps_take_the_operand_without_its_constant(hq, hkv, D, k, own_map):
+    """Channels whose every value is large (x150 here), or vectors that hold more large values than they
+    have outlier slots, get steps of 2^6 and more; the base operand (1 + code * 2^-j) * 2^e then carries
+    a constant that cancels badly in fp32 (one such case measured 4.7e-3), so those groups use
+    code * 2^(e-j) and no 2^e bias column."""
+    case = build_decode_case([1500, 333, 2100], q_heads=hq, kv_heads=hkv, head_dim=D, seed=15, permute_tables=True,
+                             sparse_frac=0.02, sparse_gain=40.0, outlier_gain=150.0, outliers_per_vector=k,
+                             kv_outlier_map=own_map)
+    exps = case.planes["k_scale"].to(torch.int32)
+    assert int((exps >= 6).sum()) > 100 and int(exps.max()) <= 15
+    err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+    wo, wl = _oracle(case)
+    for S in (None, 3):
+        o, lse = _run(case, num_kv_splits=S, err_flag=err)
+        e = (o.double() - wo).abs()
+        assert e.max().item() <= MAX_ABS and e.mean().item() <= MEAN_ABS, f"S{S}: {e.max().item():.3e}"
+        # the logits run into the thousands here: an fp32 lse carries 1e-4 of rounding per thousand
+        assert ((lse.double() - wl).abs() <= 2e-3 + 2e-6 * wl.abs()).all(), f"S{S}: lse"
+    assert int(err.item()) == 0
+
+
+def test_a_step_beyond_the_f16_operands_is_reported():
+    """K values around 1e6 give steps above 2^15, which the f16 operands of the matrix-core kernel cannot
+    carry: the step is held at 2^15, the result stays finite, and the error word says so.  The plain
+    kernel serves such a cache (fp32 throughout)."""
+    case = build_decode_case([700], q_heads=32, kv_heads=8, seed=16, outlier_gain=3.0e5)
+    assert int(case.planes["k_scale"].to(torch.int32).max()) > 15
+    err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+    o, lse = _run(case, num_kv_splits=2, err_flag=err)
+    assert int(err.item()) & _hip.ERR_VALUE_RANGE
+    assert torch.isfinite(o).all()
+    err.zero_()
+    po, pl = _run(case, num_kv_splits=2, ref_kernel=True, err_flag=err)
+    wo, wl = _oracle(case)
+    assert (po.double() - wo).abs().max().item() <= MAX_ABS
+    assert ((pl.double() - wl).abs() <= 2e-3 + 2e-6 * wl.abs()).all()       # logits in the 1e5 range
+    assert int(err.item()) == 0
 
 
 def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
