@@ -527,6 +527,20 @@ def test_a_step_beyond_the_f16_operands_is_reported():
     assert int(err.item()) == 0
 
 
+@pytest.mark.parametrize("B,hq", [(3, 32), (33, 32), (70, 32), (40, 64)])
+def test_long_tails_take_several_passes_in_every_combine_kernel(B, hq):
+    """A recent window of 300 tokens gives tails of up to 339 bf16 rows: several chunks of 64 rows in the
+    combine with one workgroup per q head (3 requests), several passes of 128 in the one per kv head,
+    with the first pass asked for early (33 and 40 requests of 8 kv heads) and without (70)."""
+    win = WindowSpec(sink_tokens=8, recent_window=300, group_tokens=32, page_size=16)
+    g = torch.Generator().manual_seed(B)
+    lens = [int(torch.randint(20, 1500, (1,), generator=g)) for _ in range(B)]
+    case = build_decode_case(lens, q_heads=hq, kv_heads=8, seed=21, permute_tables=True, sparse_frac=0.005,
+                             window=win)
+    assert int(case.b_tail_len.max()) > 256
+    _check(_run(case, num_kv_splits=4), _oracle(case), f"B{B}")
+
+
 def test_eight_q_heads_per_kv_head_partial_groups_empty_splits_and_cap():
     """The serving-recipe kernel laid out for 8 q heads per kv head (a lane keeps four heads of one
     token of either group): lengths that end inside the first / second group of a 64-token step,
