@@ -273,6 +273,21 @@ def test_store_heavy_ties_and_degenerate_vectors():
     assert_planes_equal(_hip(K, V), O.pack_kv(K, V), what="ties")
 
 
+def test_store_huge_constant_vectors_take_the_two_step_code_path():
+    """The INT2 codes come from one fused multiply-add w * 2^-e - zp * 2^-e; a constant vector of huge
+    values has a tiny step (the 1e-8 range floor) and a zero point whose scaled value overflows, so the
+    kernel must fall back to (w - zp) * 2^-e there: K at the selector's limit, V at the end of bf16."""
+    K, V = synth_kv(128, 2, 128, 31, sparse_frac=0.01)
+    K[:32, 0, 3] = 9.0e8
+    K[32:64, 1, 7] = -9.0e8
+    V[5, 0, :32] = 3.0e38
+    V[6, 1, 32:64] = -3.0e38
+    V[7, 0, 64:96] = torch.linspace(1.0e38, 3.0e38, 32).to(torch.bfloat16)
+    for fp32 in (False, True):
+        Kx, Vx = (K.float(), V.float()) if fp32 else (K, V)
+        assert_planes_equal(_hip(Kx, Vx), O.pack_kv(Kx, Vx), what=f"huge fp32={fp32}")
+
+
 def test_store_fp32_inputs_round_zero_point_and_map():
     g = torch.Generator().manual_seed(9)
     K = torch.randn(128, 2, 64, generator=g) * 3.0
