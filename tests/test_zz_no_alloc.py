@@ -95,6 +95,20 @@ def test_two_calls_in_a_row_second_smaller_match_the_workspace_entry_points():
         _close(o, lse, oo, ol, f"{name} vs oracle")
 
 
+def test_head_dim_64_and_eight_q_heads_per_kv_head_through_the_same_entry_point():
+    # the layouts of the serving-recipe kernel that came later: pairs of 64-channel kv heads, 8 q heads per kv head
+    for case, S, name in ((build_decode_case([900, 70], q_heads=8, kv_heads=2, head_dim=64, seed=6), 4, "d64"),
+                          (build_decode_case([1300], q_heads=64, kv_heads=8, seed=7, sparse_frac=0.005), 9, "gqa8")):
+        rc, o, lse = _noalloc(case, S)
+        assert rc == 0, _hip.load().ommx_last_error()
+        torch.cuda.synchronize()
+        wo, wl = _existing(case, S)
+        torch.cuda.synchronize()
+        assert (o - wo).abs().max().item() <= 1e-5, f"{name}: same kernels, same split count"
+        oo, ol = _oracle(case)
+        _close(o, lse, oo, ol, f"{name} vs oracle")
+
+
 def test_sizes_beyond_the_built_in_array_are_refused():
     case = build_decode_case([1024] * 64, seed=3)          # 64 * 32 * 257 * 129 floats > 2 Mi
     rc, _, _ = _noalloc(case, 256)
