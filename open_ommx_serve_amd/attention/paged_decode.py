@@ -137,7 +137,10 @@ def ommx_paged_decode_attention_canonical(
     requests are on average, see :func:`auto_num_kv_splits`.  ``err_flag`` (not in the reference's
     signature either): an int32 device tensor that receives ``_hip.ERR_TABLE_RANGE`` when a page id
     or group slot of the tables lies outside the planes (the kernels clamp such an entry, so nothing
-    is read out of bounds; the reference leaves these checks to the pools, ``kv_pool.py:526-550``).
+    is read out of bounds; the reference leaves these checks to the pools, ``kv_pool.py:526-550``),
+    and ``_hip.ERR_VALUE_RANGE`` when a K step lies above 2^15 (K values beyond some 1e5), which the
+    f16 operands of the matrix-core kernel cannot carry: the output is finite but off, and
+    ``_force_reference_kernel=True`` serves such a cache.
     """
     pages, ngroups = int(k_base.shape[0]), int(k_scale.shape[0])
     ps = int(page_size)
