@@ -311,11 +311,17 @@ def ommx_paged_decode_attention_canonical(
         max_seq = int(b_seq_len.max().item()) if int(b_seq_len.numel()) > 0 else 1
     # the serving-recipe kernel keeps three workgroups per compute unit resident with up to 4 q heads
     # per kv head (two with 8, and so do the other kernels); it also serves the call in one launch
-    lean = (D == 128 and Hq // Hkv <= 4 and k == 6 and group_tokens == 32 and group_channels == 32
+    tuned = D == 128 and Hq // Hkv <= 4 and k == 6
+    general4 = bitmap_read and 1 <= k <= 6 and ((D == 128 and Hq // Hkv <= 4) or      # (7, 8 outliers: two resident)
+                                                (D == 64 and Hq // Hkv <= 2 and Hkv % 2 == 0))
+    lean = ((tuned or general4) and group_tokens == 32 and group_channels == 32
             and not scale_bf16 and not v_bf16 and not _force_reference_kernel)
     if num_kv_splits is None:
-        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv, _cu_count(q.device), Hq // Hkv, group_tokens,
-                                           mean_seq_len, resident=3 if lean else 2)
+        # (at head_dim 64 a wave of that kernel takes a pair of kv heads)
+        paired = D == 64 and bitmap_read and 1 <= k <= 8 and Hq // Hkv <= 4 and Hkv % 2 == 0 and not (
+            scale_bf16 or v_bf16 or _force_reference_kernel) and group_tokens == 32 and group_channels == 32
+        num_kv_splits = auto_num_kv_splits(max_seq, B, Hkv // 2 if paired else Hkv, _cu_count(q.device),
+                                           Hq // Hkv, group_tokens, mean_seq_len, resident=3 if lean else 2)
     S = max(1, int(num_kv_splits))
     if attn_logits is None:
         attn_logits = make_attn_logits(B, Hq, S, D, q.device)

@@ -88,7 +88,8 @@ static_assert(2 * 4 * LdsMap<8>::LDS_WAVE <= 160 * 1024, "8 heads: two workgroup
 // (at most 1.4e-3 on a logit at sm_scale = 128^-0.5) gets its residual added exactly; smaller
 // ones stay below that and average a quarter of it.  The bound is held at other sm_scale values
 // (head_dim 64: 64^-0.5) by dividing the threshold by sm_scale / 128^-0.5; the general form, with
-// up to 8 entries per vector or fewer outlier slots than a vector has large values, takes half of it.
+// up to 8 entries per vector, takes three quarters of it, and half with fewer than 6 outlier slots (more
+// large values then stay in the base codes, the steps grow, and so do the entries).
 constexpr float BIG_DELTA = 2.0f;
 constexpr float BIG_DELTA_SM_SCALE = 0.08838834764831845f;
 // the running maximum of the online softmax is refreshed when a logit (base 2) exceeds it by this
@@ -133,11 +134,14 @@ __device__ __forceinline__ uint32_t pk_u16(uint32_t lo, uint32_t hi) { return (l
 // head_dim 64 (a.half): the planes of two neighbouring 64-channel kv heads read exactly like one
 // 128-channel head, so a wave takes the pair as one head whose q heads are those of both, each
 // zero on the other one's channels, and writes each q head only its own half of the output.
-template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER, int NH = 4, bool GEN = false>
-__global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
+template <int IDX, bool OWN_MAP, bool PARTIAL, int ORDER, int NH = 4, bool GEN = false, int KSLOTS = 6>
+__global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : OMMX_GQA4_WAVES) decode_gqa4_kernel(DecodeArgs a) {
     static_assert(NH == 4 || (NH == 8 && !PARTIAL), "4 heads (or fewer, PARTIAL) or exactly 8");
     static_assert(!GEN || IDX == 0, "the general form reads bitmaps");
-    constexpr int KMAX = GEN ? 8 : 6;                 // outliers per vector, upper bound
+    // outlier slots walked per vector: the general form walks 4 or 8 whatever a.kout is (loads and
+    // arithmetic of all slots go out together; only the writes of the slots beyond a.kout are skipped)
+    constexpr int KMAX = GEN ? KSLOTS : 6;
+    static_assert(KMAX == 4 || KMAX == 6 || KMAX == 8, "outlier slots");
     const int kout = GEN ? a.kout : 6;
     const bool half = GEN && a.half;
     using Lds = LdsMap<NH>;
@@ -387,7 +391,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
 #pragma unroll
         for (int r = 0; r < NH; ++r)
             qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
-        big_thr[u] = ((GEN ? 0.5f : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
+        big_thr[u] = ((GEN ? (kout < 6 ? 0.5f : 0.75f) : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
                      __builtin_amdgcn_rcpf(qm * a.sm_scale);
     }
     const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
@@ -500,8 +504,8 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
                                          : static_cast<uint32_t>(ov64 >> (nib_sh + 24 * u)) & 0xFFFFFFu;
                 const f32x2 l01 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
                 const f32x2 l23 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 1);
-                const f32x2 l45 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2);
-                const f32x2 l67 = GEN ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 3) : f32x2{0.0f, 0.0f};
+                const f32x2 l45 = KMAX > 4 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2) : f32x2{0.0f, 0.0f};
+                const f32x2 l67 = KMAX > 6 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 3) : f32x2{0.0f, 0.0f};
                 const float lv[8] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1], l67[0], l67[1]};
                 // The base MFMA takes every position of the K rows as it is stored; the tile entry of an
                 // outlier is what is missing on top of its stored 2-bit code, which the lane looks up
@@ -514,7 +518,6 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
                 uint32_t cb[KMAX];
 #pragma unroll
                 for (int sidx = 0; sidx < KMAX; ++sidx) {
-                    if (GEN && sidx >= kout) break;
                     if constexpr (IDX == 0) {
                         pos[sidx] = __builtin_ctz(bm) & 31;
                         if (sidx < KMAX - 1) bm &= bm - 1;
@@ -527,11 +530,11 @@ __global__ void __launch_bounds__(256, (NH == 8 || GEN) ? 2 : OMMX_GQA4_WAVES) d
                 }
 #pragma unroll
                 for (int sidx = 0; sidx < KMAX; ++sidx) {
-                    if (GEN && sidx >= kout) break;
                     const float dl0 = fmaf(lv[sidx], a1, b1);
                     const float code = static_cast<float>((cb[sidx] >> (code_sh + 2 * u)) & 3u);
                     const float dl = fmaf(-code, sc, dl0);
                     const _Float16 hi = static_cast<_Float16>(dl);
+                    if (GEN && sidx >= kout) continue;          // an unused slot (uniform): nothing to write
                     if constexpr (!decltype(RES)::value) {
                         dt[pos[sidx] * (TILE_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
                         dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
@@ -949,6 +952,12 @@ int launch_decode_gqa4(const DecodeArgs& a_in, int Dh, int R, hipStream_t st) {
     const int order = a.B == 1 ? 0 : (a.B > 64 && a.B <= 256 ? 2 : 1);
 #define OMMX_GO(IDX, MAP, PART, ORD, NH, GEN) \
     hipLaunchKernelGGL((decode_gqa4_kernel<IDX, MAP, PART, ORD, NH, GEN>), grid, block, shm, st, a)
+#define OMMX_GO_GEN(MAP, PART, NH)                                                                          \
+    do {                                                                                                    \
+        if (a.kout <= 4) hipLaunchKernelGGL((decode_gqa4_kernel<0, MAP, PART, 2, NH, true, 4>), grid, block, shm, st, a); \
+        else if (a.kout <= 6) hipLaunchKernelGGL((decode_gqa4_kernel<0, MAP, PART, 2, NH, true, 6>), grid, block, shm, st, a); \
+        else hipLaunchKernelGGL((decode_gqa4_kernel<0, MAP, PART, 2, NH, true, 8>), grid, block, shm, st, a);             \
+    } while (0)
 #define OMMX_GO_ORD(IDX, MAP, PART, NH)                              \
     do {                                                             \
         if (order == 0) OMMX_GO(IDX, MAP, PART, 0, NH, false);       \
@@ -957,8 +966,8 @@ int launch_decode_gqa4(const DecodeArgs& a_in, int Dh, int R, hipStream_t st) {
     } while (0)
     if (general) {
         // one instantiation per (outlier map, head layout): outlier count, head count and head_dim at run time
-        if (nh == 8) { if (own_map) OMMX_GO(0, true, false, 2, 8, true); else OMMX_GO(0, false, false, 2, 8, true); }
-        else { if (own_map) OMMX_GO(0, true, true, 2, 4, true); else OMMX_GO(0, false, true, 2, 4, true); }
+        if (nh == 8) { if (own_map) OMMX_GO_GEN(true, false, 8); else OMMX_GO_GEN(false, false, 8); }
+        else { if (own_map) OMMX_GO_GEN(true, true, 4); else OMMX_GO_GEN(false, true, 4); }
         return 0;
     }
     switch ((nh == 8 ? 8 : 0) | (nh < 4 ? 4 : 0) | (a.idx_repr ? 2 : 0) | (own_map ? 1 : 0)) {
@@ -976,6 +985,7 @@ int launch_decode_gqa4(const DecodeArgs& a_in, int Dh, int R, hipStream_t st) {
         default: OMMX_GO_ORD(1, true, false, 8); break;
     }
 #undef OMMX_GO
+#undef OMMX_GO_GEN
 #undef OMMX_GO_ORD
     return 0;
 }
