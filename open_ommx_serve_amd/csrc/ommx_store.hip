@@ -227,7 +227,10 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         float mc = 0.0f, ms = 0.0f;
         if (kout > 0 && own_map) {
             mc_b = f32_to_bf16_rne(__fdiv_rn(omx + omn, 2.0f));
-            ms_b = f32_to_bf16_rne(__fdiv_rn(12.0f, fmaxf(omx - omn, 1e-8f)));
+            // `12.0 / o_range` with a Python scalar on the left is torch's reciprocal-then-multiply
+            // (Tensor.__rtruediv__): two roundings, which differ from one division once in some 1e5
+            // vectors after the bf16 rounding (pack.py:492)
+            ms_b = f32_to_bf16_rne(__fmul_rn(__fdiv_rn(1.0f, fmaxf(omx - omn, 1e-8f)), 12.0f));
             mc = bf16_to_f32(mc_b);
             ms = bf16_to_f32(ms_b);
         }

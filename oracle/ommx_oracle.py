@@ -340,7 +340,9 @@ def pack_kv(K: torch.Tensor, V: torch.Tensor, *, page_size: int = 16,
         if kv_outlier_map:                                  # pack.py:486-498
             omn, omx = _masked_min_max(gw, omask)
             center = _bf16_rt((omx + omn) / 2.0)
-            mscale = _bf16_rt(12.0 / (omx - omn).clamp_min(1e-8))
+            # (scalar / tensor is reciprocal-then-multiply in torch: two roundings; written out so that
+            # the oracle does not depend on how a torch version spells Tensor.__rtruediv__)
+            mscale = _bf16_rt(torch.reciprocal((omx - omn).clamp_min(1e-8)) * 12.0)
             mapped = (gw - center) * mscale
         else:                                               # pack.py:502-506
             mapped = (gw - zp) / scale

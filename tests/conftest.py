@@ -14,7 +14,8 @@ if ROOT not in sys.path:
 GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
 PLANE_NAMES = ("k_base", "k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale",
                "k_fp4_mapcenter", "v_main", "v_scale", "v_zp")
-GOLDEN_CASES = ("tiny_ties", "small_gauss", "layer_outliers", "wide_range", "fp32_inputs")
+GOLDEN_CASES = ("tiny_ties", "small_gauss", "layer_outliers", "wide_range", "fp32_inputs",
+                "map_scale_rounding")
 
 
 def pytest_configure(config):

@@ -3,6 +3,7 @@
 Run ONCE in the build container, where the reference checkout is mounted:
 
     python tests/golden/make_golden.py /root/reference
+    python tests/golden/make_golden.py /root/reference --only map_scale_rounding   (adds one case)
 
 The bit pattern of ``ommx_pack_kv_canonical_block`` (outlier tie order, fp32 operation
 order, bf16 rounding, log2/log ulps) is the one thing on this path that no closed form or
@@ -30,7 +31,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PLANES = ("k_base", "k_scale", "k_zp", "k_obmp", "k_oval", "k_fp4_mapscale",
           "k_fp4_mapcenter", "v_main", "v_scale", "v_zp")
 SEEDS = {"tiny_ties": 101, "small_gauss": 202, "layer_outliers": 303, "wide_range": 404,
-         "fp32_inputs": 505}
+         "fp32_inputs": 505, "map_scale_rounding": 606}
 RECIPE = dict(outliers_per_vector=6, outlier_select="signed", outlier_repr="bitmap",
               k_format="i2f4", use_pow2=True, kv_outlier_map=True, kv_int8_scale=True,
               group_tokens=32, group_channels=32, page_size=16, v_format="i2")
@@ -79,8 +80,12 @@ def main(ref_root: str) -> None:
     from ommx_gpu_serve.attention.pack import (  # type: ignore
         dequant_kv_canonical, ommx_pack_kv_canonical_block)
 
+    only = sys.argv[3:] if len(sys.argv) > 3 and sys.argv[2] == "--only" else None
     index = {}
-    for name in SEEDS:
+    if only:      # add cases to the fixtures already written: the other files stay as they are
+        with open(os.path.join(HERE, "pack_index.json")) as f:
+            index = json.load(f)["sha256"]
+    for name in (only or SEEDS):
         g = torch.Generator().manual_seed(SEEDS[name])
         K, V = _case_inputs(name, g)
         planes = ommx_pack_kv_canonical_block(K, V, **RECIPE)
@@ -94,6 +99,8 @@ def main(ref_root: str) -> None:
         print(name, {p: tuple(planes[p].shape) for p in PLANES})
     with open(os.path.join(HERE, "pack_index.json"), "w") as f:
         json.dump({"recipe": RECIPE, "torch": torch.__version__, "sha256": index}, f, indent=1)
+    if only:
+        return
 
     vindex = {}
     for name, (over, shape, seed) in VARIANTS.items():
@@ -158,6 +165,25 @@ def _case_inputs(name: str, g: torch.Generator):
         # fp32 K/V: the zero point and the map parameters are then genuinely rounded
         T, H, D = 64, 2, 64
         return torch.randn(T, H, D, generator=g), torch.randn(T, H, D, generator=g) * 3.0
+    elif name == "map_scale_rounding":
+        # ``12.0 / o_range`` (pack.py:492) has the Python scalar on the left, which torch evaluates as
+        # reciprocal(o_range) * 12.0: two roundings.  About six ranges in a million give another bf16
+        # map scale than one correctly rounded division; every K vector here has such a range
+        # (smallest value 0, largest the range), found by search from this seed.
+        T, H, D = 32, 1, 64
+        r = torch.exp2(torch.rand(4_000_000, generator=g) * 20 - 8) * (1 + torch.rand(4_000_000, generator=g))
+        one = (torch.tensor(12.0) / r).to(torch.bfloat16).view(torch.int16)
+        two = (torch.reciprocal(r) * 12.0).to(torch.bfloat16).view(torch.int16)
+        hits = r[(one != two).nonzero().flatten()]
+        assert len(hits) >= 16, len(hits)
+        K = torch.empty(T, H, D)
+        for c in range(D):
+            rc = hits[c % len(hits)]
+            col = (0.3 + 0.4 * torch.rand(T, generator=g)) * rc
+            col[(3 * c) % T] = 0.0
+            col[(3 * c + 7) % T] = rc
+            K[:, 0, c] = col
+        return K, torch.randn(T, H, D, generator=g)
     else:
         raise KeyError(name)
     return K.to(torch.bfloat16), V.to(torch.bfloat16)
