@@ -46,12 +46,6 @@ namespace {
 
 using namespace decode_util;
 
-#ifndef OMMX_Q_IN_REGS
-#define OMMX_Q_IN_REGS 1
-#endif
-#ifndef OMMX_LATE_FETCH
-#define OMMX_LATE_FETCH 0
-#endif
 #ifndef OMMX_GQA4_WAVES
 #define OMMX_GQA4_WAVES 3          // waves per SIMD the register budget is set for
 #endif
@@ -362,18 +356,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             }
         }
     }
-#if OMMX_Q_IN_REGS
     auto q_of = [&](int u, int r) { return __uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16)); };
-#else
-    // q of head r, channel 2*lane + u: read again where it is needed (the residual walk, seldom taken)
-    auto q_of = [&](int u, int r) {
-        const int sl = min(r, heads - 1);
-        uint32_t w = *reinterpret_cast<const uint32_t*>(
-            a.q + b * a.q_sb + (int64_t)(qh0 + sl) * a.q_sh + (half ? (2 * lane) & 63 : 2 * lane));
-        if (half && (lane >> 5) != sl / r_half) w = 0u;
-        return __uint_as_float(u ? (w & 0xFFFF0000u) : (w << 16));
-    };
-#endif
     // ---- lane constants of the loop ------------------------------------------------------------
     // channel pass: lane = channels c0 = 2*lane, c0 + 1
     const uint32_t c0 = 2u * lane;
@@ -458,9 +441,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             }
         }
         lds_fence();
-#if !OMMX_LATE_FETCH
         if (more) fetch_k();
-#endif
 
         // ------------------------------------------------------------------ QK
         // 4 heads: the lane keeps the logits of its own token n0 + lane (one 16-token block of one group);
@@ -555,9 +536,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             if (res0) walk(std::true_type{}, std::integral_constant<int, 0>{});
             if (res1) walk(std::true_type{}, std::integral_constant<int, 1>{});
             lds_fence();
-#if !OMMX_LATE_FETCH
             if (more) fetch_params_g(g);
-#endif
             // both 16-token blocks of the group go through the eight k-steps together (two independent
             // accumulation chains): tile rows (read, clear), then the base codes
             f32x4 d[2] = {f32x4{0, 0, 0, 0}, f32x4{0, 0, 0, 0}};
@@ -636,9 +615,6 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) dbias = mfma_f16(aq[ks], bp[ks], dbias);
         }
-#if OMMX_LATE_FETCH
-        if (more) { fetch_k(); fetch_params_g(0); fetch_params_g(1); }
-#endif
         if (more) fetch_tables(n0 + 128);
         lds_fence();
 
