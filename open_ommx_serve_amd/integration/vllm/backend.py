@@ -320,7 +320,6 @@ class OMMXCanonicalImpl(_ImplBase):
             seq_before = int(mgr.seq_lens[i]) - (t1 - t0)
             if seq_before <= 0:
                 pool.reset_slot(slot)
-                mgr.planner.reset(slot)
             elif int(pool.seq_len[slot]) != seq_before:
                 raise RuntimeError(f"batched write: slot {slot} holds {pool.seq_len[slot]} tokens, "
                                    f"the step continues from {seq_before}")

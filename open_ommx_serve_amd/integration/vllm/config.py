@@ -1,15 +1,20 @@
 """Serving recipe + per-model geometry (reference ``integration/vllm/config.py:219-440``).
 
-Same field names, defaults and environment knobs as the reference's ``OMMXServingConfig``;
-the defaults are the serving recipe the tuned kernels are built for (i2f4, 6 signed outliers,
-flat bitmask, power-of-two steps, dedicated FP4 map, 32-token / 32-channel groups, sink 8,
-recent 32, page 16).
+The dataclass keeps the reference's field names and defaults, and the resolver reads the
+reference's environment names, because those two lists are the interface a deployment
+already has.  The defaults are the serving recipe the tuned kernels are built for (i2f4,
+6 signed outliers, flat bitmask, power-of-two steps, dedicated FP4 map, 32-token /
+32-channel groups, sink 8, recent 32, page 16).
+
+How a value is found is one table (``KNOBS``): per field the environment names that may
+carry it, in order of precedence, and the parser for its text.  ``explain_knobs()`` prints
+that table, so the list of knobs a worker honours can be read from a running process.
 """
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass, field
-from typing import Any, Optional
+from dataclasses import dataclass, field, fields
+from typing import Any, Callable, Dict, Mapping, NamedTuple, Optional, Tuple
 
 from ...attention.kv_window import WindowSpec
 
@@ -18,36 +23,7 @@ DEFAULT_OUTLIERS = 6
 DEFAULT_POW2 = True
 GROUP_TOKENS = 32
 OUTLIER_REPRS = ("relidx7", "combinadic", "bitmap")
-_OFF = {"", "0", "false", "off", "no"}
-
-
-def _env_present(name: str) -> bool:
-    return os.environ.get(name, "").strip() != ""
-
-
-def _env_str(name: str, default: str) -> str:
-    v = os.environ.get(name, "").strip()
-    return v.lower() if v else default
-
-
-def _env_int(name: str, default: int) -> int:
-    v = os.environ.get(name, "").strip()
-    return int(v) if v else int(default)
-
-
-def _env_float(name: str, default: float) -> float:
-    v = os.environ.get(name, "").strip()
-    return float(v) if v else float(default)
-
-
-def _env_bool(name: str, default: bool) -> bool:
-    if not _env_present(name):
-        return bool(default)
-    return os.environ[name].strip().lower() not in _OFF
-
-
-def _env_int_alias(canonical: str, alias: str, default: int) -> int:
-    return _env_int(canonical, _env_int(alias, default))
+K_FORMATS = ("i2f4", "itf4")
 
 
 @dataclass
@@ -96,68 +72,135 @@ class OMMXServingConfig:
                     window=self.window(), group_channels=self.group_channels)
 
 
+# ── the knob table ─────────────────────────────────────────────────────────────────────────
+
+def _word(text: str) -> str:
+    return text.lower()
+
+
+def _switch(text: str) -> bool:
+    """A knob that is set is on unless its text is one of the usual spellings of "off"."""
+    return text.lower() not in ("0", "false", "off", "no")
+
+
+class Knob(NamedTuple):
+    target: str                                  # field of OMMXServingConfig
+    names: Tuple[str, ...]                       # environment names, the first one that is set wins
+    parse: Callable[[str], Any]
+
+
+KNOBS: Tuple[Knob, ...] = (
+    Knob("k_format", ("OMMX_ATTN_K_FORMAT",), _word),
+    Knob("outliers_per_vector", ("OMMX_ATTN_OUTLIERS",), int),
+    Knob("outlier_select", ("OMMX_ATTN_OUTLIER_SELECT",), _word),
+    Knob("outlier_repr", ("OMMX_ATTN_OUTLIER_REPR",), _word),
+    Knob("use_pow2", ("OMMX_ATTN_POW2",), _switch),
+    Knob("combinadic_read", ("OMMX_ATTN_COMBINADIC_READ",), _switch),
+    Knob("bitmap_read", ("OMMX_ATTN_BITMAP_READ",), _switch),
+    Knob("sink_tokens", ("OMMX_KV_SINK", "OMMX_ATTN_SINK"), int),
+    Knob("recent_window", ("OMMX_KV_RECENT", "OMMX_ATTN_RECENT"), int),
+    Knob("group_tokens", ("OMMX_KV_GROUP_TOKENS", "OMMX_ATTN_GROUP_TOKENS"), int),
+    Knob("group_channels", ("OMMX_KV_GROUP_CHANNELS", "OMMX_ATTN_GROUP_CHANNELS"), int),
+    Knob("kv_outlier_map", ("OMMX_KV_OUTLIER_MAP",), _switch),
+    Knob("strict", ("OMMX_STRICT",), _switch),
+    Knob("max_context", ("OMMX_ATTN_MAXCTX",), int),
+)
+# Knobs that are not a field of their own: the outlier count as a share of the group, and the
+# reference's named presets (its recipe registry is not part of this package).
+SHARE_KNOB = "OMMX_OUTLIER_PERCENT"
+PRESET_KNOB = "OMMX_RECIPE"
+GEOMETRY = ("head_dim", "n_q_heads", "n_kv_heads", "page_size", "max_context")
+
+
+def _set_text(env: Mapping[str, str], name: str) -> Optional[str]:
+    """The knob's text, or None when it is unset or blank (a blank variable counts as unset)."""
+    text = env.get(name, "").strip()
+    return text or None
+
+
+def read_knobs(env: Optional[Mapping[str, str]] = None) -> Dict[str, Any]:
+    """Field values the environment asks for; fields nobody set are absent from the result."""
+    env = os.environ if env is None else env
+    found: Dict[str, Any] = {}
+    for knob in KNOBS:
+        for name in knob.names:
+            text = _set_text(env, name)
+            if text is None:
+                continue
+            try:
+                found[knob.target] = knob.parse(text)
+            except ValueError as exc:
+                raise ValueError(f"{name}={text!r} does not read as {knob.parse.__name__}") from exc
+            break
+    share = _set_text(env, SHARE_KNOB)
+    if share is not None:
+        # a share of the K vector, at least one outlier once the share is positive; it outranks the count
+        gt = found.get("group_tokens", GROUP_TOKENS)
+        frac = float(share)
+        found["outliers_per_vector"] = max(1, int(round(gt * frac))) if frac > 0 else 0
+    return found
+
+
+def explain_knobs() -> str:
+    """One line per knob: field, environment names in order of precedence, current text."""
+    rows = [f"{k.target:22s} {' > '.join(k.names):55s} {next((t for t in (_set_text(os.environ, n) for n in k.names) if t), '-')}"
+            for k in KNOBS]
+    rows.append(f"{'outliers_per_vector':22s} {SHARE_KNOB + ' (share of group_tokens, outranks the count)':55s} "
+                f"{_set_text(os.environ, SHARE_KNOB) or '-'}")
+    return "\n".join(rows)
+
+
+def _refuse(cfg: OMMXServingConfig) -> Optional[str]:
+    """Why this configuration cannot be served, or None.  Every rule is the reference's
+    (config.py:398-465) except the first, which belongs to the step seam of this package."""
+    bitmap, ranks = cfg.resolved_bitmap_read(), cfg.resolved_combinadic_read()
+    rules = (
+        (cfg.recent_window < 1 or cfg.sink_tokens < 0,
+         f"OMMX_KV_RECENT must be >= 1 and OMMX_KV_SINK >= 0 (got recent={cfg.recent_window}, "
+         f"sink={cfg.sink_tokens}): the seam packs a completed group before the forward writes the "
+         "step's own token, which is safe only while that token still sits among the bf16 recent rows"),
+        (cfg.k_format not in K_FORMATS,
+         f"OMMX_ATTN_K_FORMAT={cfg.k_format!r}: the K base format is one of {K_FORMATS}"),
+        (cfg.outlier_repr not in OUTLIER_REPRS,
+         f"OMMX_ATTN_OUTLIER_REPR={cfg.outlier_repr!r}: the index plane is one of {OUTLIER_REPRS}"),
+        (bitmap and ranks,
+         "OMMX_ATTN_BITMAP_READ and OMMX_ATTN_COMBINADIC_READ both on: a pack holds one index plane, "
+         "so the decode can read positions from one of them only"),
+        (bool(cfg.bitmap_read) and cfg.outlier_repr != "bitmap",
+         f"OMMX_ATTN_BITMAP_READ=1 with outlier_repr={cfg.outlier_repr!r}: that store writes no "
+         "k_obmp plane to read; set OMMX_ATTN_OUTLIER_REPR=bitmap"),
+        (bool(cfg.combinadic_read) and cfg.outlier_repr != "combinadic",
+         f"OMMX_ATTN_COMBINADIC_READ=1 with outlier_repr={cfg.outlier_repr!r}: that store writes no "
+         "k_crank plane to read; set OMMX_ATTN_OUTLIER_REPR=combinadic"),
+        (bitmap and cfg.outliers_per_vector > 8,
+         f"{cfg.outliers_per_vector} outliers per vector on the bitmask plane: the bitmask read stops "
+         "at 8; use OMMX_ATTN_OUTLIER_REPR=relidx7 or a lower OMMX_ATTN_OUTLIERS / OMMX_OUTLIER_PERCENT"),
+    )
+    return next((why for hit, why in rules if hit), None)
+
+
 def resolve_serving_config(*, head_dim: Optional[int] = None, n_q_heads: Optional[int] = None,
                            n_kv_heads: Optional[int] = None, page_size: Optional[int] = None,
                            max_context: Optional[int] = None) -> OMMXServingConfig:
-    """Environment knobs + model geometry -> config (config.py:342-440).  Named presets
-    (``OMMX_RECIPE``) belong to the reference's recipe registry, which this package does not
-    carry: a set variable raises instead of silently serving the default recipe."""
-    if _env_present("OMMX_RECIPE"):
-        raise NotImplementedError(
-            "OMMX_RECIPE presets are not available here; set the OMMX_ATTN_* / OMMX_KV_* knobs")
-    gt = _env_int_alias("OMMX_KV_GROUP_TOKENS", "OMMX_ATTN_GROUP_TOKENS", GROUP_TOKENS)
-    gc = _env_int_alias("OMMX_KV_GROUP_CHANNELS", "OMMX_ATTN_GROUP_CHANNELS", GROUP_TOKENS)
-    if _env_present("OMMX_OUTLIER_PERCENT"):
-        pct = _env_float("OMMX_OUTLIER_PERCENT", 0.0)
-        npv = max(1, int(round(gt * pct))) if pct > 0 else 0
-    else:
-        npv = _env_int("OMMX_ATTN_OUTLIERS", DEFAULT_OUTLIERS)
-    cfg = OMMXServingConfig(
-        k_format=_env_str("OMMX_ATTN_K_FORMAT", "i2f4"),
-        outliers_per_vector=npv,
-        outlier_select=_env_str("OMMX_ATTN_OUTLIER_SELECT", "signed"),
-        outlier_repr=_env_str("OMMX_ATTN_OUTLIER_REPR", DEFAULT_OUTLIER_REPR),
-        use_pow2=_env_bool("OMMX_ATTN_POW2", DEFAULT_POW2),
-        combinadic_read=(_env_bool("OMMX_ATTN_COMBINADIC_READ", False)
-                         if _env_present("OMMX_ATTN_COMBINADIC_READ") else None),
-        bitmap_read=(_env_bool("OMMX_ATTN_BITMAP_READ", False)
-                     if _env_present("OMMX_ATTN_BITMAP_READ") else None),
-        sink_tokens=_env_int_alias("OMMX_KV_SINK", "OMMX_ATTN_SINK", 8),
-        recent_window=_env_int_alias("OMMX_KV_RECENT", "OMMX_ATTN_RECENT", 32),
-        group_tokens=gt, group_channels=gc,
-        kv_outlier_map=_env_bool("OMMX_KV_OUTLIER_MAP", True),
-        strict=_env_bool("OMMX_STRICT", False),
-        max_context=_env_int("OMMX_ATTN_MAXCTX", 4096),
-    )
-    for name, val in (("head_dim", head_dim), ("n_q_heads", n_q_heads), ("n_kv_heads", n_kv_heads),
-                      ("page_size", page_size), ("max_context", max_context)):
-        if val is not None:
-            setattr(cfg, name, int(val))
-    if cfg.recent_window < 1 or cfg.sink_tokens < 0:
-        # the step seam packs completed groups before the forward writes token seq-1; that token
-        # stays outside the packed region only while at least one recent row is kept as bf16
-        raise ValueError(f"OMMX_KV_RECENT must be >= 1 and OMMX_KV_SINK >= 0; got recent="
-                         f"{cfg.recent_window}, sink={cfg.sink_tokens}: with no recent row the "
-                         "seam would pack a group whose last token is not written yet")
-    if cfg.k_format not in ("i2f4", "itf4"):
-        raise ValueError(f"OMMX_ATTN_K_FORMAT must be i2f4|itf4; got {cfg.k_format!r}")
-    if cfg.outlier_repr not in OUTLIER_REPRS:
-        raise ValueError(f"OMMX_ATTN_OUTLIER_REPR must be one of {OUTLIER_REPRS}; got {cfg.outlier_repr!r}")
-    if cfg.resolved_bitmap_read() and cfg.resolved_combinadic_read():
-        raise ValueError("OMMX_ATTN_BITMAP_READ and OMMX_ATTN_COMBINADIC_READ are mutually exclusive "
-                         "outlier-index sources (a pack carries exactly one index plane)")
-    if cfg.bitmap_read and cfg.outlier_repr != "bitmap":
-        raise ValueError("OMMX_ATTN_BITMAP_READ=1 needs OMMX_ATTN_OUTLIER_REPR=bitmap: the store "
-                         f"allocates no k_obmp plane under outlier_repr={cfg.outlier_repr!r}")
-    if cfg.combinadic_read and cfg.outlier_repr != "combinadic":
-        raise ValueError("OMMX_ATTN_COMBINADIC_READ=1 needs OMMX_ATTN_OUTLIER_REPR=combinadic: the "
-                         f"store allocates no k_crank plane under outlier_repr={cfg.outlier_repr!r}")
-    if cfg.resolved_bitmap_read() and cfg.outliers_per_vector > 8:
-        raise ValueError(f"outlier_repr=bitmap cannot serve outliers_per_vector={cfg.outliers_per_vector}: "
-                         "the bitmask read is limited to k <= 8 (config.py:458-465).  Set "
-                         "OMMX_ATTN_OUTLIER_REPR=relidx7, or lower OMMX_ATTN_OUTLIERS / OMMX_OUTLIER_PERCENT.")
+    """Defaults, then environment knobs, then the model's geometry (reference config.py:342-440).
+    A named preset raises: serving the default recipe under a preset's name would be silent."""
+    if _set_text(os.environ, PRESET_KNOB) is not None:
+        raise NotImplementedError(f"{PRESET_KNOB} presets come from the reference's recipe registry, which "
+                                  "is not part of this package; spell the recipe with the OMMX_ATTN_* / "
+                                  "OMMX_KV_* knobs (explain_knobs() lists them)")
+    cfg = OMMXServingConfig(**read_knobs())
+    given = dict(head_dim=head_dim, n_q_heads=n_q_heads, n_kv_heads=n_kv_heads, page_size=page_size,
+                 max_context=max_context)
+    for name in GEOMETRY:
+        if given[name] is not None:
+            setattr(cfg, name, int(given[name]))
+    why = _refuse(cfg)
+    if why is not None:
+        raise ValueError(why)
     return cfg
 
 
-__all__ = ["OMMXServingConfig", "resolve_serving_config", "DEFAULT_OUTLIER_REPR",
-           "DEFAULT_OUTLIERS", "DEFAULT_POW2", "GROUP_TOKENS", "OUTLIER_REPRS"]
+assert {k.target for k in KNOBS} <= {f.name for f in fields(OMMXServingConfig)}
+
+__all__ = ["OMMXServingConfig", "resolve_serving_config", "read_knobs", "explain_knobs", "KNOBS",
+           "DEFAULT_OUTLIER_REPR", "DEFAULT_OUTLIERS", "DEFAULT_POW2", "GROUP_TOKENS", "OUTLIER_REPRS"]

@@ -28,7 +28,6 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from ..common.batched_seam import BatchedStepPlanner
 from .config import OMMXServingConfig
 
 _UNSAFE_ROW_INDEX_ENV = "OMMX_UNSAFE_ROW_INDEX_SLOTS"
@@ -388,7 +387,6 @@ class OMMXBatchedStepManager(_Stoppable):
         self.num_seqs = self.cap = max(int(num_seqs), 1)
         self._make_pool = pool_cls
         self._pool_kwargs = dict(pool_kwargs or {})
-        self.planner = BatchedStepPlanner(self.window, cfg.max_context)
         self.max_seq_len_fixed = max(int(cfg.max_context), 1)
         self.max_tail_cap = int(self.window.max_tail_len(cfg.max_context))
         self._ctl_host = torch.zeros(3, self.cap, dtype=torch.long)
@@ -402,7 +400,6 @@ class OMMXBatchedStepManager(_Stoppable):
 
     def reset(self) -> None:
         self.pools.clear()
-        self.planner.reset()
         self.dead, self.dead_reason = False, None
         self._ledger = SlotLedger(self.num_seqs)
         self._keys_are_row_index = False
@@ -566,7 +563,6 @@ class OMMXBatchedStepManager(_Stoppable):
             # moves forward: start the newcomer from zero in every layer
             for pool in self.pools.values():
                 pool.seq_len[slot] = pool.packed_groups[slot] = 0
-            self.planner.reset(slot)
         return placed
 
 

@@ -10,7 +10,6 @@ import pytest
 import torch
 
 from open_ommx_serve_amd.attention.kv_window import WindowSpec, packed_boundary
-from open_ommx_serve_amd.integration.common import BatchedStepPlanner
 from open_ommx_serve_amd.integration.vllm import backend as BK
 from open_ommx_serve_amd.integration.vllm.config import OMMXServingConfig, resolve_serving_config
 from open_ommx_serve_amd.integration.vllm.metadata import (
@@ -294,20 +293,6 @@ def test_identity_is_required_unless_the_unsafe_hatch_is_set(monkeypatch):
     assert not m2.dead and sorted(m2.slots) == [0, 1]   # row 0 is a real request, not a null block
     with pytest.raises(OMMXSlotAllocationError, match="duplicate"):
         _bmgr(graph=False, strict=True)[0].on_build(_md([5, 6], [4, 4]))
-
-
-def test_planner_matches_the_window_arithmetic():
-    win = WindowSpec()
-    p = BatchedStepPlanner(win, 2048)
-    plan = p.plan([40, 41, 700, 3], slots=[2, 0, 1, 3])
-    assert plan.b_seq_len.tolist() == [win.packed_len(n) for n in (40, 41, 700, 3)]
-    assert plan.b_tail_len.tolist() == [len(win.tail_indices(n)) for n in (40, 41, 700, 3)]
-    assert plan.tail_pos[2, :int(plan.b_tail_len[2])].tolist() == win.tail_indices(700)
-    assert plan.regroup == [(0, win.num_groups(n)) for n in (40, 41, 700, 3)]
-    plan = p.plan([72, 41, 732, 0], slots=[2, 0, 1, 3])
-    assert plan.regroup[0] == (win.num_groups(40), win.num_groups(72))
-    assert plan.regroup[2] == (win.num_groups(700), win.num_groups(732))
-    assert plan.max_tail_len == win.max_tail_len(2048) and plan.max_seq_len == win.packed_len(732)
 
 
 # ── config and route decisions ───────────────────────────────────────────────────────────
