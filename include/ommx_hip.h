@@ -54,11 +54,14 @@ extern "C" {
 #define OMMX_ERR_EXP_RANGE     8   /* scale exponent does not fit the int8 plane */
 /* error bit OR-ed into *err_flag by ommx_ring_write / ommx_tail_gather */
 #define OMMX_ERR_RING_RANGE   16   /* row outside the history (kv_store_ops.py:33-34,52-53) */
-/* error bit OR-ed into *err_flag by the decode entry points */
+/* error bits OR-ed into *err_flag by the decode entry points */
 #define OMMX_ERR_TABLE_RANGE  64   /* a page id or group slot outside the planes (kv_pool.py:526-550 guards these on the host) */
+#define OMMX_ERR_VALUE_RANGE 128   /* a K step above 2^15 (K values beyond some 1e5) does not fit the f16 operands of
+                                      the matrix-core kernels; it is held at 2^15 and the result is off */
+/* not an error: OR-ed into *err_flag by ommx_store_pack when it writes a K step above 2^15, so that the owner
+   of the cache can send its decodes to ommx_decode_splitkv_ref before OMMX_ERR_VALUE_RANGE ever happens */
+#define OMMX_NOTE_WIDE_STEP  256
 /* error bit OR-ed into *err_flag by ommx_index_convert */
-#define OMMX_ERR_VALUE_RANGE 128   /* decode: a K step above 2^15 (K values beyond some 1e5) does not fit the f16
-                                      operands of the matrix-core kernels; it is held at 2^15 and the result is off */
 #define OMMX_ERR_INDEX_PLANE  32   /* a vector that does not name exactly k positions below group_tokens
                                       (codec.py:173-178 raises ValueError there) */
 
@@ -236,8 +239,7 @@ int ommx_decode_combine(const float* attn_logits, int64_t al_stride_b, int64_t a
 /*
  * Whole decode step (split-KV stage, then the combine with the bf16 tail) for callers that
  * cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
- * that forbid hipMalloc.  It has no counterpart in the reference, whose launcher allocates the
- * workspace `attn_logits` with torch when none is passed (paged_decode.py:3220-3222).
+ * that forbid hipMalloc.  It has no counterpart in the reference.
  * Arguments are those of ommx_decode_splitkv and ommx_decode_combine without the workspace:
  * the partial states of the splits are kept in a device array built into the library
  * (2 Mi floats = 8 MiB, held by every GPU the library runs on until the process ends).

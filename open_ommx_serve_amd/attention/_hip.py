@@ -31,6 +31,7 @@ ERR_NONFINITE_K, ERR_NONFINITE_V, ERR_UNDERFILLED, ERR_EXP_RANGE, ERR_RING_RANGE
 ERR_INDEX_PLANE = 32
 ERR_TABLE_RANGE = 64
 ERR_VALUE_RANGE = 128
+NOTE_WIDE_STEP = 256        # not an error: the store wrote a K step above 2^15 (see kv_pool.check_errors)
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 

@@ -197,6 +197,7 @@ class MultiSeqKVPool:
         self.max_tail_len = int(self.window.max_tail_len(self.max_seq_len))
         # device error bits of the store / ring kernels; read by check_errors()
         self.err_flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.wide_steps = False      # a packed K step above 2^15 was seen: decode on the plain kernel
         self._dbuf: Optional[Dict[str, object]] = None
         self._planes_cache: Optional[dict] = None
 
@@ -216,6 +217,19 @@ class MultiSeqKVPool:
         bits = int(self.err_flag.item())
         if bits:
             self.err_flag.zero_()
+        if bits & _hip.NOTE_WIDE_STEP:
+            # not an error: some packed K step is above 2^15, beyond the f16 operands of the matrix-core
+            # decode kernels; from here on this cache is decoded by the plain fp32 kernel
+            self.wide_steps = True
+        if bits & _hip.ERR_VALUE_RANGE:
+            self.wide_steps = True
+            raise ValueError("OMMX decode: a K step above 2^15 (K values beyond some 1e5) met the matrix-core "
+                             "kernel, whose f16 operands held it at 2^15: outputs since the last check are off "
+                             "for the requests that hold such a group.  This cache is served by the plain "
+                             "kernel from now on (_force_reference_kernel=True)")
+        if bits & _hip.ERR_TABLE_RANGE:
+            raise IndexError("OMMX decode: a page id or group slot of the request tables lies outside the planes "
+                             "(it was clamped; the output of that request is not meaningful)")
         if bits & _hip.ERR_RING_RANGE:
             raise IndexError("OMMX KV write/gather outside residual capacity")  # kv_store_ops.py:34,53
         raise_for_store_errors(bits)
@@ -523,6 +537,8 @@ class MultiSeqKVPool:
         if tables is None:
             tables = (self._req_to_token.index_select(0, sel), self._req_to_group.index_select(0, sel))
         planes["req_to_token"], planes["req_to_group"] = tables
+        # beside the planes: where the decode kernels report, and whether this cache needs the plain kernel
+        planes["err_flag"], planes["force_reference_kernel"] = self.err_flag, self.wide_steps
         return {
             "planes": planes, "k_tail": kt, "v_tail": vt,
             "b_tail_len": b_tail, "b_seq_len": b_seq,

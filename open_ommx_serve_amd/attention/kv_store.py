@@ -145,6 +145,7 @@ class CanonicalKVStore:
         self.k_tail_buf = z(1, self.tail_cap, self.H, self.D, dtype=bf, device=dev)
         self.v_tail_buf = z(1, self.tail_cap, self.H, self.D, dtype=bf, device=dev)
         self.err_flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.wide_steps = False      # a packed K step above 2^15 was seen: decode on the plain kernel
 
     # ── ring address mapping (kv_store.py:301-327) ────────────────────────────────────
 
@@ -162,6 +163,19 @@ class CanonicalKVStore:
         bits = int(self.err_flag.item())
         if bits:
             self.err_flag.zero_()
+        if bits & _hip.NOTE_WIDE_STEP:
+            # not an error: some packed K step is above 2^15, beyond the f16 operands of the matrix-core
+            # decode kernels; from here on this cache is decoded by the plain fp32 kernel
+            self.wide_steps = True
+        if bits & _hip.ERR_VALUE_RANGE:
+            self.wide_steps = True
+            raise ValueError("OMMX decode: a K step above 2^15 (K values beyond some 1e5) met the matrix-core "
+                             "kernel, whose f16 operands held it at 2^15: outputs since the last check are off "
+                             "for the requests that hold such a group.  This cache is served by the plain "
+                             "kernel from now on (_force_reference_kernel=True)")
+        if bits & _hip.ERR_TABLE_RANGE:
+            raise IndexError("OMMX decode: a page id or group slot of the request tables lies outside the planes "
+                             "(it was clamped; the output of that request is not meaningful)")
         if bits & _hip.ERR_RING_RANGE:
             raise IndexError("OMMX KV write/gather outside residual capacity")
         raise_for_store_errors(bits)
@@ -325,6 +339,7 @@ class CanonicalKVStore:
                "req_to_group": self._req_to_group_full[:, :G],
                "num_tokens": G * self.gt, "n_groups": G}
         out.update(self._meta())
+        out["err_flag"], out["force_reference_kernel"] = self.err_flag, self.wide_steps
         return out
 
     def decode_planes_full(self) -> dict:
@@ -335,6 +350,7 @@ class CanonicalKVStore:
                "v_main": self.v_main, "v_scale": self.v_scale, "v_zp": self.v_zp,
                "req_to_token": self._req_to_token_full, "req_to_group": self._req_to_group_full}
         out.update(self._meta())
+        out["err_flag"], out["force_reference_kernel"] = self.err_flag, self.wide_steps
         return out
 
     def tail_bf16(self) -> Tuple[torch.Tensor, torch.Tensor, int]:

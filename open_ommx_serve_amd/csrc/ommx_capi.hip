@@ -223,6 +223,12 @@ extern "C" int ommx_tail_gather(
         set_error("ommx_tail_gather: the ring is too short for recent_rows + a group + packed_lag");
         return -1;
     }
+    if (seq && T < sink_rows + recent_rows + group_tokens - 1 + packed_lag) {
+        // the tail of a request can hold that many rows (sink, recent, a group short of one token, the lag);
+        // the kernel writes min(rows, T), sink rows first, so a shorter buffer would drop the newest tokens
+        set_error("ommx_tail_gather: T is below sink_rows + recent_rows + group_tokens - 1 + packed_lag");
+        return -1;
+    }
     launch_tail_gather(a, seq, tail_idx, k_tail, v_tail, B, T, recent_rows, group_tokens,
                        packed_lag, b_tail_len, b_seq_len, static_cast<hipStream_t>(stream));
     if (hipGetLastError() != hipSuccess) { set_error("ommx_tail_gather: launch failed"); return -2; }

@@ -94,7 +94,7 @@ constexpr float MAX_SLACK = 8.0f;
 // the step's two groups take the operand code*2^(2m-10+e) instead (one packed subtraction more per operand
 // register, exact: both terms share the exponent) and drops the 2^e bias column.
 constexpr int EXACT_STEP_EXP = 5;
-// f16 operands: steps above 2^15 do not fit (K values beyond some 1e5); such a step is held at 2^15
+// f16 operands: steps above 2^15 do not fit (K or V values beyond some 1e5); such a step is held at 2^15
 // and OMMX_ERR_VALUE_RANGE is reported
 constexpr int MAX_STEP_EXP = 15;
 
@@ -156,7 +156,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
     const int r_half = max(heads >> 1, 1);            // head_dim 64: q heads per kv head of the pair
     const int Dout = half ? 64 : D;                   // channels of an output state
     const int sp = blockIdx.x;
-    int b = blockIdx.z, L;
+    int b = ORDER == 0 ? 0 : static_cast<int>(blockIdx.z), L;      // ORDER 0 is launched for one request only
     if (ORDER >= 1 && a.B > 1 && a.B <= 64) {
         const int my_len = lane < a.B ? a.seq[lane] : 0;
         const uint32_t key = (static_cast<uint32_t>(my_len) << 6) | (63u - lane);
@@ -208,6 +208,33 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             qraw[r] = (!half || (lane >> 5) == sl / r_half) ? w : 0u;
         }
     }
+    // The A operands are q * 2^(10-2m) as f16, up to q * 2^8: a query element of 256 or more would not
+    // fit.  When the wave's largest |q| reaches 2^7 the whole query is taken divided by a power of two
+    // (exact) that brings it below, and the softmax scale carries the factor back; 0 for ordinary queries.
+    int q_down = 0;
+    {
+        float qa = 0.0f;
+#pragma unroll
+        for (int r = 0; r < NH; ++r)
+            qa = fmaxf(qa, fmaxf(fabsf(__uint_as_float(qraw[r] << 16)), fabsf(__uint_as_float(qraw[r] & 0xFFFF0000u))));
+        if (__builtin_expect(__any(qa >= 128.0f) != 0, 0)) {
+            float m4[4] = {qa, qa, qa, qa};
+            wave_max4(m4);
+            q_down = min(static_cast<int>((__float_as_uint(m4[0]) >> 23) & 0xFFu) - 127 - 6, 100);
+        }
+    }
+    const float q_mul = __uint_as_float(static_cast<uint32_t>(127 - q_down) << 23);      // 2^-q_down
+    // (uniform: kept in a scalar register, like the argument it stands for)
+    const float sm_scale = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(
+        a.sm_scale * __uint_as_float(static_cast<uint32_t>(127 + q_down) << 23))));
+    if (__builtin_expect(q_down != 0, 0)) {
+        // the per-channel copies too (thresholds and exact residuals below then need no factor of their own)
+#pragma unroll
+        for (int r = 0; r < NH; ++r) {
+            const float lo = __uint_as_float(qraw[r] << 16) * q_mul, hi = __uint_as_float(qraw[r] & 0xFFFF0000u) * q_mul;
+            qraw[r] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
+        }
+    }
     // The 32-token groups are dealt out evenly: every split takes G/S groups and the first G%S
     // splits one more, so no two splits differ by more than one group and none is empty while
     // G >= S.  (One 32-bit division; the combine weighs the states by their lse, -inf for an
@@ -255,7 +282,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
         }
     };
     bool bad_id = false;            // a table entry outside the planes was seen (and clamped)
-    bool over_step = false;         // a K step above 2^MAX_STEP_EXP was seen (and held there); wave-uniform
+    bool over_step = false;         // a K or V step above 2^MAX_STEP_EXP was seen (and held there); wave-uniform
     u32x4 kr[2], vr[2];
     u32x2 vzp;
     uint32_t vsc, vrow;
@@ -351,7 +378,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
-                const float qs = static_cast<float>(1 << (10 - 2 * k_pos(4 * (ks & 1) + rr)));
+                const float qs = static_cast<float>(1 << (10 - 2 * k_pos(4 * (ks & 1) + rr))) * q_mul;
                 aq[ks][rr] = pack_f16x2(qs * q_at(cl), qs * q_at(cl + 8));
             }
         }
@@ -375,13 +402,13 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
         for (int r = 0; r < NH; ++r)
             qm = fmaxf(qm, fabsf(__uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16))));
         big_thr[u] = ((GEN ? (kout < 6 ? 0.5f : 0.75f) : 1.0f) * BIG_DELTA * 16.0f * BIG_DELTA_SM_SCALE) * (u ? cs1 : cs0) *
-                     __builtin_amdgcn_rcpf(qm * a.sm_scale);
+                     __builtin_amdgcn_rcpf(qm * sm_scale);
     }
     const uint32_t kt_lane = OFF_KT + (c0 >> 2);                   // code byte of the channel pair (4 channels a byte), row 0
     const uint32_t code_sh = 2u * (c0 & 3u);                      // bit of channel c0's code in that byte; c0 + 1 sits two on
     const uint32_t kbytes = static_cast<uint32_t>(kout + 1) >> 1;            // nibble bytes per channel
     const uint32_t nib_sh = 8u * ((2u * kbytes * lane) & 3u);
-    const float c2 = a.sm_scale * 1.4426950408889634f;
+    const float c2 = sm_scale * 1.4426950408889634f;
 
     // in the order the first step needs them: K rows, the group parameters, then V
     fetch_k();
@@ -409,7 +436,8 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
                 __builtin_bit_cast(s16x2e, __builtin_amdgcn_perm(0u, g_sc[0], 0x010C000Cu)),
                 __builtin_bit_cast(s16x2e, __builtin_amdgcn_perm(0u, g_sc[1], 0x010C000Cu)));
             const short e_top = top2[0] > top2[1] ? top2[0] : top2[1];
-            exact_step = __any(e_top >= EXACT_STEP_EXP * 256) != 0;
+            // (a scaled-down query means operands near the top of f16: the same cancellation, the same remedy)
+            exact_step = __any(e_top >= EXACT_STEP_EXP * 256) != 0 || q_down != 0;
             if (__builtin_expect(exact_step, 0)) over_step |= __any(e_top > MAX_STEP_EXP * 256) != 0;
         }
         {
@@ -625,6 +653,8 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             for (int c = 0; c < 8; ++c) vt[c * VT_COL] = vr[c >> 2][c & 3];
             typedef short s16x2 __attribute__((ext_vector_type(2)));
             typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+            // a V step above 2^MAX_STEP_EXP (a signed exponent byte of 16 or more) is held there and reported
+            if (__builtin_expect(__any((((vsc & 0x7F7F7F7Fu) + 0x70707070u) & ~vsc & 0x80808080u) != 0u) != 0, 0)) over_step = true;
             uint16_t* vs16 = reinterpret_cast<uint16_t*>(sm + OFF_VS) + lane;
             uint16_t* vz16 = reinterpret_cast<uint16_t*>(sm + OFF_VZ) + lane;
 #pragma unroll
@@ -632,7 +662,9 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
                 // f16 2^e of two channel groups: (e + 15) << 10 per half; below 2^-15 the step is
                 // immaterial and is held there
                 const uint32_t e2 = __builtin_amdgcn_perm(0u, vsc, h2 ? 0x030C020Cu : 0x010C000Cu);   // (e << 8) pairs
-                const s16x2 ec = __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256});
+                const s16x2 ec = __builtin_elementwise_min(
+                    __builtin_elementwise_max(__builtin_bit_cast(s16x2, e2), s16x2{-15 * 256, -15 * 256}),
+                    s16x2{MAX_STEP_EXP * 256, MAX_STEP_EXP * 256});
                 const u16x2 st = __builtin_bit_cast(u16x2, ec) * u16x2{4, 4} + u16x2{0x3C00, 0x3C00};
                 const uint32_t s2 = __builtin_bit_cast(uint32_t, st);
                 vs16[(2 * h2) * PT_ROW] = static_cast<uint16_t>(s2);
@@ -666,7 +698,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
             if (a.cap > 0.0f) {
                 asm volatile("" ::: "memory");
 #pragma unroll
-                for (int r = 0; r < 4; ++r) x[r] = apply_cap(x[r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+                for (int r = 0; r < 4; ++r) x[r] = apply_cap(x[r] * sm_scale, a.cap) * 1.4426950408889634f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) pe[r] = x[r] - m_run[r];
             } else {
@@ -732,7 +764,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
 #pragma unroll
                 for (int g = 0; g < 2; ++g)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) x[g][r] = apply_cap(x[g][r] * a.sm_scale, a.cap) * 1.4426950408889634f;
+                    for (int r = 0; r < 4; ++r) x[g][r] = apply_cap(x[g][r] * sm_scale, a.cap) * 1.4426950408889634f;
             } else {
 #pragma unroll
                 for (int g = 0; g < 2; ++g)

@@ -216,6 +216,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
         const Step st = make_step(raw, scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        if (st.e > 15) err |= OMMX_NOTE_WIDE_STEP;      // beyond the f16 operands of the matrix-core decode
         const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
@@ -394,6 +395,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const float raw = __fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f);
         const Step st = make_step(raw, scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        if (st.e > 15) err |= OMMX_NOTE_WIDE_STEP;
         const float scale = st.scale;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);

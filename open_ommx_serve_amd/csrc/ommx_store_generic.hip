@@ -107,6 +107,7 @@ __global__ void __launch_bounds__(256) store_generic_kernel(StoreArgs a) {
         if (omx < -1e8f) omx = 0.0f;
         const Step st = make_step(__fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f), a.scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        if (st.e > 15) err |= OMMX_NOTE_WIDE_STEP;      // beyond the f16 operands of the matrix-core decode
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
 
@@ -224,6 +225,7 @@ __global__ void __launch_bounds__(256) store_generic_kernel(StoreArgs a) {
         if (!fin) err |= OMMX_ERR_NONFINITE_V;
         const Step st = make_step(__fdiv_rn(fmaxf(mx - mn, 1e-8f), 3.0f), a.scale_mode, tab);
         if (!st.in_range) err |= OMMX_ERR_EXP_RANGE;
+        if (st.e > 15) err |= OMMX_NOTE_WIDE_STEP;
         const uint16_t zp_b = f32_to_bf16_rne(mn);
         const float zp = bf16_to_f32(zp_b);
         uint32_t* dst = reinterpret_cast<uint32_t*>(a.v_main + (prow * H + h) * (D / 4) + j * (GC / 4));

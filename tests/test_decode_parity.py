@@ -527,6 +527,47 @@ def test_a_step_beyond_the_f16_operands_is_reported():
     assert int(err.item()) == 0
 
 
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim", [(32, 8, 128), (16, 2, 128), (8, 4, 64)])
+def test_query_elements_of_several_hundred(q_heads, kv_heads, head_dim):
+    """The matrix-core kernel's QK operand is q * 2^(10-2m) as f16, up to q * 2^8: a query element of 256 or
+    more would saturate it.  The kernel divides such a query by a power of two first (exact) and lets the
+    softmax scale carry the factor; the result is held against the oracle like any other, with the lse bound
+    widened by 1e-5 of its value (logits now run into the thousands, where 2e-3 is eight fp32 ulps)."""
+    case = build_decode_case([900, 330], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, seed=31,
+                             permute_tables=True, sparse_frac=0.005)
+    g = torch.Generator().manual_seed(7)
+    q = case.q.float().cpu()
+    flat = q.view(-1)
+    where = torch.randperm(flat.numel(), generator=g)[:20]
+    flat[where] = torch.tensor([300.0, -512.0, 1000.0, -776.0, 256.0] * 4)
+    case.q.copy_(q.to(case.q.dtype))
+    err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+    wo, wl = _oracle(case)
+    for S in (1, 3):
+        o, lse = _run(case, num_kv_splits=S, err_flag=err)
+        assert torch.isfinite(o).all()
+        d = (o.double() - wo).abs()
+        assert d.max().item() <= MAX_ABS and d.mean().item() <= MEAN_ABS, f"S{S}: {d.max().item():.3e}"
+        assert ((lse.double() - wl).abs() <= 2e-3 + 1e-5 * wl.abs()).all(), f"S{S}: lse"
+    assert int(err.item()) == 0
+
+
+def test_a_v_step_beyond_the_f16_operands_is_reported():
+    """V values around 1e6 give V steps above 2^15: held at 2^15 and reported, like the K steps above."""
+    case = build_decode_case([300], q_heads=32, kv_heads=8, seed=18)
+    vs = case.planes["v_scale"]
+    vs.view(-1)[5::97] = 17                      # a handful of vectors with a step of 2^17
+    err = torch.zeros(1, dtype=torch.int32, device=case.q.device)
+    o, lse = _run(case, num_kv_splits=2, err_flag=err)
+    assert int(err.item()) & _hip.ERR_VALUE_RANGE
+    assert torch.isfinite(o).all()
+    err.zero_()
+    po, pl = _run(case, num_kv_splits=2, ref_kernel=True, err_flag=err)
+    wo, wl = _oracle(case)
+    assert ((po.double() - wo).abs() <= MAX_ABS + 1e-5 * wo.abs()).all()      # outputs in the thousands, fp32 sums
+    assert int(err.item()) == 0
+
+
 @pytest.mark.parametrize("B,hq", [(3, 32), (33, 32), (70, 32), (40, 64)])
 def test_long_tails_take_several_passes_in_every_combine_kernel(B, hq):
     """A recent window of 300 tokens gives tails of up to 339 bf16 rows: several chunks of 64 rows in the

@@ -290,6 +290,24 @@ def test_ring_ops_validate_before_touching_the_device():
         gather_tails(kh[0], kh[0], kh, kh, 0, 0, seq=torch.zeros(1, dtype=torch.int64))
 
 
+def test_tail_gather_refuses_a_buffer_shorter_than_the_longest_tail():
+    """In the length-driven form a request's tail can hold sink + recent + group - 1 + lag rows and the kernel
+    writes min(rows, T), sink rows first: a shorter buffer would drop the newest tokens, so the entry point
+    refuses it before any launch (the pointers below are never followed)."""
+    lib = _hip.load()
+    fake = 4096
+    args = dict(sink=8, recent=32, gt=32)
+    need = args["sink"] + args["recent"] + args["gt"] - 1
+
+    def call(T, lag):
+        return lib.ommx_tail_gather(fake, fake, 100 * 2 * 64, 100, None, fake, None, fake, fake, None, None,
+                                    1, T, 2, 64, args["sink"], args["recent"], args["gt"], 0, lag, None, None)
+
+    assert call(need - 1, 0) == -1 and b"T is below" in lib.ommx_last_error()
+    assert call(need, 1) == -1 and b"T is below" in lib.ommx_last_error()
+    assert call(need + 4, 5) == -1
+
+
 def test_table_id_clamp_arithmetic():
     """The clamp every decode kernel applies to the page ids and group slots it reads: ids inside
     the plane pass, anything else (negative ids included) lands on the nearest valid id and is

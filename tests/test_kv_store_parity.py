@@ -403,6 +403,68 @@ def test_pool_device_counter_path_equals_the_host_path():
     pools[0].check_errors()
 
 
+def test_pool_with_values_beyond_the_f16_operands_is_served_by_the_plain_kernel():
+    """K values in the millions give steps above 2^15, which the matrix-core decode cannot carry.  Nobody
+    passes a flag: the store kernel notes such a step in the pool's own error word, the pool's plane dicts
+    carry that word to the decode, and ``check_errors`` (a) raises if a decode already met such a step and
+    (b) sends every later decode of this pool to the plain kernel, whose output matches the oracle."""
+    from open_ommx_serve_amd.attention.reference_op import ommx_paged_decode
+    H, D, Hq = 8, 128, 32
+    win = WindowSpec()
+    n = 400
+    K, V = synth_kv(n, H, D, seed=77, sparse_frac=0.0)
+    K = (K.float() * 1.0e6).to(torch.bfloat16)
+    q = synth_q(1, Hq, D, seed=9).reshape(1, Hq, D).to(DEV)
+    q = (q.float() * 1.0e-6).to(torch.bfloat16)          # keeps the logits of order one
+    sm_scale = 1.0 / math.sqrt(D)
+    want = _oracle_decode(q, [K], [V], win, sm_scale)
+
+    def decode(pool):
+        b = pool.decode_inputs_batched([1])
+        o, lse = ommx_paged_decode(q, b["planes"], b["k_tail"], b["v_tail"], b["b_tail_len"], b["b_seq_len"],
+                                   sm_scale=sm_scale, max_seq_len=b["max_seq_len"], max_tail_len=b["max_tail_len"])
+        torch.cuda.synchronize()
+        return o.cpu(), lse.cpu()
+
+    # (a) decode before anybody looked at the error word: reported at the next check
+    pool = MultiSeqKVPool(D, H, num_seqs=2, max_seq_len=512, window=win, device=DEV, **RECIPE)
+    pool.append_block(1, K.to(DEV), V.to(DEV))
+    assert int(pool.k_scale.to(torch.int32).max()) > 15
+    decode(pool)
+    with pytest.raises(ValueError, match="2\\^15"):
+        pool.check_errors()
+    assert pool.wide_steps
+    got = decode(pool)                                     # now on the plain kernel
+    assert (got[0].double() - want[0]).abs().max().item() <= MAX_ABS
+    assert ((got[1].double() - want[1]).abs() <= 2e-3 + 2e-6 * want[1].abs()).all()
+    pool.check_errors()
+    # (b) checked after the pack, before the first decode: nothing is ever served wrong
+    pool = MultiSeqKVPool(D, H, num_seqs=2, max_seq_len=512, window=win, device=DEV, **RECIPE)
+    pool.append_block(1, K.to(DEV), V.to(DEV))
+    pool.check_errors()
+    assert pool.wide_steps
+    got = decode(pool)
+    assert (got[0].double() - want[0]).abs().max().item() <= MAX_ABS
+    pool.check_errors()
+
+
+def test_pool_raises_for_a_table_entry_outside_the_planes():
+    from open_ommx_serve_amd.attention.reference_op import ommx_paged_decode
+    H, D, Hq = 8, 128, 32
+    K, V = synth_kv(200, H, D, seed=78)
+    pool = MultiSeqKVPool(D, H, num_seqs=2, max_seq_len=256, window=WindowSpec(), device=DEV, **RECIPE)
+    pool.append_block(0, K.to(DEV), V.to(DEV))
+    b = pool.decode_inputs_batched([0])
+    b["planes"]["req_to_token"] = b["planes"]["req_to_token"].clone()
+    b["planes"]["req_to_token"][0, 2] = 1 << 20             # a page far outside the pool
+    q = synth_q(1, Hq, D, seed=3).reshape(1, Hq, D).to(DEV)
+    o, _ = ommx_paged_decode(q, b["planes"], b["k_tail"], b["v_tail"], b["b_tail_len"], b["b_seq_len"],
+                             sm_scale=0.1, max_seq_len=b["max_seq_len"], max_tail_len=b["max_tail_len"])
+    assert torch.isfinite(o).all()                           # the entry was held inside the planes
+    with pytest.raises(IndexError, match="outside the planes"):
+        pool.check_errors()
+
+
 def test_pool_reports_non_finite_rows_lazily():
     H, D = 2, 64
     pool = MultiSeqKVPool(D, H, num_seqs=1, max_seq_len=200, device=DEV, kv_ring=False, **RECIPE)

@@ -6,7 +6,8 @@ Checked through the C ABI against the existing pair of entry points
 to the decode tolerance (max-abs 2e-3 / mean-abs 2e-4 on ``o``, 2e-3 on ``lse``; the same
 kernels run, so the results normally agree to the last bits), and against the CPU oracle; two
 calls in a row, the second with a smaller input, so that stale contents of the shared array
-would show.  Also: sizes beyond the array are refused with a message."""
+would show.  Also: the driver's free device memory is the same before and after the second call
+(the call allocates nothing), and sizes beyond the array are refused with a message."""
 import pytest
 import torch
 
@@ -29,6 +30,8 @@ def _noalloc(case, S):
     p = case.planes
     lib = _hip.load()
     with torch.cuda.device(dev):
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]       # device memory the driver has left (hipMemGetInfo)
         rc = lib.ommx_decode_attention_noalloc(
             case.q.data_ptr(), case.q.stride(0), case.q.stride(1),
             p["k_base"].data_ptr(), p["k_scale"].data_ptr(), p["k_zp"].data_ptr(),
@@ -46,6 +49,8 @@ def _noalloc(case, S):
             B, Hq, case.kv_heads, D, case.page_size, case.outliers_per_vector, _hip.INDEX_BITMAP, 0,
             32, 32, 0, S, int(case.k_tail.shape[1]), float(case.sm_scale), 0.0, 0, int(p["k_base"].shape[0]), int(p["k_scale"].shape[0]), None,
             _hip.current_stream_ptr(dev))
+        torch.cuda.synchronize()
+        _noalloc.taken = free_before - torch.cuda.mem_get_info()[0]
     return rc, o, lse
 
 
@@ -87,6 +92,10 @@ def test_two_calls_in_a_row_second_smaller_match_the_workspace_entry_points():
         rc, o, lse = _noalloc(case, S)
         assert rc == 0, _hip.load().ommx_last_error()
         torch.cuda.synchronize()
+        if name == "small":
+            # the first call on a device may load the array's symbol; from the second call on the
+            # driver's free memory must read the same before and after the call
+            assert _noalloc.taken == 0, f"the call took {_noalloc.taken} bytes of device memory"
         wo, wl = _existing(case, S)
         torch.cuda.synchronize()
         _close(o, lse, wo, wl, f"{name} vs workspace entry points")
