@@ -258,7 +258,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
     }
 
     // ---- addressing ---------------------------------------------------------------------------
-    const uint32_t row_bytes = (uint32_t)Hkv * 32u;
+    const uint32_t row_bytes = (uint32_t)Hkv * 32u;          // of a code row (k_base, v_main): below 2^24
     const int last = n_end - 1;
     const int ps_sh = __ffs(a.ps) - 1, ps_mask = a.ps - 1;
     const int tsh = a.i64 ? 3 : 2;
@@ -283,29 +283,30 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
     };
     bool bad_id = false;            // a table entry outside the planes was seen (and clamped)
     bool over_step = false;         // a K or V step above 2^MAX_STEP_EXP was seen (and held there); wave-uniform
+    // Every plane this kernel is launched on is smaller than 4 GiB (the launcher sends larger ones to the
+    // kernel in ommx_decode.hip), so a row or a group is a scalar plane pointer plus a 32-bit byte offset:
+    // no 64-bit address arithmetic in the loop.
     u32x4 kr[2], vr[2];
     u32x2 vzp;
-    uint32_t vsc, vrow;
-    auto fetch_k = [&]() {          // K code row of this lane's token; remembers the row for fetch_v
+    uint32_t vsc, vro;
+    auto at = [](const void* base, uint32_t byte_off) { return static_cast<const char*>(base) + byte_off; };
+    auto fetch_k = [&]() {          // K code row of this lane's token; remembers the row offset for fetch_v
         pg1 = clamp_id(pg1, a.n_pages, bad_id);
-        vrow = (uint32_t)((pg1 << ps_sh) + ps1);
-        const uint64_t ro = (uint64_t)vrow * row_bytes;
-        kr[0] = *reinterpret_cast<const u32x4*>(kb_head + ro);
-        kr[1] = *reinterpret_cast<const u32x4*>(kb_head + ro + 16);
+        vro = __umul24(static_cast<uint32_t>((pg1 << ps_sh) + ps1), row_bytes);
+        kr[0] = *reinterpret_cast<const u32x4*>(at(kb_head, vro));
+        kr[1] = *reinterpret_cast<const u32x4*>(at(kb_head, vro + 16));
     };
-    auto fetch_v = [&]() {
-        const uint64_t ro = (uint64_t)vrow * row_bytes;
-        vr[0] = *reinterpret_cast<const u32x4*>(vb_head + ro);
-        vr[1] = *reinterpret_cast<const u32x4*>(vb_head + ro + 16);
-        vsc = *reinterpret_cast<const uint32_t*>(vs_head + (uint64_t)vrow * (uint32_t)(Hkv * 4));
-        vzp = *reinterpret_cast<const u32x2*>(vz_head + (uint64_t)vrow * (uint32_t)(Hkv * 4));
+    auto fetch_v = [&]() {          // a row of v_scale is an eighth, a row of v_zp a quarter of a code row
+        vr[0] = *reinterpret_cast<const u32x4*>(at(vb_head, vro));
+        vr[1] = *reinterpret_cast<const u32x4*>(at(vb_head, vro + 16));
+        vsc = *reinterpret_cast<const uint32_t*>(at(vs_head, vro >> 3));
+        vzp = *reinterpret_cast<const u32x2*>(at(vz_head, vro >> 2));
     };
     // channel pair (2*lane, 2*lane+1) parameters of both groups
     uint32_t g_sc[2], g_zp[2], g_ms[2] = {0, 0}, g_mc[2] = {0, 0};
     u32x2 g_bm[2], g_ov[2];
     uint32_t g_bx[2] = {0, 0};
     const uint32_t kvh_s = __builtin_amdgcn_readfirstlane(kvh);
-    auto at = [](const void* base, uint32_t byte_off) { return static_cast<const char*>(base) + byte_off; };
     auto fetch_params_g = [&](int g) {
         // (the lane number goes through an opaque copy: otherwise plane pointer + lane offset is kept
         // as a 64-bit register pair per plane across the loop, twelve registers the QK phase lacks;
@@ -313,35 +314,74 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
         uint32_t lane_b = lane;
         asm volatile("" : "+v"(lane_b));
         const uint32_t gs = __builtin_amdgcn_readfirstlane(clamp_id(gsl[g], a.n_gslots, bad_id));
-        const uint64_t gidx = ((uint64_t)gs * (uint32_t)Hkv + kvh_s) * D;
-        g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale + gidx, 2 * lane_b));
-        g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp + gidx, 4 * lane_b));
+        const uint32_t gidx = (gs * static_cast<uint32_t>(Hkv) + kvh_s) * D;      // first channel of the group, in elements
+        const uint32_t ch = gidx + 2 * lane_b;                                    // this lane's channel pair
+        g_sc[g] = *reinterpret_cast<const uint16_t*>(at(a.k_scale, ch));
+        g_zp[g] = *reinterpret_cast<const uint32_t*>(at(a.k_zp, 2 * ch));
         if (OWN_MAP) {
-            g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms + gidx, 4 * lane_b));
-            g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc + gidx, 4 * lane_b));
+            g_ms[g] = *reinterpret_cast<const uint32_t*>(at(a.k_ms, 2 * ch));
+            g_mc[g] = *reinterpret_cast<const uint32_t*>(at(a.k_mc, 2 * ch));
         }
         if constexpr (IDX == 0) {
-            g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp + gidx * 4, 8 * lane_b));
+            g_bm[g] = *reinterpret_cast<const u32x2*>(at(a.k_obmp, 4 * ch));
         } else {
-            const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp + gidx * 6, 12 * lane_b));
+            const uint32_t* ixp = reinterpret_cast<const uint32_t*>(at(a.k_obmp, 6 * ch));
             g_bm[g] = u32x2{ixp[0], ixp[1]};
             g_bx[g] = ixp[2];
         }
         if constexpr (!GEN) {
-            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * 3, 4 * ((3 * lane_b) / 2)));
+            // 3 nibble bytes per channel: the two dwords that hold the pair's six bytes
+            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval, 3 * gidx + 4 * ((3 * lane_b) / 2)));
             g_ov[g] = u32x2{ovp[0], ovp[1]};
         } else {
             // (kout + 1) / 2 bytes per channel, two channels per lane: the dword(s) that hold them
             const uint32_t kb = static_cast<uint32_t>(kout + 1) >> 1;
-            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval + gidx * kb, (2 * kb * lane_b) & ~3u));
+            const uint32_t* ovp = reinterpret_cast<const uint32_t*>(at(a.k_oval, gidx * kb + ((2 * kb * lane_b) & ~3u)));
             g_ov[g][0] = ovp[0];
             g_ov[g][1] = kb > 2 ? ovp[1] : 0u;       // 1 or 2 bytes per channel: one dword holds the pair
         }
     };
-    // The page and group ids of the first step are asked for here; what follows (clearing LDS, the
-    // A operands, the lane constants) needs none of it and runs while they are on their way.
+    // The page and group ids of the first step are asked for here; what follows (the A operands) needs
+    // none of it and runs while they are on their way.
     fetch_tables(n_begin);
     asm volatile("" ::: "memory");
+
+    // ---- A operand of QK: q * 2^(10-2m) of head j % 4 for this lane's 32-channel quarter, f16, in
+    // pair order: k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2).  The base codes,
+    // the outlier tile and the bias columns all use this one operand (the tile and the zero points
+    // are stored divided by the channel's 2^(10-2m)).
+    u32x4 aq[4];
+    {
+        auto q_at = [&](int c) {
+            return __uint_as_float((c & 1) ? (qw[c >> 1] & 0xFFFF0000u) : (qw[c >> 1] << 16));
+        };
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
+                const float qs = static_cast<float>(1 << (10 - 2 * k_pos(4 * (ks & 1) + rr))) * q_mul;
+                aq[ks][rr] = pack_f16x2(qs * q_at(cl), qs * q_at(cl + 8));
+            }
+        }
+    }
+    // The first step's data is asked for as soon as the page and group ids are here; clearing LDS, the
+    // accumulators and the lane constants need none of it and run while it is on its way (the A operands
+    // above ran while the ids were; with the clearing of LDS up there as well the request goes out late
+    // again: 31.0 against 29.8 us at batch 1, 64K).  The instantiation with the most registers in flight (position
+    // streams with their own outlier map, 4 heads) asks after the constants instead: with the loaded rows
+    // live across them it would spill.
+    constexpr bool FETCH_FIRST = !(IDX == 1 && OWN_MAP && NH == 4);
+    auto first_fetch = [&]() {
+        // in the order the first step needs them: K rows, the group parameters, then V
+        fetch_k();
+        fetch_params_g(0);
+        fetch_params_g(1);
+        fetch_v();
+        fetch_tables(n_begin + 64);
+        asm volatile("" ::: "memory");
+    };
+    if constexpr (FETCH_FIRST) first_fetch();
 
     // ---- LDS that starts out constant: zero tile, zero corrections, the zero and one rows ----
     {
@@ -364,25 +404,6 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
     for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
 
 
-    // ---- A operand of QK: q * 2^(10-2m) of head j % 4 for this lane's 32-channel quarter, f16, in
-    // pair order: k=(ks,kq,r) <-> channel 32kq + 16(ks/2) + 4(ks%2) + r/2 + 8(r%2).  The base codes,
-    // the outlier tile and the bias columns all use this one operand (the tile and the zero points
-    // are stored divided by the channel's 2^(10-2m)).
-    u32x4 aq[4];
-    {
-        auto q_at = [&](int c) {
-            return __uint_as_float((c & 1) ? (qw[c >> 1] & 0xFFFF0000u) : (qw[c >> 1] << 16));
-        };
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                const int cl = 16 * (ks >> 1) + 4 * (ks & 1) + rr;
-                const float qs = static_cast<float>(1 << (10 - 2 * k_pos(4 * (ks & 1) + rr))) * q_mul;
-                aq[ks][rr] = pack_f16x2(qs * q_at(cl), qs * q_at(cl + 8));
-            }
-        }
-    }
     auto q_of = [&](int u, int r) { return __uint_as_float(u ? (qraw[r] & 0xFFFF0000u) : (qraw[r] << 16)); };
     // ---- lane constants of the loop ------------------------------------------------------------
     // channel pass: lane = channels c0 = 2*lane, c0 + 1
@@ -409,13 +430,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
     const uint32_t kbytes = static_cast<uint32_t>(kout + 1) >> 1;            // nibble bytes per channel
     const uint32_t nib_sh = 8u * ((2u * kbytes * lane) & 3u);
     const float c2 = sm_scale * 1.4426950408889634f;
-
-    // in the order the first step needs them: K rows, the group parameters, then V
-    fetch_k();
-    fetch_params_g(0);
-    fetch_params_g(1);
-    fetch_v();
-    fetch_tables(n_begin + 64);
+    if constexpr (!FETCH_FIRST) first_fetch();
 
     for (int n0 = n_begin; n0 < n_end; n0 += 64) {
         const bool more = n0 + 64 < n_end;
@@ -950,6 +965,15 @@ int launch_decode_gqa4(const DecodeArgs& a_in, int Dh, int R, hipStream_t st) {
         nh = 2 * R;
     } else {
         return 1;
+    }
+    {
+        // the kernel addresses a plane by 32-bit byte offsets: it takes planes whose extents are given and
+        // below 4 GiB (code rows: pages * page size * kv heads * 32 B; the widest group plane has 6 B per channel)
+        const uint64_t lim = 0xFFFFFF00ull;
+        if (a.n_pages <= 0 || a.n_gslots <= 0) return 1;
+        if (static_cast<uint64_t>(a.n_pages) * static_cast<uint64_t>(a.ps) >= (1ull << 24)) return 1;
+        if (static_cast<uint64_t>(a.n_pages) * a.ps * a.Hkv * 32ull > lim) return 1;
+        if (static_cast<uint64_t>(a.n_gslots) * a.Hkv * D * 6ull > lim) return 1;
     }
     const bool general = a.half || a.kout != 6;
     if (general && a.idx_repr != 0) return 1;       // the general form reads bitmaps only
