@@ -504,6 +504,10 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": "decode_splitkv", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": TRAFFIC_BYTES_CTX64K if (args.ctx == 65536 and not args.splits and headline) else None,
+                     "traffic_source": ("profiles/decode_ctx64k_hbm_traffic.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE of "
+                                        "this kernel and workload, scaled by a copy kernel; a constant of the script, "
+                                        "not a counter read in this run)")
+                     if (args.ctx == 65536 and not args.splits and headline) else None,
                      "bytes_per_launch": packed_bytes,
                      "avg_kernel_us": round(k1, 3)},
         "cpu_baseline": cpu,

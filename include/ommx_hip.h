@@ -159,8 +159,15 @@ int ommx_store_pack(const void* K, const void* V, int in_dtype,
  *                 access leaves the planes, and OMMX_ERR_TABLE_RANGE is OR-ed into *err_flag
  *                 (NULL allowed; the caller zeroes it).  0 = extent not given, entries used as
  *                 they are.  A negative b_seq_len counts as 0 and is reported the same way.
- *                 OMMX_ERR_VALUE_RANGE: a K step above 2^15 met by the serving-recipe kernel, whose
- *                 f16 operands end there (the step is held at 2^15: finite output, but off).
+ *                 The serving-recipe kernel addresses its planes by 32-bit byte offsets: it runs when
+ *                 both extents are given and every plane is below 4 GiB (pages * page_size * Hkv * 32
+ *                 bytes of code rows, group slots * Hkv * D * 6 bytes of index plane); other calls run
+ *                 on the matrix-core kernel with 64-bit addressing (same results, more time).
+ *                 OMMX_ERR_VALUE_RANGE: a K or V step above 2^15 met by the serving-recipe kernel, whose
+ *                 f16 operands end there (the step is held at 2^15: finite output, but off); the store
+ *                 announces such a cache with OMMX_NOTE_WIDE_STEP, and ommx_decode_splitkv_ref serves it.
+ *                 Query elements of any size are served (a query with elements of 128 or more is taken
+ *                 divided by a power of two, exactly, and the softmax scale carries the factor).
  */
 int ommx_decode_splitkv(const uint16_t* q, int64_t q_stride_b, int64_t q_stride_h,
                         const uint8_t* k_base, const void* k_scale, const uint16_t* k_zp,
