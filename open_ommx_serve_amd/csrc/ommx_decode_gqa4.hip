@@ -496,8 +496,37 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             if (g == 1 && !g1_live) break;
-            float dl_max[2] = {0.0f, 0.0f};
-            auto walk = [&](auto RES, auto U) {
+            float* lc = reinterpret_cast<float*>(sm + OFF_LC);
+            // The channel pass of a group in two halves, so that the code bytes of both channels are on their
+            // way before either channel's entries need them: positions and code reads, then entries and scatter.
+            // The base MFMA takes every position of the K rows as it is stored; the tile entry of an
+            // outlier is what is missing on top of its stored 2-bit code, which the lane looks up
+            // in the staged K rows (a byte read per outlier; the packer's code of an outlier is the
+            // clamped 0 or 3 nearly always, so the entry is small).
+            auto walk_read = [&](auto U, int (&pos)[KMAX], uint32_t (&cb)[KMAX]) {
+                constexpr int u = decltype(U)::value;
+                uint32_t bm = 0, ix_lo = 0, ix_hi = 0;
+                if constexpr (IDX == 0) {
+                    bm = g_bm[g][u];
+                } else {
+                    ix_lo = u ? __builtin_amdgcn_alignbit(g_bx[g], g_bm[g][1], 16) : g_bm[g][0];
+                    ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
+                }
+                const uint8_t* kt = sm + kt_lane + g * 32 * KT_ROW;
+#pragma unroll
+                for (int sidx = 0; sidx < KMAX; ++sidx) {
+                    if constexpr (IDX == 0) {
+                        pos[sidx] = __builtin_ctz(bm) & 31;
+                        if (sidx < KMAX - 1) bm &= bm - 1;
+                    } else {
+                        pos[sidx] = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
+                                  : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
+                                              : ((ix_hi >> 3) & 31);
+                    }
+                    cb[sidx] = kt[pos[sidx] * KT_ROW];
+                }
+            };
+            auto walk_write = [&](auto U, const int (&pos)[KMAX], const uint32_t (&cb)[KMAX], float (&dls)[KMAX]) {
                 constexpr int u = decltype(U)::value;
                 const float zp = __uint_as_float(u ? (g_zp[g] & 0xFFFF0000u) : (g_zp[g] << 16));
                 const int e = static_cast<int8_t>((g_sc[g] >> (8 * u)) & 0xFFu);
@@ -516,13 +545,6 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
                     a1 = sc;
                     b1 = 0.0f;
                 }
-                uint32_t bm = 0, ix_lo = 0, ix_hi = 0;
-                if constexpr (IDX == 0) {
-                    bm = g_bm[g][u];
-                } else {
-                    ix_lo = u ? __builtin_amdgcn_alignbit(g_bx[g], g_bm[g][1], 16) : g_bm[g][0];
-                    ix_hi = u ? (g_bx[g] >> 16) : g_bm[g][1];
-                }
                 const uint64_t ov64 = (static_cast<uint64_t>(g_ov[g][1]) << 32) | g_ov[g][0];
                 const uint32_t nib = GEN ? static_cast<uint32_t>(ov64 >> (nib_sh + 8 * kbytes * u))
                                          : static_cast<uint32_t>(ov64 >> (nib_sh + 24 * u)) & 0xFFFFFFu;
@@ -531,53 +553,55 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
                 const f32x2 l45 = KMAX > 4 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 2) : f32x2{0.0f, 0.0f};
                 const f32x2 l67 = KMAX > 6 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 3) : f32x2{0.0f, 0.0f};
                 const float lv[8] = {l01[0], l01[1], l23[0], l23[1], l45[0], l45[1], l67[0], l67[1]};
-                // The base MFMA takes every position of the K rows as it is stored; the tile entry of an
-                // outlier is what is missing on top of its stored 2-bit code, which the lane looks up
-                // in the staged K rows (a byte read per outlier; the packer's code of an outlier is the
-                // clamped 0 or 3 nearly always, so the entry is small).
-                const uint8_t* kt = sm + kt_lane + g * 32 * KT_ROW;
-                float* lc = reinterpret_cast<float*>(sm + OFF_LC);
                 uint16_t* dt = reinterpret_cast<uint16_t*>(sm + OFF_TILE) + hw0 + 2 * u;      // pair order, like MAG
-                int pos[KMAX];
-                uint32_t cb[KMAX];
-#pragma unroll
-                for (int sidx = 0; sidx < KMAX; ++sidx) {
-                    if constexpr (IDX == 0) {
-                        pos[sidx] = __builtin_ctz(bm) & 31;
-                        if (sidx < KMAX - 1) bm &= bm - 1;
-                    } else {
-                        pos[sidx] = sidx < 4 ? ((ix_lo >> (7 * sidx)) & 31)
-                                  : sidx == 4 ? (__builtin_amdgcn_alignbit(ix_hi, ix_lo, 28) & 31)
-                                              : ((ix_hi >> 3) & 31);
-                    }
-                    cb[sidx] = kt[pos[sidx] * KT_ROW];
-                }
+                float dl_max = 0.0f;
 #pragma unroll
                 for (int sidx = 0; sidx < KMAX; ++sidx) {
                     const float dl0 = fmaf(lv[sidx], a1, b1);
                     const float code = static_cast<float>((cb[sidx] >> (code_sh + 2 * u)) & 3u);
-                    const float dl = fmaf(-code, sc, dl0);
-                    const _Float16 hi = static_cast<_Float16>(dl);
+                    float dl = fmaf(-code, sc, dl0);
+                    // (the entry as a value of its own: rounded to f16 here exactly as the residual pass rounds it)
+                    asm("" : "+v"(dl));
+                    dls[sidx] = dl;
                     if (GEN && sidx >= kout) continue;          // an unused slot (uniform): nothing to write
-                    if constexpr (!decltype(RES)::value) {
-                        dt[pos[sidx] * (TILE_ROW / 2)] = __builtin_bit_cast(uint16_t, hi);
-                        dl_max[u] = fmaxf(dl_max[u], fabsf(dl));
-                    } else {
-                        if (fabsf(dl) >= big_thr[u]) {
-                            const float lo = (dl - static_cast<float>(hi)) * __builtin_amdgcn_rcpf(cs);
+                    dt[pos[sidx] * (TILE_ROW / 2)] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(dl));
+                    dl_max = fmaxf(dl_max, fabsf(dl));
+                }
+                return dl_max;
+            };
+            // Entries whose f16 rounding matters add what the rounding dropped to the logits, exactly
+            // (rare, and kept out of the walks so that both channels' walks run as one stretch of code:
+            // their positions and entries are still at hand)
+            auto residuals = [&](auto U, const int (&pos)[KMAX], const float (&dls)[KMAX]) {
+                constexpr int u = decltype(U)::value;
+                const float un = __builtin_amdgcn_rcpf(u ? cs1 : cs0);
 #pragma unroll
-                            for (int r = 0; r < NH; ++r)
-                                __hip_atomic_fetch_add(lc + pos[sidx] * NH + r, lo * q_of(u, r), __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_WAVEFRONT);
-                        }
+                for (int sidx = 0; sidx < KMAX; ++sidx) {
+                    if (GEN && sidx >= kout) continue;
+                    const float dl = dls[sidx];
+                    if (fabsf(dl) >= big_thr[u]) {
+                        const float lo = (dl - static_cast<float>(static_cast<_Float16>(dl))) * un;
+#pragma unroll
+                        for (int r = 0; r < NH; ++r)
+                            __hip_atomic_fetch_add(lc + pos[sidx] * NH + r, lo * q_of(u, r), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_WAVEFRONT);
                     }
                 }
             };
-            walk(std::false_type{}, std::integral_constant<int, 0>{});
-            walk(std::false_type{}, std::integral_constant<int, 1>{});
-            const bool res0 = __any(dl_max[0] >= big_thr[0]), res1 = __any(dl_max[1] >= big_thr[1]);
-            if (res0) walk(std::true_type{}, std::integral_constant<int, 0>{});
-            if (res1) walk(std::true_type{}, std::integral_constant<int, 1>{});
+            int pos0[KMAX], pos1[KMAX];
+            uint32_t cb0[KMAX], cb1[KMAX];
+            float dls0[KMAX], dls1[KMAX];
+            // (the general form has fewer registers to spare: one channel after the other there)
+            walk_read(std::integral_constant<int, 0>{}, pos0, cb0);
+            if constexpr (!GEN) walk_read(std::integral_constant<int, 1>{}, pos1, cb1);
+            const float dlm0 = walk_write(std::integral_constant<int, 0>{}, pos0, cb0, dls0);
+            if constexpr (GEN) walk_read(std::integral_constant<int, 1>{}, pos1, cb1);
+            const float dlm1 = walk_write(std::integral_constant<int, 1>{}, pos1, cb1, dls1);
+            const bool res_any = __any(dlm0 >= big_thr[0] || dlm1 >= big_thr[1]) != 0;
+            if (__builtin_expect(res_any, 0)) {
+                residuals(std::integral_constant<int, 0>{}, pos0, dls0);
+                residuals(std::integral_constant<int, 1>{}, pos1, dls1);
+            }
             lds_fence();
             if (more) fetch_params_g(g);
             // both 16-token blocks of the group go through the eight k-steps together (two independent
@@ -633,7 +657,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2)
                     if (kq == 2 * g + t2) dsel[0] = d[t2];
-                if (res0 || res1) {       // exact residuals of this group's large deltas, then zero again
+                if (res_any) {       // exact residuals of this group's large deltas, then zero again
                     const f32x4 corr = *reinterpret_cast<const f32x4*>(sm + OFF_LC + 16 * (lane & 31));
                     if ((kq >> 1) == g) dsel[0] += corr;
                     lds_fence();
@@ -641,7 +665,7 @@ __global__ void __launch_bounds__(256, (NH == 8 || (GEN && KSLOTS == 8)) ? 2 : O
                 }
             } else {
                 dsel[g] = (kq >> 1) ? d[1] : d[0];
-                if (res0 || res1) {
+                if (res_any) {
                     // the lane's token of this group, its four heads
                     dsel[g] += *reinterpret_cast<const f32x4*>(sm + OFF_LC + 32 * (16 * (kq >> 1) + j) + 16 * (kq & 1));
                     lds_fence();
