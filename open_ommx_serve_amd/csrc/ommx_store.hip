@@ -69,10 +69,23 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                 const int64_t row = a.src_rows[g * 32 + i];
                 w[i] = load_elem<F32>(a.K, row * a.k_ts + (int64_t)h * a.k_hs + d);
             }
-        } else {            // consecutive rows: one base, 32 strides
-            const int64_t base = (int64_t)g * 32 * a.k_ts + (int64_t)h * a.k_hs + d;
+        } else {
+            // consecutive rows: the row address is the same for the whole workgroup (scalar registers,
+            // advanced by one stride per row); the thread adds its channel as one 32-bit offset shared by
+            // the 32 loads
+            typedef const __attribute__((address_space(1))) char* gptr;      // a global-memory address
+            uint64_t row = reinterpret_cast<uint64_t>(a.K) +
+                           static_cast<uint64_t>(((int64_t)g * 32 * a.k_ts + (int64_t)h * a.k_hs) * (F32 ? 4 : 2));
+            const uint64_t stride = static_cast<uint64_t>(a.k_ts * (F32 ? 4 : 2));
+            const uint32_t off = static_cast<uint32_t>(d) * (F32 ? 4u : 2u);
 #pragma unroll
-            for (int i = 0; i < 32; ++i) w[i] = load_elem<F32>(a.K, base + i * a.k_ts);
+            for (int i = 0; i < 32; ++i) {
+                if (F32) w[i] = *reinterpret_cast<const __attribute__((address_space(1))) float*>(reinterpret_cast<gptr>(row) + off);
+                else w[i] = bf16_to_f32(*reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>(reinterpret_cast<gptr>(row) + off));
+                row += stride;
+                asm volatile("" : "+s"(row));        // keeps the row address a scalar of its own: folded into one
+                                                     // vector expression it costs four vector instructions a load
+            }
         }
         if (!FAST6) {
 #pragma unroll
@@ -133,8 +146,8 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             int b1 = INT_MAX, b2 = INT_MAX, b3 = INT_MAX;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
-                const int kt_i = ordered_bits_bf16(w[i] + 0.0f) | (31 - i);      // FAST6 is a bf16-input instantiation
-                const int kb_i = kt_i ^ 31;
+                const int ob = ordered_bits_bf16(w[i] + 0.0f);                   // FAST6 is a bf16-input instantiation
+                const int kt_i = ob | (31 - i), kb_i = ob | i;
                 const int n4 = med3_i32(t3, t4, kt_i), n3 = med3_i32(t2, t3, kt_i), n2 = med3_i32(t1, t2, kt_i);
                 t1 = max(t1, kt_i); t2 = n2; t3 = n3; t4 = n4;
                 const int m4 = med3_i32(b3, b4, kb_i), m3 = med3_i32(b2, b3, kb_i), m2 = med3_i32(b1, b2, kb_i);
@@ -346,12 +359,8 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             const uint4 u = cr[q4];
             const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                uint32_t x = uw[k] & 0x03030303u;
-                x |= x >> 6;
-                x |= x >> 12;
-                kb8 |= static_cast<uint64_t>(x & 0xFFu) << (8 * (4 * q4 + k));
-            }
+            for (int k = 0; k < 4; ++k)      // bytes (c0, c1, c2, c3) . (1, 4, 16, 64): one dot product per byte of the row
+                kb8 |= static_cast<uint64_t>(__builtin_amdgcn_udot4(uw[k], 0x40100401u, 0u, false)) << (8 * (4 * q4 + k));
         }
         reinterpret_cast<uint64_t*>(a.k_base)[(prow * a.H + h) * NGV + j] = kb8;
 
@@ -405,8 +414,13 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
         const float zc = -zp * inv_scale;
         if (inv_ok && fabsf(zc) < INFINITY) {
 #pragma unroll
-            for (int c = 0; c < 32; ++c)
-                vb8 |= static_cast<uint64_t>(int2_code_fused(v[c], inv_scale, zc)) << (2 * c);
+            for (int c4 = 0; c4 < 8; ++c4) {
+                uint32_t four = 0u;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    four = __builtin_amdgcn_cvt_pk_u8_f32(fminf(__builtin_fmaf(v[4 * c4 + k], inv_scale, zc), 3.0f), k, four);
+                vb8 |= static_cast<uint64_t>(__builtin_amdgcn_udot4(four, 0x40100401u, 0u, false)) << (8 * c4);
+            }
         } else if (inv_ok) {
 #pragma unroll
             for (int c = 0; c < 32; ++c)
