@@ -75,6 +75,9 @@ def measure_store_table() -> torch.Tensor:
     up = idx >= torch.arange(1, 8).unsqueeze(-1)
     first = _first_true_monotone(up, "log")
     table[257:264] = win.gather(-1, first.unsqueeze(-1)).squeeze(-1)
+    # the kernels walk down the FP4 boundaries by halves, which takes them in ascending order
+    if not bool((table[257:264].diff() > 0).all()):
+        raise RuntimeError("measured FP4 level boundaries are not ascending")
     return table
 
 

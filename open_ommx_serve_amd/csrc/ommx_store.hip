@@ -28,8 +28,8 @@ __device__ __forceinline__ int ordered_bits_bf16(float x) {
 }
 __device__ __forceinline__ float from_ordered_bits(int k) {
     const int s = k & static_cast<int>(0xFFFF0000u);
-    // negative images had their low 16 bits set before the clearing; restore them
-    return __int_as_float(s < 0 ? ((s | 0xFFFF) ^ 0x7FFFFFFF) : s);
+    // the image is its own inverse: the sign bit stays, the others flip under a set sign
+    return __int_as_float(s ^ ((s >> 31) & 0x7FFF0000));
 }
 __device__ __forceinline__ int med3_i32(int a, int b, int c) {
     return max(min(a, b), min(max(a, b), c));          // v_med3_i32
@@ -37,7 +37,8 @@ __device__ __forceinline__ int med3_i32(int a, int b, int c) {
 
 // IDXT: index plane known at compile time (0 bitmap, 1 relidx7) or read from the arguments (2)
 template <bool F32, bool FAST6, int IDXT>
-__global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
+// (six waves per SIMD for the tuned bitmask instantiation, which fits their 80 registers without spilling)
+__global__ void __launch_bounds__(256, (FAST6 && IDXT == 0) ? 6 : 1) store_pack_kernel(StoreArgs a) {
     static_assert(!(F32 && FAST6), "the tuned path reads bf16 input");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // head_dim 128 is compiled in for the tuned instantiations (their launch checks it): row offsets
@@ -276,6 +277,11 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
             }
             // |(w - mc) * ms| is largest at the extreme lanes, which are outliers: they decide
             // whether every mapped value is finite (codec.py:55-57 checks all of them)
+            float thr[8];      // the FP4 boundaries, the same for every thread: scalar registers
+#pragma unroll
+            for (int j2 = 1; j2 < 8; ++j2)
+                thr[j2] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(tab[256 + j2])));
+            thr[0] = 0.0f;
 #pragma unroll
             for (int r = 0; r < 6; ++r) {
                 const int key = r < 3 ? key_hi[r] : key_lo[r - 3];
@@ -283,7 +289,7 @@ __global__ void __launch_bounds__(256) store_pack_kernel(StoreArgs a) {
                 const float mapped = fp4_input(from_ordered_bits(key));
                 mfin = mfin && is_finite_f32(mapped);
                 const int slot = __popc(om & ((1u << pos) - 1u));
-                nib |= fp4_encode(mapped, tab + 256) << (4 * slot);
+                nib |= fp4_encode_sorted(mapped, thr) << (4 * slot);
             }
         } else {
             int slot = 0;

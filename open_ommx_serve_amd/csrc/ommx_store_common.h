@@ -53,12 +53,24 @@ __device__ __forceinline__ float exp2_int(int e) {   // exact 2^e, e in [-126,12
     return __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
 }
 
+// FP4 code of m: sign bit and the number of magnitude thresholds fthr[1..7] (ascending) that |m| has
+// reached.
 __device__ __forceinline__ uint32_t fp4_encode(float m, const float* __restrict__ fthr) {
     const float a = fabsf(m);
     uint32_t idx = 0;
 #pragma unroll
     for (int j = 1; j <= 7; ++j) idx += (a >= fthr[j]) ? 1u : 0u;
     return ((m < 0.0f) ? 8u : 0u) | idx;
+}
+// The same with the seven thresholds in (scalar) registers t[1..7]: three compares down the sorted
+// thresholds instead of seven.
+__device__ __forceinline__ uint32_t fp4_encode_sorted(float m, const float (&t)[8]) {
+    const float a = fabsf(m);
+    const bool c4 = a >= t[4];
+    const bool c2 = a >= (c4 ? t[6] : t[2]);
+    const float lo = c4 ? t[5] : t[1], hi = c4 ? t[7] : t[3];
+    const bool c1 = a >= (c2 ? hi : lo);
+    return ((m < 0.0f) ? 8u : 0u) | (c4 ? 4u : 0u) | (c2 ? 2u : 0u) | (c1 ? 1u : 0u);
 }
 
 // x / 2^e is computed as x * 2^-e: 2^-e is exact for e in [-126,126], the product and the
